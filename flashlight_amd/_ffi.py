@@ -1,0 +1,252 @@
+"""ctypes binding of libflashlight_amd.so (declared in include/flashlight_amd.h).
+
+PyTorch is used only for device memory and the current HIP stream; every compute call goes through the C ABI.
+There is no fallback: a missing library or a non-GPU tensor raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+import os
+from pathlib import Path
+from typing import Optional, Sequence
+
+import torch
+
+LIB_NAME = "libflashlight_amd.so"
+LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
+
+MASK_NONE, MASK_CAUSAL, MASK_SLIDING, MASK_PREFIX_LM, MASK_DOCUMENT, MASK_DOCUMENT_CAUSAL = range(6)
+FL_BF16 = 0
+ABI_VERSION = 1
+
+
+class FlAttnParams(C.Structure):
+    """Mirror of `fl_attn_params` (include/flashlight_amd.h); field order and types must match."""
+
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+        ("q_strides", C.c_int64 * 4), ("k_strides", C.c_int64 * 4),
+        ("v_strides", C.c_int64 * 4), ("o_strides", C.c_int64 * 4),
+        ("B", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32), ("Lq", C.c_int32), ("Lk", C.c_int32),
+        ("Dqk", C.c_int32), ("Dv", C.c_int32),
+        ("scale", C.c_float),
+        ("mask_kind", C.c_int32), ("window", C.c_int32), ("prefix", C.c_int32),
+        ("doc_ids", C.c_void_p), ("doc_stride", C.c_int64),
+        ("alibi_heads", C.c_int32), ("softcap", C.c_float),
+        ("bias", C.c_void_p * 2), ("bias_strides", (C.c_int64 * 4) * 2), ("bias_batch_div", C.c_int32 * 2),
+        ("gate", C.c_void_p), ("gate_strides", C.c_int64 * 4),
+        ("diff", C.c_int32), ("lambda_", C.c_float),
+        ("dtype", C.c_int32),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
+        ("attended_dump", C.c_void_p),
+        ("reserved", C.c_int32 * 8),
+    ]
+
+
+class FlashlightError(RuntimeError):
+    """fl_attn_fwd / fl_attn_validate returned non-zero; `.code` holds the return value."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"flashlight_amd error {code}: {message}")
+        self.code = code
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
+    """Loads the in-tree shared library once.  Raises if it has not been built (no silent fallback)."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = Path(path) if path else LIB_PATH
+    if not p.exists():
+        raise FileNotFoundError(
+            f"{p} is missing: build it with `python -m flashlight_amd.build` (needs hipcc); "
+            "flashlight_amd has no non-HIP execution path")
+    lib = C.CDLL(str(p))
+    lib.fl_version.restype = C.c_int
+    lib.fl_last_error.restype = C.c_char_p
+    lib.fl_params_sizeof.restype = C.c_uint64
+    lib.fl_workspace_bytes.restype = C.c_uint64
+    lib.fl_workspace_bytes.argtypes = [C.POINTER(FlAttnParams)]
+    lib.fl_attn_validate.restype = C.c_int
+    lib.fl_attn_validate.argtypes = [C.POINTER(FlAttnParams)]
+    lib.fl_attn_plan.restype = C.c_int
+    lib.fl_attn_plan.argtypes = [C.POINTER(FlAttnParams), C.POINTER(C.c_int64)]
+    lib.fl_attn_fwd.restype = C.c_int
+    lib.fl_attn_fwd.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
+    if lib.fl_version() != ABI_VERSION:
+        raise RuntimeError(f"{p}: ABI version {lib.fl_version()} != expected {ABI_VERSION}")
+    if lib.fl_params_sizeof() != C.sizeof(FlAttnParams):
+        raise RuntimeError(f"{p}: fl_attn_params is {lib.fl_params_sizeof()} bytes, binding expects {C.sizeof(FlAttnParams)}")
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load_library().fl_last_error().decode()
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise FlashlightError(rc, last_error())
+
+
+def _strides4(t: torch.Tensor) -> Sequence[int]:
+    return tuple(int(s) for s in t.stride())
+
+
+def _require_gpu_bf16(name: str, t: torch.Tensor) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise NotImplementedError(
+            f"{name} is on {t.device}: flashlight_amd only runs its HIP kernels on a GPU tensor (no CPU path)")
+    if t.dtype != torch.bfloat16:
+        raise NotImplementedError(f"{name} has dtype {t.dtype}: the HIP kernels take bfloat16")
+
+
+def _dim_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """The kernels address [batch, head, seq, dim] through strides but need dim contiguous and 16-byte rows."""
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        return t.contiguous()
+    return t
+
+
+def attn_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    scale: Optional[float] = None,
+    mask_kind: int = MASK_NONE,
+    window: int = 0,
+    prefix: int = 0,
+    doc_ids: Optional[torch.Tensor] = None,
+    alibi_heads: int = 0,
+    softcap: float = 0.0,
+    biases: Sequence[tuple[torch.Tensor, int]] = (),
+    gate: Optional[torch.Tensor] = None,
+    diff: bool = False,
+    lambda_full: float = 0.0,
+    out: Optional[torch.Tensor] = None,
+    attended_dump: Optional[torch.Tensor] = None,
+    validate_only: bool = False,
+) -> torch.Tensor:
+    """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
+
+    `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, broadcastable to [B/batch_div, Hq, Lq, Lk]
+    (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
+    """
+    lib = load_library()
+    for name, t in (("query", q), ("key", k), ("value", v)):
+        _require_gpu_bf16(name, t)
+        if t.dim() != 4:
+            raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
+    q, k, v = _dim_contiguous(q), _dim_contiguous(k), _dim_contiguous(v)
+    B, Hq_all, Lq, Dqk = q.shape
+    Bk, Hk_all, Lk, Dk = k.shape
+    Bv, Hv, Lv, Dv = v.shape
+    if not (B == Bk == Bv) or Dqk != Dk or Lk != Lv:
+        raise ValueError(f"inconsistent shapes: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if diff:
+        if Hq_all % 2 or Hk_all % 2:
+            raise ValueError("differential attention needs an even number of query and key heads")
+        Hq, Hkv = Hq_all // 2, Hk_all // 2
+    else:
+        Hq, Hkv = Hq_all, Hk_all
+    if Hv != Hkv:
+        raise ValueError(f"value has {Hv} heads, expected {Hkv}")
+    if out is None:
+        out = torch.empty((B, Hq, Lq, Dv), dtype=torch.bfloat16, device=q.device)
+    elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != torch.bfloat16 or out.device != q.device:
+        raise ValueError("out has the wrong shape, dtype or device")
+
+    p = FlAttnParams()
+    p.q, p.k, p.v, p.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.q_strides[:] = _strides4(q)
+    p.k_strides[:] = _strides4(k)
+    p.v_strides[:] = _strides4(v)
+    p.o_strides[:] = _strides4(out)
+    p.B, p.Hq, p.Hkv, p.Lq, p.Lk, p.Dqk, p.Dv = B, Hq, Hkv, Lq, Lk, Dqk, Dv
+    p.scale = float(1.0 / math.sqrt(Dqk) if scale is None else scale)
+    p.mask_kind, p.window, p.prefix = int(mask_kind), int(window), int(prefix)
+    keep = [q, k, v, out]
+    if doc_ids is not None:
+        if doc_ids.dim() != 2 or doc_ids.shape[1] != Lk or doc_ids.shape[0] not in (1, B):
+            raise ValueError(f"document ids must be [B, L] = [{B}, {Lk}], got {tuple(doc_ids.shape)}")
+        d = doc_ids.to(device=q.device, dtype=torch.int64)
+        if d.stride(1) != 1:
+            d = d.contiguous()
+        p.doc_ids = d.data_ptr()
+        p.doc_stride = int(d.stride(0)) if d.shape[0] == B and B > 1 else 0
+        keep.append(d)
+    p.alibi_heads = int(alibi_heads)
+    p.softcap = float(softcap)
+    if len(biases) > 2:
+        raise ValueError("at most two additive biases are supported")
+    for i, (b, div) in enumerate(biases):
+        _require_gpu_bf16(f"bias[{i}]", b)
+        if b.dim() != 4:
+            raise ValueError(f"bias[{i}] must be 4-D, got {tuple(b.shape)}")
+        want = (B // div, Hq, Lq, Lk)
+        if B % div:
+            raise ValueError(f"bias[{i}]: batch divisor {div} does not divide {B}")
+        strides = []
+        for ax, (n, w) in enumerate(zip(b.shape, want)):
+            if n == w and n != 1:
+                strides.append(int(b.stride(ax)))
+            elif n == 1:
+                strides.append(0)
+            else:
+                raise ValueError(f"bias[{i}] shape {tuple(b.shape)} does not broadcast to {want}")
+        if strides[3] not in (0, 1):
+            b = b.contiguous()
+            strides = [int(s) if n != 1 else 0 for s, n in zip(b.stride(), b.shape)]
+        p.bias[i] = b.data_ptr()
+        p.bias_strides[i][:] = strides
+        p.bias_batch_div[i] = int(div)
+        keep.append(b)
+    if gate is not None:
+        _require_gpu_bf16("gate", gate)
+        if tuple(gate.shape) != (B, Hq, Lq, Dv):
+            raise ValueError(f"gate must have the output's shape {(B, Hq, Lq, Dv)}, got {tuple(gate.shape)}")
+        if gate.stride(-1) != 1 or any(s % 4 for s in gate.stride()[:-1]) or gate.data_ptr() % 8:
+            gate = gate.contiguous()
+        p.gate = gate.data_ptr()
+        p.gate_strides[:] = _strides4(gate)
+        keep.append(gate)
+    p.diff = 1 if diff else 0
+    p.lambda_ = float(lambda_full)
+    p.dtype = FL_BF16
+    if attended_dump is not None:
+        if attended_dump.dtype != torch.uint8 or tuple(attended_dump.shape) != (B, Hq, Lq, Lk) or \
+                not attended_dump.is_contiguous() or attended_dump.device != q.device:
+            raise ValueError("attended_dump must be a contiguous uint8 [B, Hq, Lq, Lk] tensor on the inputs' device")
+        p.attended_dump = attended_dump.data_ptr()
+    need = lib.fl_workspace_bytes(C.byref(p))
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), need
+        keep.append(ws)
+    if validate_only:
+        _check(lib.fl_attn_validate(C.byref(p)))
+        return out
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(lib.fl_attn_fwd(C.byref(p), C.c_void_p(stream)))
+    # tensors in `keep` were last used on the current stream; the caching allocator orders their reuse after it
+    del keep
+    return out
+
+
+def plan(p: FlAttnParams) -> dict:
+    """Tile shape / launch shape the library would use for `p` (host only)."""
+    lib = load_library()
+    out = (C.c_int64 * 8)()
+    _check(lib.fl_attn_plan(C.byref(p), out))
+    return {"rows_per_workgroup": out[0], "keys_per_tile": out[1], "threads": out[2], "workgroups": out[3],
+            "lds_bytes": out[4], "features": out[5]}

@@ -1,0 +1,110 @@
+"""Builds libflashlight_amd.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+One translation unit per kernel instance (rows of csrc/instance_list.inc) so the instances compile in parallel;
+objects are cached under csrc/build/ keyed by a hash of the sources and flags.
+"""
+from __future__ import annotations
+
+import concurrent.futures as cf
+import hashlib
+import os
+import re
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+INCLUDE = PKG_DIR.parent / "include"
+BUILD_DIR = CSRC / "build"
+LIB_PATH = PKG_DIR / "libflashlight_amd.so"
+
+ARCH = "gfx950"
+# -packed-fp32-ops: keep hipcc from forming v_pk_*_f32; the kernels are written for scalar fp32 VALU ops.
+HIPCC_FLAGS = [
+    "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-ignored-optimization-argument",
+    f"-I{INCLUDE}", f"-I{CSRC}",
+]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and Path(cand).exists():
+            return cand
+    raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
+
+
+def instance_rows() -> list[tuple[str, str]]:
+    rows = []
+    for line in (CSRC / "instance_list.inc").read_text().splitlines():
+        m = re.match(r"\s*X\(\s*(\w+)\s*,\s*(.*)\)\s*$", line)
+        if m:
+            rows.append((m.group(1), m.group(2).replace(" ", "")))
+    if not rows:
+        raise RuntimeError("instance_list.inc holds no instances")
+    return rows
+
+
+def _sources_digest() -> str:
+    h = hashlib.sha256()
+    for f in sorted(list(CSRC.glob("*.h")) + list(CSRC.glob("*.hip")) + list(CSRC.glob("*.inc")) + list(INCLUDE.glob("*.h"))):
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def _compile(args: tuple[list[str], Path]) -> str:
+    cmd, out = args
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {out.name}:\n{' '.join(cmd)}\n{log}")
+    return log
+
+
+def build(force: bool = True, jobs: int | None = None, verbose: bool = False) -> Path:
+    """Compiles every kernel instance and links the shared library.  force=False reuses cached objects."""
+    cc = hipcc()
+    digest = _sources_digest()
+    objdir = BUILD_DIR / digest
+    if force and BUILD_DIR.exists():
+        shutil.rmtree(BUILD_DIR)
+    objdir.mkdir(parents=True, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+
+    tasks: list[tuple[list[str], Path]] = []
+    objs: list[Path] = []
+    for name, args in instance_rows():
+        o = objdir / f"inst_{name}.o"
+        objs.append(o)
+        if not o.exists():
+            tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_NAME={name}", f"-DFL_INST_ARGS={args}", "-c",
+                           str(CSRC / "instance_unit.hip"), "-o", str(o)], o))
+    # the instance table is host data only: compiling it for the device would reference the host launchers
+    for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("api.hip", [])):
+        o = objdir / (Path(src).stem + ".o")
+        objs.append(o)
+        if not o.exists():
+            tasks.append(([cc, *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(o)], o))
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for log in ex.map(_compile, tasks):
+            if verbose and log.strip():
+                print(log, file=sys.stderr)
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    _compile(([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", *map(str, objs), "-o", str(tmp)], tmp))
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--incremental", action="store_true", help="reuse cached objects when sources are unchanged")
+    ap.add_argument("-j", "--jobs", type=int, default=None)
+    a = ap.parse_args()
+    print(build(force=not a.incremental, jobs=a.jobs, verbose=True))

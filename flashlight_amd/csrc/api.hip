@@ -1,0 +1,281 @@
+// C ABI of libflashlight_amd.so: argument validation (host only), instance selection, launch.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "flashlight_amd.h"
+#include "instances.h"
+
+namespace fl {
+// Builds (min, max) of the document ids of every block of kDocBlock positions.
+static __global__ void doc_table_kernel(const int64_t* ids, int64_t ids_stride, int L, int nblocks, int total, int64_t* table) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  int b = i / nblocks, blk = i % nblocks;
+  const int64_t* p = ids + (int64_t)b * ids_stride;
+  int p0 = blk * kDocBlock, p1 = min(L, p0 + kDocBlock);
+  int64_t mn = p[p0], mx = mn;
+  for (int j = p0 + 1; j < p1; ++j) {
+    int64_t x = p[j];
+    mn = x < mn ? x : mn;
+    mx = x > mx ? x : mx;
+  }
+  table[2 * (int64_t)i] = mn;
+  table[2 * (int64_t)i + 1] = mx;
+}
+
+}  // namespace fl
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool is_doc(int kind) { return kind == FL_MASK_DOCUMENT || kind == FL_MASK_DOCUMENT_CAUSAL; }
+
+uint32_t wanted_features(const fl_attn_params* p) {
+  uint32_t f = 0;
+  if (p->alibi_heads > 0) f |= fl::F_ALIBI;
+  if (p->softcap > 0.f) f |= fl::F_SOFTCAP;
+  if (p->bias[0] || p->bias[1]) f |= fl::F_BIAS;
+  if (is_doc(p->mask_kind)) f |= fl::F_DOC;
+  if (p->diff) f |= fl::F_DIFF;
+  if (p->gate) f |= fl::F_GATE;
+  if (p->attended_dump) f |= fl::F_DUMP;
+  return f;
+}
+
+// Features a kernel may be compiled with yet leave unused at run time (null pointer / zero slope).
+constexpr uint32_t kOptionalFeatures = fl::F_ALIBI | fl::F_BIAS | fl::F_GATE;
+
+const fl::Instance* select_instance(const fl_attn_params* p) {
+  const uint32_t want = wanted_features(p);
+  const fl::Instance* best = nullptr;
+  int best_extra = 1 << 30;
+  for (int i = 0; i < fl::kNumInstances; ++i) {
+    const fl::Instance& in = fl::kInstances[i];
+    if (in.dqk != p->Dqk || in.dv != p->Dv) continue;
+    if ((in.feat & want) != want) continue;
+    const uint32_t extra = in.feat & ~want;
+    if (extra & ~kOptionalFeatures) continue;
+    const int n = __builtin_popcount(extra);
+    if (n < best_extra) {
+      best = &in;
+      best_extra = n;
+    }
+  }
+  return best;
+}
+
+int check_strides(const char* what, const int64_t* s, int align) {
+  if (s[3] != 1) return fail(FL_ERR_STRIDE, "%s: the last (dim) stride must be 1, got %lld", what, (long long)s[3]);
+  for (int i = 0; i < 3; ++i) {
+    if (s[i] < 0) return fail(FL_ERR_STRIDE, "%s: negative stride %lld", what, (long long)s[i]);
+    if (s[i] % align != 0)
+      return fail(FL_ERR_ALIGN, "%s: stride[%d]=%lld must be a multiple of %d elements", what, i, (long long)s[i], align);
+  }
+  return 0;
+}
+
+int check_ptr(const char* what, const void* ptr, int align) {
+  if (!ptr) return fail(FL_ERR_NULL, "%s pointer is null", what);
+  if (reinterpret_cast<uintptr_t>(ptr) % align != 0)
+    return fail(FL_ERR_ALIGN, "%s pointer must be %d-byte aligned", what, align);
+  return 0;
+}
+
+int validate(const fl_attn_params* p, const fl::Instance** out) {
+  if (!p) return fail(FL_ERR_NULL, "params is null");
+  int rc;
+  if ((rc = check_ptr("q", p->q, 16)) || (rc = check_ptr("k", p->k, 16)) || (rc = check_ptr("v", p->v, 16)) ||
+      (rc = check_ptr("o", p->o, 8)))
+    return rc;
+  if (p->dtype != FL_BF16) return fail(FL_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lq <= 0 || p->Lk <= 0 || p->Dqk <= 0 || p->Dv <= 0)
+    return fail(FL_ERR_SHAPE, "sizes must be positive: B=%d Hq=%d Hkv=%d Lq=%d Lk=%d Dqk=%d Dv=%d", p->B, p->Hq, p->Hkv,
+                p->Lq, p->Lk, p->Dqk, p->Dv);
+  if (p->Hq % p->Hkv != 0)
+    return fail(FL_ERR_SHAPE, "query heads (%d) must be a multiple of key/value heads (%d)", p->Hq, p->Hkv);
+  if ((int64_t)p->B * p->Hq > (int64_t)1 << 30) return fail(FL_ERR_SHAPE, "B*Hq too large");
+  if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(FL_ERR_ARG, "scale must be finite and > 0, got %g", p->scale);
+  if ((rc = check_strides("q", p->q_strides, 8)) || (rc = check_strides("k", p->k_strides, 8)) ||
+      (rc = check_strides("v", p->v_strides, 8)) || (rc = check_strides("o", p->o_strides, 4)))
+    return rc;
+  for (int i = 0; i < 8; ++i)
+    if (p->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
+
+  switch (p->mask_kind) {
+    case FL_MASK_NONE:
+    case FL_MASK_CAUSAL: break;
+    case FL_MASK_SLIDING:
+      if (p->window < 0) return fail(FL_ERR_ARG, "window must be >= 0, got %d", p->window);
+      if (p->Lq != p->Lk) return fail(FL_ERR_SHAPE, "sliding window needs Lq == Lk (got %d, %d)", p->Lq, p->Lk);
+      break;
+    case FL_MASK_PREFIX_LM:
+      if (p->Lq != p->Lk) return fail(FL_ERR_SHAPE, "prefix-LM needs Lq == Lk (got %d, %d)", p->Lq, p->Lk);
+      break;
+    case FL_MASK_DOCUMENT:
+    case FL_MASK_DOCUMENT_CAUSAL:
+      if (!p->doc_ids) return fail(FL_ERR_NULL, "doc_ids pointer is null");
+      if (reinterpret_cast<uintptr_t>(p->doc_ids) % 8) return fail(FL_ERR_ALIGN, "doc_ids must be 8-byte aligned");
+      if (p->Lq != p->Lk) return fail(FL_ERR_SHAPE, "document mask needs Lq == Lk (got %d, %d)", p->Lq, p->Lk);
+      if (p->doc_stride < 0) return fail(FL_ERR_STRIDE, "doc_stride must be >= 0");
+      break;
+    default: return fail(FL_ERR_ARG, "unknown mask_kind %d", p->mask_kind);
+  }
+  if (p->alibi_heads < 0) return fail(FL_ERR_ARG, "alibi_heads must be >= 0");
+  if (!(p->softcap >= 0.f) || !std::isfinite(p->softcap)) return fail(FL_ERR_ARG, "softcap must be finite and >= 0");
+  for (int nb = 0; nb < 2; ++nb) {
+    if (!p->bias[nb]) continue;
+    if (reinterpret_cast<uintptr_t>(p->bias[nb]) % 2) return fail(FL_ERR_ALIGN, "bias[%d] must be 2-byte aligned", nb);
+    if (p->bias_batch_div[nb] <= 0) return fail(FL_ERR_ARG, "bias_batch_div[%d] must be >= 1", nb);
+    for (int i = 0; i < 4; ++i)
+      if (p->bias_strides[nb][i] < 0) return fail(FL_ERR_STRIDE, "bias[%d]: negative stride", nb);
+    if (p->bias_strides[nb][3] > 1) return fail(FL_ERR_STRIDE, "bias[%d]: the key stride must be 0 or 1", nb);
+  }
+  if (p->gate) {
+    if ((rc = check_ptr("gate", p->gate, 8)) || (rc = check_strides("gate", p->gate_strides, 4))) return rc;
+  }
+  if (p->diff) {
+    if (!std::isfinite(p->lambda)) return fail(FL_ERR_ARG, "lambda must be finite");
+  }
+  const fl::Instance* in = select_instance(p);
+  if (!in)
+    return fail(FL_ERR_UNSUPPORTED,
+                "no kernel instance for Dqk=%d Dv=%d features=0x%x (alibi=1 softcap=2 bias=4 doc=8 diff=16 gate=32 dump=64)",
+                p->Dqk, p->Dv, wanted_features(p));
+  const int64_t nkt = ((int64_t)p->Lk + in->bn - 1) / in->bn;
+  if (nkt > fl::kMaxKeyTiles)
+    return fail(FL_ERR_SHAPE, "Lk=%d exceeds the supported maximum of %d keys", p->Lk, fl::kMaxKeyTiles * in->bn);
+  const int64_t bm = (int64_t)in->rw * in->nw;
+  const int64_t grid = (int64_t)p->B * p->Hq * (((int64_t)p->Lq + bm - 1) / bm);
+  if (grid > 0x7fffffff) return fail(FL_ERR_SHAPE, "too many workgroups (%lld)", (long long)grid);
+  if (is_doc(p->mask_kind)) {
+    const uint64_t need = fl_workspace_bytes(p);
+    if (!p->workspace || p->workspace_bytes < need)
+      return fail(FL_ERR_WORKSPACE, "document mask needs a %llu-byte workspace (got %llu)", (unsigned long long)need,
+                  (unsigned long long)(p->workspace ? p->workspace_bytes : 0));
+    if (reinterpret_cast<uintptr_t>(p->workspace) % 8) return fail(FL_ERR_ALIGN, "workspace must be 8-byte aligned");
+  }
+  if (out) *out = in;
+  g_err[0] = 0;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fl_version(void) { return FL_ABI_VERSION; }
+
+const char* fl_last_error(void) { return g_err; }
+
+uint64_t fl_params_sizeof(void) { return sizeof(fl_attn_params); }
+
+uint64_t fl_workspace_bytes(const fl_attn_params* p) {
+  if (!p || !is_doc(p->mask_kind) || p->B <= 0 || p->Lk <= 0) return 0;
+  const uint64_t blocks = ((uint64_t)p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
+  return (uint64_t)p->B * blocks * 2 * sizeof(int64_t);
+}
+
+int fl_attn_validate(const fl_attn_params* p) { return validate(p, nullptr); }
+
+int fl_attn_plan(const fl_attn_params* p, int64_t out[8]) {
+  const fl::Instance* in = nullptr;
+  int rc = validate(p, &in);
+  if (rc) return rc;
+  if (!out) return fail(FL_ERR_NULL, "out is null");
+  const int64_t bm = (int64_t)in->rw * in->nw;
+  out[0] = bm;
+  out[1] = in->bn;
+  out[2] = in->nw * 64;
+  out[3] = (int64_t)p->B * p->Hq * ((p->Lq + bm - 1) / bm);
+  out[4] = in->lds_bytes;
+  out[5] = in->feat;
+  out[6] = 0;
+  out[7] = 0;
+  return 0;
+}
+
+int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
+  const fl::Instance* in = nullptr;
+  int rc = validate(p, &in);
+  if (rc) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+  fl::KParams kp;
+  std::memset(&kp, 0, sizeof(kp));
+  kp.q = static_cast<const fl::bf16_t*>(p->q);
+  kp.k = static_cast<const fl::bf16_t*>(p->k);
+  kp.v = static_cast<const fl::bf16_t*>(p->v);
+  kp.o = static_cast<fl::bf16_t*>(p->o);
+  for (int i = 0; i < 3; ++i) {
+    kp.qs[i] = p->q_strides[i];
+    kp.ks[i] = p->k_strides[i];
+    kp.vs[i] = p->v_strides[i];
+    kp.os[i] = p->o_strides[i];
+    kp.gs[i] = p->gate_strides[i];
+  }
+  kp.B = p->B;
+  kp.Hq = p->Hq;
+  kp.Hkv = p->Hkv;
+  kp.Lq = p->Lq;
+  kp.Lk = p->Lk;
+  kp.group = p->Hq / p->Hkv;
+  kp.scale = p->scale;
+  kp.scale_log2 = p->scale * 1.4426950408889634f;
+  kp.mask_kind = p->mask_kind;
+  kp.window = p->window;
+  kp.prefix = p->prefix;
+  kp.doc_ids = p->doc_ids;
+  kp.doc_stride = p->doc_stride;
+  kp.alibi_heads = p->alibi_heads;
+  kp.softcap = p->softcap;
+  for (int nb = 0; nb < 2; ++nb) {
+    kp.bias[nb] = static_cast<const fl::bf16_t*>(p->bias[nb]);
+    kp.bdiv[nb] = p->bias[nb] ? p->bias_batch_div[nb] : 1;
+    bool vec = p->bias[nb] && p->bias_strides[nb][3] == 1 && reinterpret_cast<uintptr_t>(p->bias[nb]) % 8 == 0;
+    for (int i = 0; i < 4; ++i) {
+      kp.bs[nb][i] = p->bias_strides[nb][i];
+      if (i < 3 && p->bias_strides[nb][i] % 4 != 0) vec = false;
+    }
+    kp.bias_vec[nb] = vec ? 1 : 0;
+  }
+  kp.gate = static_cast<const fl::bf16_t*>(p->gate);
+  kp.lambda = p->lambda;
+  if (p->diff) {
+    // heads [0, H) are branch 0, heads [H, 2H) branch 1 (query: H = Hq, key: H = Hkv)
+    kp.q_branch_stride = (int64_t)p->Hq * p->q_strides[1];
+    kp.k_branch_stride = (int64_t)p->Hkv * p->k_strides[1];
+  }
+  kp.dump = p->attended_dump;
+  const int bm = in->rw * in->nw;
+  kp.n_qtiles = (p->Lq + bm - 1) / bm;
+  kp.n_ktiles = (p->Lk + in->bn - 1) / in->bn;
+  const int grid = p->B * p->Hq * kp.n_qtiles;
+
+  if (is_doc(p->mask_kind)) {
+    const int blocks = (p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
+    const int total = p->B * blocks;
+    int64_t* table = static_cast<int64_t*>(p->workspace);
+    hipLaunchKernelGGL(fl::doc_table_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, p->doc_ids, p->doc_stride,
+                       p->Lk, blocks, total, table);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "doc_table_kernel launch failed: %s", hipGetErrorString(e));
+    kp.doc_table = table;
+    kp.doc_blocks = blocks;
+  }
+  hipError_t e = in->launch(kp, grid, stream);
+  if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+// Kernel instance registry: one launcher per compiled (head dims, tile shape, feature set).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "fwd_kernel.h"
+
+namespace fl {
+
+struct Instance {
+  const char* name;
+  int dqk, dv;
+  int rw, bn, nw;  // rows per wave, keys per tile, waves per workgroup
+  uint32_t feat;
+  int lds_bytes;
+  hipError_t (*launch)(const KParams&, int grid, hipStream_t);
+};
+
+// Defined by instances_table.cpp from the per-file launchers.
+extern const Instance kInstances[];
+extern const int kNumInstances;
+
+template <class T>
+hipError_t launch_fwd(const KParams& kp, int grid, hipStream_t stream) {
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<T>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+  if (attr != hipSuccess) return attr;
+  hipLaunchKernelGGL(fwd_kernel<T>, dim3(grid), dim3(T::NT), T::LDS_BYTES, stream, kp);
+  return hipGetLastError();
+}
+
+}  // namespace fl
+
+// Declares (FL_INSTANCE_DECL) or defines (FL_INSTANCE_DEF) the launcher of one instance.
+#define FL_INSTANCE_DECL(NAME, DQK, DV, RW, BN, NW, FEAT) \
+  namespace fl { hipError_t launch_##NAME(const KParams&, int, hipStream_t); }
+#define FL_INSTANCE_DEF(NAME, DQK, DV, RW, BN, NW, FEAT)                                   \
+  namespace fl {                                                                           \
+  hipError_t launch_##NAME(const KParams& kp, int grid, hipStream_t s) {                   \
+    return launch_fwd<FwdTraits<DQK, DV, RW, BN, NW, (FEAT)>>(kp, grid, s);                \
+  }                                                                                        \
+  }
+#define FL_INSTANCE_ROW(NAME, DQK, DV, RW, BN, NW, FEAT) \
+  {#NAME, DQK, DV, RW, BN, NW, (FEAT), fl::FwdTraits<DQK, DV, RW, BN, NW, (FEAT)>::LDS_BYTES, &fl::launch_##NAME},

@@ -1,0 +1,138 @@
+/*
+ * flashlight_amd.h -- C ABI of libflashlight_amd.so
+ *
+ * Fused FlashAttention-style forward kernels for gfx950 (MI355X), one launch per call:
+ * QK^T on bf16 MFMA -> score modification / masking in registers -> online softmax ->
+ * P.V on MFMA -> normalise -> bf16 store.  Tiles whose mask is empty are never visited.
+ *
+ * The reference (bozhiyou/flashlight) has no FFI: its boundary for this path is the set
+ * of eager PyTorch functions under attention_variants/ that callers wrap in
+ * torch.compile (tests/test_causal.py:14-17,33; benchmarks/run_flex_variants.py:118-147).
+ * What torch.compile + monkeypatch/fusion generate for those functions (one fused Triton
+ * kernel, monkeypatch/fusion/block_reduction.py:1302-1522) is what fl_attn_fwd replaces.
+ * Each field below cites the reference argument it carries.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; the library never allocates,
+ *     frees or retains device memory and never synchronises: work is queued on `stream`.
+ *   - strides are in ELEMENTS, order [batch, head, seq, dim]; the dim stride must be 1.
+ *   - return value: 0 ok; <0 invalid argument (nothing was launched, see fl_last_error());
+ *     >0 a hipError_t from the launch.
+ *   - re-entrant; the only mutable state is the thread-local error string.
+ */
+#ifndef FLASHLIGHT_AMD_H
+#define FLASHLIGHT_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FL_ABI_VERSION 1
+
+/* Which (q, k) pairs are attended.  q, k are 0-based positions, top-left aligned. */
+enum fl_mask_kind {
+  FL_MASK_NONE = 0,       /* vanilla.py:20-35, alibi.py:13-33, softcap.py:4-53, diff_attn.py:6-30, evoformer.py:8-36 */
+  FL_MASK_CAUSAL = 1,     /* k <= q                      causal.py:32-33 */
+  FL_MASK_SLIDING = 2,    /* 0 <= q - k <= window        sliding_window.py:4-12 (window+1 keys) */
+  FL_MASK_PREFIX_LM = 3,  /* k < prefix || k <= q        prefix_lm.py:33-42 */
+  FL_MASK_DOCUMENT = 4,   /* doc[q] == doc[k]            document_mask.py:25-27 */
+  FL_MASK_DOCUMENT_CAUSAL = 5 /* doc[q] == doc[k] && k <= q  (what the reference's Flex baseline computes,
+                                 benchmarks/run_flex_variants.py:86) */
+};
+
+enum fl_dtype { FL_BF16 = 0 };
+
+/* error codes (negative) */
+#define FL_ERR_NULL (-1)
+#define FL_ERR_SHAPE (-2)
+#define FL_ERR_STRIDE (-3)
+#define FL_ERR_UNSUPPORTED (-4)
+#define FL_ERR_ARG (-5)
+#define FL_ERR_WORKSPACE (-6)
+#define FL_ERR_ALIGN (-7)
+
+typedef struct fl_attn_params {
+  /* query [B, Hq, Lq, Dqk], key [B, Hkv, Lk, Dqk], value [B, Hkv, Lk, Dv], out [B, Hq, Lq, Dv]
+   * (causal.py:8-10).  With diff != 0, query/key hold 2*Hq / 2*Hkv heads: heads [0, H) feed softmax 0
+   * and heads [H, 2H) feed softmax 1 (diff_attn.py:14-17). */
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  int64_t q_strides[4], k_strides[4], v_strides[4], o_strides[4];
+  int32_t B, Hq, Hkv, Lq, Lk, Dqk, Dv;
+  /* multiplies QK^T before anything else (`scale` / `sm_scale` of every reference function); must be > 0 */
+  float scale;
+
+  int32_t mask_kind; /* enum fl_mask_kind */
+  int32_t window;    /* FL_MASK_SLIDING: `window_size` of sliding_window.py:14 */
+  int32_t prefix;    /* FL_MASK_PREFIX_LM: `prefix_lengths` of prefix_lm.py:5 */
+  /* FL_MASK_DOCUMENT*: `document_id`, int64 [B, L] with Lq == Lk (document_mask.py:10,25-27); any integers */
+  const int64_t* doc_ids;
+  int64_t doc_stride; /* elements between batches */
+
+  /* score = softcap_or_identity(qk * scale) + alibi + bias[0] + bias[1], then the mask.
+   * alibi_heads > 0 adds 2^(-8 (h+1) / alibi_heads) * (k - q) for query head h (alibi.py:5-9).
+   * softcap > 0 applies softcap * tanh(x / softcap) (softcap.py:48). */
+  int32_t alibi_heads;
+  float softcap;
+
+  /* Optional additive biases (evoformer.py:26-27), bf16, logical shape [B, Hq, Lq, Lk] with
+   * strides in elements over (batch / bias_batch_div, head, q, k); a stride of 0 broadcasts; the k
+   * stride must be 1 (or 0 when Lk == 1). */
+  const void* bias[2];
+  int64_t bias_strides[2][4];
+  int32_t bias_batch_div[2];
+
+  /* Optional sigmoid gate: out *= sigmoid(gate); bf16 gate logits addressed like `o` with gate_strides.
+   * No counterpart in the reference (Evoformer gating is applied outside evoformer.py:8-36). */
+  const void* gate;
+  int64_t gate_strides[4];
+
+  /* diff != 0: out = softmax(q0 k0^T) v - lambda * softmax(q1 k1^T) v  (diff_attn.py:29) */
+  int32_t diff;
+  float lambda;
+
+  int32_t dtype; /* enum fl_dtype */
+
+  /* Scratch for the document-mask tile table; size from fl_workspace_bytes(); may be NULL otherwise. */
+  void* workspace;
+  uint64_t workspace_bytes;
+
+  /* Test hook: when non-NULL, a uint8 [B, Hq, Lq, Lk] buffer, zeroed by the caller; the kernel writes 1
+   * for every (q, k) pair it attends (after tile skipping and the element predicate). */
+  uint8_t* attended_dump;
+
+  int32_t reserved[8]; /* must be 0 */
+} fl_attn_params;
+
+/* ABI version of the loaded library (FL_ABI_VERSION it was built with). */
+int fl_version(void);
+
+/* sizeof(fl_attn_params) in the loaded library, for bindings to check their own mirror of the struct. */
+uint64_t fl_params_sizeof(void);
+
+/* Message for the last negative/positive return on this thread ("" if none). */
+const char* fl_last_error(void);
+
+/* Host-only argument check: the same validation fl_attn_fwd runs before it launches.  Touches no GPU. */
+int fl_attn_validate(const fl_attn_params* p);
+
+/* Bytes of device scratch fl_attn_fwd needs for *p (0 unless a document mask is used). */
+uint64_t fl_workspace_bytes(const fl_attn_params* p);
+
+/* Runs the fused forward on hipStream_t `stream` (NULL = default stream).
+ * Replaces torch.compile(fn)(q, k, v, ...) for the functions of attention_variants/. */
+int fl_attn_fwd(const fl_attn_params* p, void* stream);
+
+/* Describes the kernel instance fl_attn_fwd would pick for *p: tile sizes and launch shape.
+ * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
+int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHLIGHT_AMD_H */

@@ -1,0 +1,37 @@
+"""Shared argument handling for the variant front-ends."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _ffi
+
+
+def check_heads(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, enable_gqa: bool) -> None:
+    for name, t in (("query", query), ("key", key), ("value", value)):
+        if t.dim() != 4:
+            raise ValueError(f"{name} must be [N, H, L, E], got shape {tuple(t.shape)}")
+    hq, hkv = query.size(1), key.size(1)
+    if value.size(1) != hkv:
+        raise ValueError(f"key has {hkv} heads but value has {value.size(1)}")
+    if enable_gqa:
+        if hq % hkv:
+            raise ValueError(f"enable_gqa: {hq} query heads are not a multiple of {hkv} key/value heads")
+    elif hq != hkv and hkv != 1:  # a single key/value head broadcasts in the reference's matmul
+        raise ValueError(f"{hq} query heads vs {hkv} key/value heads: pass enable_gqa=True for grouped-query attention")
+
+
+def grouped_view(out: torch.Tensor, key: torch.Tensor, enable_gqa: bool) -> torch.Tensor:
+    """Result layout of the reference's variants under GQA: [N, Hkv, G, L, Ev] (they never view back, e.g.
+    attention_variants/causal.py:27-36).  Same memory as the 4-D result."""
+    if not enable_gqa:
+        return out
+    n, hq, l, ev = out.shape
+    hkv = key.size(1)
+    return out.view(n, hkv, hq // hkv, l, ev)
+
+
+def run(query, key, value, *, scale: Optional[float], enable_gqa: bool, **kw) -> torch.Tensor:
+    check_heads(query, key, value, enable_gqa)
+    return _ffi.attn_fwd(query, key, value, scale=scale, **kw)

@@ -1,0 +1,40 @@
+"""CPU oracle for the fused attention forward path.  TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+This package restates, in plain eager PyTorch (fp32 unless the caller passes another dtype), what the reference's
+attention_variants/*.py compute.  It is the checker for the HIP kernels: only tests/, __graft_entry__.smoke() and
+the `cpu_baseline` leg of bench.py may import it.  flashlight_amd/ never does.
+
+How each function is pinned (tests/test_oracle_pinned.py) without running the reference:
+  vanilla / GQA      torch.nn.functional.scaled_dot_product_attention; pure-Python triple loop at S <= 12
+  causal             SDPA is_causal=True; row 0 equals value[0]
+  sliding window     SDPA with a loop-built boolean mask; W >= S-1 == causal; W == 0 returns value
+  prefix-LM          SDPA with a loop-built mask; P <= 1 == causal; P >= S == vanilla
+  document mask      SDPA with a loop-built mask; equals independent attention per document
+  ALiBi              SDPA with a loop-built float mask; zero slopes == vanilla
+  softcap            pure-Python loop with math.tanh; cap -> inf == vanilla
+  diff-attn          difference of two SDPA calls; lambda = 0 == branch 0; equal branches == (1 - lambda) * SDPA
+  Evoformer          SDPA on transposed inputs with the summed bias as float mask; zero bias == vanilla
+  gate               elementwise sigmoid written with math.exp in a loop
+The committed fixtures under tests/golden/ were produced by tests/golden/make_golden.py from those library
+routines (never from this package), so they pin it from outside as well.
+"""
+from .attention import (  # noqa: F401
+    alibi_slopes,
+    attention_alibi,
+    attention_causal,
+    attention_document_mask,
+    attention_evoformer,
+    attention_prefix_lm,
+    attention_sliding_window,
+    attention_softcapped,
+    attention_vanilla,
+    attention_vanilla_nogqa,
+    diff_attention,
+    tanh_softcap,
+)
+from .masks import (  # noqa: F401
+    attend_matrix,
+    attended_pairs,
+    document_lengths_cfg3,
+    document_ids_from_lengths,
+)

@@ -1,0 +1,140 @@
+"""The C-ABI library: loads without a GPU, exports what include/flashlight_amd.h declares, and validates arguments
+on the host (no launch).  Device pointers are faked with aligned integers; nothing here dereferences them."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+from flashlight_amd import _ffi
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "flashlight_amd.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not _ffi.LIB_PATH.exists():
+        from flashlight_amd import build
+        build.build(force=False)
+    return _ffi.load_library()
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return re.findall(r"^\s*(?:const\s+)?[\w\s\*]+?\b(fl_\w+)\s*\(", text, flags=re.M)
+
+
+def test_exports_every_declared_symbol(lib):
+    names = declared_functions()
+    assert {"fl_version", "fl_last_error", "fl_attn_validate", "fl_workspace_bytes", "fl_attn_fwd", "fl_attn_plan",
+            "fl_params_sizeof"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+
+
+def test_version_and_struct_size(lib):
+    assert lib.fl_version() == _ffi.ABI_VERSION
+    assert lib.fl_params_sizeof() == C.sizeof(_ffi.FlAttnParams)
+
+
+def good_params(B=2, Hq=4, Hkv=2, L=300, D=64, Dv=None):
+    Dv = Dv or D
+    p = _ffi.FlAttnParams()
+    p.q, p.k, p.v, p.o = 0x10000, 0x20000, 0x30000, 0x40000
+    p.q_strides[:] = (Hq * L * D, L * D, D, 1)
+    p.k_strides[:] = (Hkv * L * D, L * D, D, 1)
+    p.v_strides[:] = (Hkv * L * Dv, L * Dv, Dv, 1)
+    p.o_strides[:] = (Hq * L * Dv, L * Dv, Dv, 1)
+    p.B, p.Hq, p.Hkv, p.Lq, p.Lk, p.Dqk, p.Dv = B, Hq, Hkv, L, L, D, Dv
+    p.scale = 0.125
+    return p
+
+
+def rc(lib, p):
+    return lib.fl_attn_validate(C.byref(p))
+
+
+def test_valid_params_pass(lib):
+    for D in (32, 64, 128):
+        assert rc(lib, good_params(D=D)) == 0, _ffi.last_error()
+    p = good_params()
+    p.mask_kind, p.window = _ffi.MASK_SLIDING, 17
+    assert rc(lib, p) == 0
+    assert _ffi.last_error() == ""
+
+
+def test_plan_reports_launch_shape(lib):
+    p = good_params(B=2, Hq=4, L=300, D=128)
+    plan = _ffi.plan(p)
+    assert plan["threads"] % 64 == 0 and plan["lds_bytes"] <= 160 * 1024
+    bm = plan["rows_per_workgroup"]
+    assert plan["workgroups"] == 2 * 4 * ((300 + bm - 1) // bm)
+
+
+@pytest.mark.parametrize("mutate, code, word", [
+    (lambda p: setattr(p, "q", 0), -1, "q pointer is null"),
+    (lambda p: setattr(p, "o", None), -1, "o pointer"),
+    (lambda p: setattr(p, "k", 0x20008), -7, "16-byte"),
+    (lambda p: setattr(p, "Lq", 0), -2, "positive"),
+    (lambda p: setattr(p, "Hq", 3), -2, "multiple"),
+    (lambda p: p.q_strides.__setitem__(3, 2), -3, "stride must be 1"),
+    (lambda p: p.k_strides.__setitem__(2, 63), -7, "multiple of 8"),
+    (lambda p: setattr(p, "scale", 0.0), -5, "scale"),
+    (lambda p: setattr(p, "scale", float("nan")), -5, "scale"),
+    (lambda p: setattr(p, "mask_kind", 9), -5, "mask_kind"),
+    (lambda p: (setattr(p, "mask_kind", _ffi.MASK_SLIDING), setattr(p, "window", -1)), -5, "window"),
+    (lambda p: (setattr(p, "mask_kind", _ffi.MASK_PREFIX_LM), setattr(p, "Lk", 299)), -2, "Lq == Lk"),
+    (lambda p: setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), -1, "doc_ids"),
+    (lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000)), -6, "workspace"),
+    (lambda p: setattr(p, "softcap", -1.0), -5, "softcap"),
+    (lambda p: setattr(p, "alibi_heads", -2), -5, "alibi"),
+    (lambda p: setattr(p, "dtype", 3), -4, "dtype"),
+    (lambda p: (setattr(p, "Dqk", 48), setattr(p, "Dv", 48)), -4, "no kernel instance"),
+    (lambda p: (setattr(p, "diff", 1), setattr(p, "lambda_", float("inf"))), -5, "lambda"),
+    (lambda p: p.reserved.__setitem__(0, 1), -5, "reserved"),
+    (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 0)), -5, "bias_batch_div"),
+    (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 1),
+                p.bias_strides[0].__setitem__(3, 2)), -3, "key stride"),
+    (lambda p: setattr(p, "gate", 0x70004), -7, "gate"),
+])
+def test_invalid_arguments_are_rejected_without_a_launch(lib, mutate, code, word):
+    p = good_params()
+    mutate(p)
+    assert rc(lib, p) == code, _ffi.last_error()
+    assert word in _ffi.last_error()
+    # fl_attn_fwd runs the same check first and must not reach the GPU
+    assert lib.fl_attn_fwd(C.byref(p), None) == code
+
+
+def test_null_params(lib):
+    assert lib.fl_attn_validate(None) == -1
+    assert lib.fl_workspace_bytes(None) == 0
+
+
+def test_workspace_size_for_document_masks(lib):
+    p = good_params(B=3, L=1000)
+    assert lib.fl_workspace_bytes(C.byref(p)) == 0
+    p.mask_kind = _ffi.MASK_DOCUMENT_CAUSAL
+    assert lib.fl_workspace_bytes(C.byref(p)) == 3 * ((1000 + 31) // 32) * 16
+    p.doc_ids, p.workspace, p.workspace_bytes = 0x50000, 0x80000, 3 * 32 * 16
+    assert rc(lib, p) == 0, _ffi.last_error()
+    p.workspace_bytes -= 1
+    assert rc(lib, p) == -6
+
+
+def test_too_many_keys_is_an_error_not_a_fault(lib):
+    p = good_params(B=1, Hq=1, Hkv=1, L=64 * 4096 + 64, D=64)
+    assert rc(lib, p) == -2 and "maximum" in _ffi.last_error()
+
+
+def test_front_end_refuses_cpu_and_fp32_tensors(lib):
+    import torch
+    from flashlight_amd.attention_variants import attention_pytorch_causal, attention_pytorch_alibi
+    q = torch.randn(1, 2, 16, 64)
+    with pytest.raises(NotImplementedError, match="no CPU path"):
+        attention_pytorch_causal(q.bfloat16(), q.bfloat16(), q.bfloat16())
+    with pytest.raises(NotImplementedError):
+        attention_pytorch_alibi(q, q, q, score_mod=lambda a, b: None)
+    with pytest.raises(TypeError):
+        attention_pytorch_alibi(q, q, q)

@@ -1,0 +1,259 @@
+"""Parity of the HIP kernels (through the C ABI) with the CPU oracle and the committed known-answer vectors.
+Tolerance: bf16 kernel against an fp32/fp64 reference, max-abs 2e-2 and mean-abs 2e-3."""
+import math
+import random
+
+import pytest
+import torch
+
+import flashlight_amd.attention_variants as A
+import oracle as O
+from flashlight_amd import _ffi
+from flashlight_amd import workloads as W
+from tests.conftest import assert_parity
+from tests.variant_calls import GOLDEN_NAMES, hip_call
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def f32(*ts):
+    return tuple(t.float() for t in ts)
+
+
+def qkv(B, Hq, Hkv, S, D, Dv=None, seed=0, lo_hi=None):
+    g = torch.Generator().manual_seed(seed)
+    shapes = [(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, Dv or D)]
+    if lo_hi is None:
+        ts = [torch.randn(s, generator=g) for s in shapes]
+    else:  # the reference's tests draw uniformly in [-9, 9] (torch.testing.make_tensor defaults)
+        ts = [torch.rand(s, generator=g) * (lo_hi[1] - lo_hi[0]) + lo_hi[0] for s in shapes]
+    return tuple(t.to(torch.bfloat16).to(DEV) for t in ts)
+
+
+@pytest.mark.parametrize("name", GOLDEN_NAMES)
+def test_known_answer_vectors(golden, name):
+    case = golden[name]
+    out = hip_call(name, case.to(DEV), case.meta)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16
+    assert_parity(out, case.expected, name)
+
+
+def oracle_for(w: W.Workload, t: dict, q_block):
+    """fp32 oracle evaluation of a benchmark workload, on the tensors' device (plain eager PyTorch either way)."""
+    q, k, v = f32(t["q"], t["k"], t["v"])
+    n = w.name.split("/")[1]
+    if n == "vanilla":
+        return O.attention_vanilla(q, k, v, q_block=q_block)
+    if n == "causal":
+        return O.attention_causal(q, k, v, q_block=q_block)
+    if n == "sliding_window":
+        win = W.pairs_sliding  # noqa: F841  (window recovered from the pair count below)
+        S = q.size(2)
+        window = next(x for x in (256, 128, 64, 32, 16) if W.pairs_sliding(S, x) == w.pairs_per_head)
+        return O.attention_sliding_window(q, k, v, window_size=window, q_block=q_block)
+    if n == "gqa_alibi_softcap_causal":
+        return O.attention_alibi(q, k, v, score_mod=q.size(1), is_causal=True, honor_causal=True, enable_gqa=True,
+                                 softcap=50.0, q_block=q_block)
+    if n == "document_mask_causal":
+        return O.attention_document_mask(q, k, v, t["document_id"], is_causal=True, q_block=q_block)
+    if n == "prefix_lm":
+        S = q.size(2)
+        P = next(x for x in (1024, 512, 256, 128, 64) if W.pairs_prefix(S, x) == w.pairs_per_head)
+        return O.attention_prefix_lm(q, k, v, prefix_lengths=P, q_block=q_block)
+    if n == "diff_attn_causal":
+        return O.diff_attention(q, k, v, lambda_full=0.8, is_causal=True, q_block=q_block)
+    if n == "evoformer_bias_gate":
+        return O.attention_evoformer(q, k, v, [t["pair_bias"].float()], gate=t["gate"].float(), q_block=q_block)
+    raise KeyError(w.name)
+
+
+WORKLOAD_NAMES = [w.name for w in W.build_workloads()]
+
+
+@pytest.mark.parametrize("name", WORKLOAD_NAMES)
+def test_benchmark_configs_reduced(name):
+    """Every benchmark configuration at 1/4 sequence length, oracle on the host CPU."""
+    w = W.workload_by_name(name, scale_down=4)
+    t = w.make(DEV)
+    out = w.call(t)
+    torch.cuda.synchronize()
+    ref = oracle_for(w, {k: v.cpu() for k, v in t.items()}, q_block=512)
+    assert_parity(out, ref, name)
+
+
+@pytest.mark.parametrize("name", WORKLOAD_NAMES)
+def test_benchmark_configs_full_size(name):
+    """Full BASELINE sizes.  The oracle (same eager fp32 code) is evaluated on the GPU tensors, in blocks of
+    query rows, because the dense score matrices do not fit a CPU run of a few seconds."""
+    w = W.workload_by_name(name)
+    t = w.make(DEV)
+    out = w.call(t)
+    torch.cuda.synchronize()
+    ref = oracle_for(w, t, q_block=512)
+    assert_parity(out, ref, name)
+    del ref, out, t
+    torch.cuda.empty_cache()
+
+
+# ---- shapes and input distribution of the reference's own test scripts (tests/test_*.py there), sequence lengths
+# ---- kept, batch reduced where the fp32 oracle would not fit; inputs uniform in [-9, 9] like make_tensor.
+# ---- Outputs reach magnitude 9 there, where one bf16 ulp is 0.03, so these use the tolerance those scripts state:
+# ---- assert_close(atol=2e-2, rtol=1e-2) (e.g. tests/test_causal.py:36 of the reference).
+
+def assert_script_tolerance(out, ref, what=""):
+    assert tuple(out.shape) == tuple(ref.shape), what
+    torch.testing.assert_close(out.float(), ref.float().to(out.device), atol=2e-2, rtol=1e-2, msg=lambda m: f"{what}: {m}")
+
+
+def test_reference_script_vanilla_and_causal():   # tests/test_vanilla.py:21-36, tests/test_causal.py:21-36
+    q, k, v = qkv(2, 1, 1, 16384, 128, seed=1, lo_hi=(-9, 9))
+    assert_script_tolerance(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v), q_block=1024), "vanilla")
+    assert_script_tolerance(A.attention_pytorch_causal(q, k, v), O.attention_causal(*f32(q, k, v), q_block=1024), "causal")
+
+
+def test_reference_script_alibi():                 # tests/test_alibi.py:20-40
+    q, k, v = qkv(4, 16, 2, 1024, 64, seed=2, lo_hi=(-9, 9))
+    out = A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(q.size(-3)), enable_gqa=True)
+    assert out.shape == (4, 2, 8, 1024, 64)
+    assert_script_tolerance(out, O.attention_alibi(*f32(q, k, v), score_mod=16, enable_gqa=True), "alibi")
+
+
+def test_reference_script_sliding_window():        # tests/test_sliding_window.py:13-33
+    q, k, v = qkv(4, 16, 2, 1024, 64, seed=3, lo_hi=(-9, 9))
+    out = A.attention_pytorch_sliding_window(q, k, v, window_size=256, enable_gqa=True)
+    assert_script_tolerance(out, O.attention_sliding_window(*f32(q, k, v), window_size=256, enable_gqa=True), "sliding")
+
+
+def test_reference_script_prefix_lm():             # tests/test_prefix_lm.py:14-34 (batch 32 -> 4)
+    q, k, v = qkv(4, 16, 2, 1024, 64, seed=4, lo_hi=(-9, 9))
+    out = A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=256, enable_gqa=True)
+    assert_script_tolerance(out, O.attention_prefix_lm(*f32(q, k, v), prefix_lengths=256, enable_gqa=True), "prefix")
+
+
+def test_reference_script_document_mask():         # tests/test_document_mask.py:15-35
+    q, k, v = qkv(1, 16, 2, 16384, 64, seed=5, lo_hi=(-9, 9))
+    random.seed(0)
+    ids = A.create_document_id(1, 16384, 12, device=DEV)
+    assert ids.shape == (1, 16384) and ids.dtype == torch.int64 and int(ids.max()) == 11
+    out = A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True)
+    assert_script_tolerance(out, O.attention_document_mask(*f32(q, k, v), ids, enable_gqa=True, q_block=1024), "document")
+
+
+def test_reference_script_gqa():                   # tests/test_gqa.py:69-96 (batch 32 -> 2), tolerance 1e-2 there
+    q, k, v = qkv(2, 16, 2, 4096, 64, seed=6, lo_hi=(-9, 9))
+    out = A.attention_pytorch(q, k, v, enable_gqa=True)
+    assert out.shape == (2, 16, 4096, 64)
+    assert_script_tolerance(out, O.attention_vanilla(*f32(q, k, v), enable_gqa=True, q_block=1024), "gqa")
+
+
+def test_reference_script_diffattn():              # tests/test_diffattn.py:20-41 uses head_dim 128 / value dim 256,
+    # which has no kernel instance yet; the benchmark's head_dim 64 / value dim 128 shape is checked instead
+    q, k, v = qkv(4, 16, 16, 1024, 64, Dv=128, seed=7, lo_hi=(-9, 9))
+    v = v[:, :8].contiguous()
+    assert_script_tolerance(A.diffattn(q, k, v), O.diff_attention(*f32(q, k, v)), "diffattn")
+
+
+def test_reference_script_evoformer():             # tests/test_evoattn.py:21-71 (randn inputs, batch 2)
+    g = torch.Generator().manual_seed(8)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)
+    B, N, S, H, D = 2, 256, 256, 4, 32
+    Q, K, V = mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D)
+    b1, b2 = mk(B, N, 1, 1, S), mk(B, 1, H, S, S)
+    out = A.attention_reference(Q, K, V, [b1, b2], 1 / math.sqrt(D))
+    assert out.shape == (B, N, S, H, D)
+    ref = O.attention_evoformer(*f32(Q, K, V), [b1.float(), b2.float()], 1 / math.sqrt(D))
+    assert_script_tolerance(out, ref, "evoformer")
+
+
+# ---- edge cases ----------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("S", [1, 2, 31, 63, 64, 65, 255, 256, 257, 1000])
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_ragged_lengths(S, D):
+    q, k, v = qkv(1, 2, 1, S, D, seed=S + D)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch(q, k, v, enable_gqa=True), O.attention_vanilla(qf, kf, vf, enable_gqa=True))
+    assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True).flatten(1, 2),
+                  O.attention_causal(qf, kf, vf, enable_gqa=True).flatten(1, 2))
+    assert_parity(A.attention_pytorch_sliding_window(q, k, v, window_size=40, enable_gqa=True),
+                  O.attention_sliding_window(qf, kf, vf, window_size=40, enable_gqa=True))
+
+
+def test_cross_attention_lengths_differ():
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(2, 2, 300, 64, generator=g).bfloat16().to(DEV)
+    k = torch.randn(2, 2, 77, 64, generator=g).bfloat16().to(DEV)
+    v = torch.randn(2, 2, 77, 64, generator=g).bfloat16().to(DEV)
+    assert_parity(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v)))
+    # causal is top-left aligned (causal.py:32): query rows beyond the keys see every key
+    assert_parity(A.attention_pytorch_causal(q, k, v), O.attention_causal(*f32(q, k, v)))
+    assert_parity(A.attention_pytorch_causal(k, q, q), O.attention_causal(*f32(k, q, q)))
+
+
+def test_strided_inputs_and_explicit_scale():
+    g = torch.Generator().manual_seed(12)
+    packed = torch.randn(2, 200, 3, 4, 64, generator=g).bfloat16().to(DEV)   # [B, S, 3, H, D] as benchmarks/_utils.py:221-240
+    q, k, v = (packed[:, :, i].transpose(1, 2) for i in range(3))            # non-contiguous [B, H, S, D] views
+    assert not q.is_contiguous()
+    assert_parity(A.attention_pytorch(q, k, v, scale=0.3), O.attention_vanilla(*f32(q, k, v), scale=0.3))
+    assert_parity(A.attention_pytorch_causal(q, k, v, scale=0.05), O.attention_causal(*f32(q, k, v), scale=0.05))
+
+
+def test_document_ids_arbitrary_values_and_per_batch():
+    q, k, v = qkv(2, 2, 2, 500, 64, seed=13)
+    g = torch.Generator().manual_seed(14)
+    ids = torch.randint(-3, 3, (2, 500), generator=g).to(DEV) * 1_000_000_007   # large, unsorted, negative
+    for causal in (False, True):
+        out = A.attention_pytorch_document_mask(q, k, v, ids, is_causal=causal)
+        assert_parity(out, O.attention_document_mask(*f32(q, k, v), ids, is_causal=causal), f"causal={causal}")
+
+
+def test_large_logits_and_masked_neighbours_stay_finite():
+    q, k, v = qkv(1, 2, 2, 512, 128, seed=15)
+    q = (q.float() * 30).bfloat16()
+    out = A.attention_pytorch_causal(q, k, v)
+    assert_parity(out, O.attention_causal(*f32(q, k, v)))
+
+
+def test_softcap_default_threshold_and_causal_extension():
+    q, k, v = qkv(1, 4, 4, 300, 64, seed=16)
+    q = (q.float() * 6).bfloat16()
+    assert_parity(A.attention_softcapped(q, k, v), O.attention_softcapped(*f32(q, k, v), score_mod=30.0))
+    assert_parity(A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(10.0), is_causal=True),
+                  O.attention_softcapped(*f32(q, k, v), score_mod=10.0, is_causal=True, honor_causal=True))
+
+
+def test_evoformer_bias_layouts():
+    g = torch.Generator().manual_seed(17)
+    mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(DEV)
+    B, N, S, H, D = 2, 5, 100, 4, 32
+    Q, K, V = mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D)
+    cases = {
+        "pair only": [mk(B, 1, H, S, S)],
+        "mask only": [mk(B, N, 1, 1, S)],
+        "shared pair": [mk(1, 1, H, S, S)],
+        "three biases": [mk(B, N, 1, 1, S), mk(B, 1, H, S, S), mk(1, 1, 1, S, S)],
+        "full": [mk(B, N, H, S, S)],
+        "none": [],
+    }
+    for name, biases in cases.items():
+        out = A.attention_reference(Q, K, V, biases)
+        ref = O.attention_evoformer(*f32(Q, K, V), [b.float() for b in biases])
+        assert_parity(out, ref, name)
+
+
+def test_front_end_errors_on_gpu_tensors():
+    q, k, v = qkv(1, 4, 2, 64, 64)
+    with pytest.raises(ValueError, match="enable_gqa"):
+        A.attention_pytorch_causal(q, k, v)
+    with pytest.raises(NotImplementedError, match="bfloat16"):
+        A.attention_pytorch(q.float(), k.float(), v.float(), enable_gqa=True)
+    with pytest.raises(AssertionError):
+        A.attention_pytorch_sliding_window(q, k[:, :, :32], v[:, :, :32], enable_gqa=True)
+    with pytest.raises(ValueError, match="generated for"):
+        A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(8), enable_gqa=True)
+    q48 = torch.randn(1, 2, 64, 48, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
+        A.attention_pytorch(q48, q48, q48)

@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-other-configs] [--calibrate-copy]
+
+A step is one pass of the hot path over the benchmark batch of BASELINE config 1 (B=4, H=16, S=4096, D=128, bf16,
+seeded N(0,1) inputs already resident in HBM): one vanilla, one causal and one sliding-window (window 256) forward,
+three kernel launches.  `value` is the unmasked (algorithmic) FLOPs of the step divided by its wall time.  Prints one
+JSON line; per-variant numbers, the roofline of the dominant kernel, the other configurations (measured outside the
+timed region) and the CPU baseline ride along in it.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the eager CPU timing (about 20 s)")
+    ap.add_argument("--no-other-configs", action="store_true", help="only run the configuration the metric is quoted on")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one 256 MiB device-to-device copy (known traffic, for scaling rocprofv3 counters)")
+    return ap.parse_args()
+
+
+def event_pair():
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def time_launches(fn, iters: int, warmup: int = 3):
+    """Mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
+    current stream (the stream the kernels are launched on)."""
+    for _ in range(warmup):
+        fn()
+    pairs = [event_pair() for _ in range(iters)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in pairs]
+    return statistics.fmean(ts), statistics.median(ts)
+
+
+def cpu_baseline(threads_hint: int = 0) -> dict:
+    """The eager fp32 restatement of the reference's CPU-runnable path (oracle/), timed on this host's cores on a
+    bounded sample of the benchmark workload: the same three variants at the same S and D, on 1 batch x 2 heads."""
+    import oracle as O  # the checker, imported here only to be timed as the CPU baseline
+    from flashlight_amd import workloads as W
+
+    B, H, S, D = 1, 2, 4096, 128
+    g = torch.Generator().manual_seed(1001)
+    q, k, v = (torch.randn(B, H, S, D, generator=g) for _ in range(3))
+    fns = {"vanilla": lambda: O.attention_vanilla(q, k, v),
+           "causal": lambda: O.attention_causal(q, k, v),
+           "sliding_window": lambda: O.attention_sliding_window(q, k, v, window_size=256)}
+    pairs = {"vanilla": W.pairs_none(S), "causal": W.pairs_causal(S), "sliding_window": W.pairs_sliding(S, 256)}
+    flops = sum(4 * D * p * B * H for p in pairs.values())
+    for f in fns.values():
+        f()  # warm-up
+    reps, t_total = 0, 0.0
+    per = {n: [] for n in fns}
+    while reps < 3 or (t_total < 10.0 and reps < 40):
+        for n, f in fns.items():
+            t0 = time.perf_counter()
+            f()
+            per[n].append(time.perf_counter() - t0)
+        t_total = sum(sum(x) for x in per.values())
+        reps += 1
+    step_s = sum(statistics.fmean(x) for x in per.values())
+    # configuration 0 of the baseline file: causal, B=2 H=8 S=512 D=64 fp32, the reference's own CPU-sized case
+    g0 = torch.Generator().manual_seed(1000)
+    q0, k0, v0 = (torch.randn(2, 8, 512, 64, generator=g0) for _ in range(3))
+    O.attention_causal(q0, k0, v0)
+    t0s = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        O.attention_causal(q0, k0, v0)
+        t0s.append(time.perf_counter() - t0)
+    cfg0_flops = 4 * 64 * W.pairs_causal(512) * 16
+    return {
+        "value": flops / step_s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"eager fp32 oracle, dense scores like the reference, vanilla+causal+sliding(256) at B={B} H={H} "
+                  f"S={S} D={D} ({reps} reps, {t_total:.1f} s); unmasked FLOPs",
+        "ms_per_variant": {n: 1e3 * statistics.fmean(x) for n, x in per.items()},
+        "host_cpus": os.cpu_count(),
+        "cfg0_causal_fp32_B2_H8_S512_D64": {"ms": 1e3 * statistics.median(t0s),
+                                              "unmasked_GFLOPs": cfg0_flops / statistics.median(t0s) / 1e9},
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the fused forward is a single-device kernel and this build has no "
+                 "multi-GPU path; run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X: no GPU is visible and there is no CPU execution path")
+    from flashlight_amd import _ffi
+    from flashlight_amd import workloads as W
+
+    _ffi.load_library()  # fail loudly if the HIP extension is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    all_w = W.build_workloads()
+    cfg1 = [w for w in all_w if w.config == 1]
+    tens = cfg1[0].make(dev)  # the three variants share q, k, v (same seed)
+    step_flops = sum(w.flops for w in cfg1)
+
+    def step():
+        for w in cfg1:
+            w.call(tens)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-launch durations of each variant, HIP events on the launch stream
+    variants = {}
+    for w in cfg1:
+        mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(20, args.steps))
+        tf = w.flops / mean_ms / 1e9
+        variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
+                            "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
+                            "hbm_floor_GBps_at_this_time": w.min_bytes / mean_ms / 1e6}
+    dom = max(cfg1, key=lambda w: variants[w.name]["ms"])  # the launch that dominates the step
+    dv = variants[dom.name]
+    roofline = {"bound": "mfma", "kernel": f"fl::fwd_kernel ({dom.name})", "achieved": dv["tflops"],
+                "peak": W.PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dv["tflops"] / W.PEAK_BF16_TFLOPS,
+                "traffic": None, "launch_ms": dv["ms"], "flops_per_launch": dom.flops}
+
+    others = {}
+    if not args.no_other_configs:
+        del tens
+        for w in all_w:
+            if w.config == 1:
+                continue
+            t = w.make(dev)
+            mean_ms, med_ms = time_launches(lambda: w.call(t), iters=20)
+            tf = w.flops / mean_ms / 1e9
+            others[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf,
+                              "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS, "unmasked_flops": w.flops,
+                              "min_bytes": w.min_bytes, "GBps_on_min_bytes": w.min_bytes / mean_ms / 1e6}
+            del t
+            torch.cuda.empty_cache()
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+
+    line = {
+        "metric": "fwd TFLOP/s (unmasked FLOPs)", "value": step_flops / wall_ms / 1e9, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: vanilla + causal + sliding-window(256, causal) forward, "
+                               "B=4 H=16 S=4096 D=128, one launch each per step",
+                   "seed": cfg1[0].seed, "unmasked_flops_per_step": step_flops},
+        "pct_mfma_peak": 100 * step_flops / wall_ms / 1e9 / W.PEAK_BF16_TFLOPS,
+        "peak_used_TFLOPs": W.PEAK_BF16_TFLOPS,
+        "variants": variants, "roofline": roofline, "other_configs": others,
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -14,7 +14,7 @@ from typing import Optional, Sequence
 import torch
 
 LIB_NAME = "libflashlight_amd.so"
-LIB_PATH = Path(__file__).resolve().parent / LIB_NAME
+LIB_PATH = Path(os.environ.get("FL_LIB") or Path(__file__).resolve().parent / LIB_NAME)
 
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING, MASK_PREFIX_LM, MASK_DOCUMENT, MASK_DOCUMENT_CAUSAL = range(6)
 FL_BF16 = 0

@@ -25,9 +25,14 @@ ARCH = "gfx950"
 HIPCC_FLAGS = [
     "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument", "-Wno-ignored-optimization-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm", "-Wno-ignored-optimization-argument",
     f"-I{INCLUDE}", f"-I{CSRC}",
 ]
+
+
+# Development knobs: extra hipcc flags (e.g. -DFL_SCHED=2) and an alternative output path for side-by-side builds.
+HIPCC_FLAGS += os.environ.get("FL_HIPCC_EXTRA", "").split()
+LIB_PATH = Path(os.environ.get("FL_LIB", str(LIB_PATH)))
 
 
 def hipcc() -> str:

@@ -2,6 +2,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "flashlight_amd.h"
@@ -60,12 +61,17 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   const uint32_t want = wanted_features(p);
   const fl::Instance* best = nullptr;
   int best_extra = 1 << 30;
+  // Tuning knob: FL_TILE=<rows per wave>x<keys per tile>x<waves>x<ring depth>, e.g. 32x32x4x4, restricts the choice
+  // to instances of that shape (the default is the first listed instance that fits).
+  int want_rw = 0, want_bn = 0, want_nw = 0, want_ns = 0;
+  if (const char* e = std::getenv("FL_TILE")) std::sscanf(e, "%dx%dx%dx%d", &want_rw, &want_bn, &want_nw, &want_ns);
   for (int i = 0; i < fl::kNumInstances; ++i) {
     const fl::Instance& in = fl::kInstances[i];
     if (in.dqk != p->Dqk || in.dv != p->Dv) continue;
     if ((in.feat & want) != want) continue;
     const uint32_t extra = in.feat & ~want;
     if (extra & ~kOptionalFeatures) continue;
+    if (want_rw && (in.rw != want_rw || in.bn != want_bn || in.nw != want_nw || (want_ns && in.ns != want_ns))) continue;
     const int n = __builtin_popcount(extra);
     if (n < best_extra) {
       best = &in;
@@ -73,6 +79,17 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
     }
   }
   return best;
+}
+
+// LDS bytes of a launch: the instance's fixed part plus 4 bytes per key tile for the tile list.
+int64_t lds_bytes_for(const fl::Instance* in, const fl_attn_params* p) {
+  const int64_t nkt = ((int64_t)p->Lk + in->bn - 1) / in->bn;
+  return in->lds_fixed_bytes + 4 * nkt;
+}
+int64_t max_keys_for(const fl::Instance* in) {
+  int64_t tiles = (fl::kMaxLdsBytes - in->lds_fixed_bytes) / 4;
+  if (tiles > fl::kMaxKeyTiles) tiles = fl::kMaxKeyTiles;
+  return tiles * in->bn;
 }
 
 int check_strides(const char* what, const int64_t* s, int align) {
@@ -153,8 +170,14 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
                 "no kernel instance for Dqk=%d Dv=%d features=0x%x (alibi=1 softcap=2 bias=4 doc=8 diff=16 gate=32 dump=64)",
                 p->Dqk, p->Dv, wanted_features(p));
   const int64_t nkt = ((int64_t)p->Lk + in->bn - 1) / in->bn;
-  if (nkt > fl::kMaxKeyTiles)
-    return fail(FL_ERR_SHAPE, "Lk=%d exceeds the supported maximum of %d keys", p->Lk, fl::kMaxKeyTiles * in->bn);
+  if (nkt > fl::kMaxKeyTiles || lds_bytes_for(in, p) > fl::kMaxLdsBytes)
+    return fail(FL_ERR_SHAPE, "Lk=%d exceeds the supported maximum of %lld keys for this kernel", p->Lk,
+                (long long)max_keys_for(in));
+  // per-lane byte offsets inside one key tile are 32-bit
+  if (((int64_t)in->bn * p->k_strides[2] + p->Dqk) * 2 >= ((int64_t)1 << 31) ||
+      ((int64_t)in->bn * p->v_strides[2] + p->Dv) * 2 >= ((int64_t)1 << 31))
+    return fail(FL_ERR_STRIDE, "key/value sequence stride too large (%lld, %lld elements)", (long long)p->k_strides[2],
+                (long long)p->v_strides[2]);
   const int64_t bm = (int64_t)in->rw * in->nw;
   const int64_t grid = (int64_t)p->B * p->Hq * (((int64_t)p->Lq + bm - 1) / bm);
   if (grid > 0x7fffffff) return fail(FL_ERR_SHAPE, "too many workgroups (%lld)", (long long)grid);
@@ -198,7 +221,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]) {
   out[1] = in->bn;
   out[2] = in->nw * 64;
   out[3] = (int64_t)p->B * p->Hq * ((p->Lq + bm - 1) / bm);
-  out[4] = in->lds_bytes;
+  out[4] = lds_bytes_for(in, p);
   out[5] = in->feat;
   out[6] = 0;
   out[7] = 0;
@@ -235,6 +258,14 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   kp.mask_kind = p->mask_kind;
   kp.window = p->window;
   kp.prefix = p->prefix;
+  {
+    const int kFar = 1 << 29;
+    const bool causal_like = p->mask_kind == FL_MASK_CAUSAL || p->mask_kind == FL_MASK_SLIDING ||
+                             p->mask_kind == FL_MASK_PREFIX_LM || p->mask_kind == FL_MASK_DOCUMENT_CAUSAL;
+    kp.dmax = causal_like ? 0 : kFar;
+    kp.dmin = p->mask_kind == FL_MASK_SLIDING ? -(p->window < kFar ? p->window : kFar) : -kFar;
+    kp.pfx = p->mask_kind == FL_MASK_PREFIX_LM ? (p->prefix < 0 ? 0 : p->prefix) : 0;
+  }
   kp.doc_ids = p->doc_ids;
   kp.doc_stride = p->doc_stride;
   kp.alibi_heads = p->alibi_heads;
@@ -273,7 +304,7 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
     kp.doc_table = table;
     kp.doc_blocks = blocks;
   }
-  hipError_t e = in->launch(kp, grid, stream);
+  hipError_t e = in->launch(kp, grid, (int)lds_bytes_for(in, p), stream);
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));
   return 0;
 }

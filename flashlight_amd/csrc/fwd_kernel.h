@@ -16,6 +16,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace fl {
 
 typedef __bf16 bf16_t;
@@ -40,8 +42,8 @@ enum : uint32_t {
 enum : int { MASK_NONE = 0, MASK_CAUSAL = 1, MASK_SLIDING = 2, MASK_PREFIX = 3, MASK_DOC = 4, MASK_DOC_CAUSAL = 5 };
 enum : int { TILE_EMPTY = 0, TILE_PARTIAL = 1, TILE_FULL = 2 };
 
-// Maximum number of key tiles whose class fits the LDS table.
-constexpr int kMaxKeyTiles = 4096;
+// Key tiles are numbered in 16 bits inside the LDS tile list.
+constexpr int kMaxKeyTiles = 65535;
 // Granularity (positions) of the document-id min/max table built by doc_table_kernel.
 constexpr int kDocBlock = 32;
 
@@ -56,6 +58,8 @@ struct KParams {
   float scale;          // multiplies qk
   float scale_log2;     // scale * log2(e)
   int32_t mask_kind, window, prefix;
+  // element predicate of every positional mask: key < Lk && ((dmin <= key - q <= dmax) || key < pfx)
+  int32_t dmin, dmax, pfx;
   const int64_t* doc_ids;
   int64_t doc_stride;
   const int64_t* doc_table;  // [B][ceil(L/kDocBlock)][2] = (min, max)
@@ -103,18 +107,41 @@ __device__ __forceinline__ float xhalf_sum(float x) {
   return a + b;
 }
 
-// ---- mask logic (integer, shared by the tile classifier and the element predicate) -------------------------------
+// 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane l of the wave reads
+// gbase + voff[l] and writes LDS bytes [lds_base + 16 l, +16).  gbase and lds_base are wave-uniform.  Written as asm
+// so that the compiler does not order later LDS reads of *other* buffers behind it with a vmcnt(0) wait; completion
+// is awaited explicitly (dma_wait) before the barrier that publishes the data.
+__device__ __forceinline__ void dma16(const void* gbase, unsigned voff, unsigned lds_base_uniform) {
+  // readfirstlane pins the (already uniform) base to scalar registers whatever the compiler's divergence analysis says
+  const uint64_t b = reinterpret_cast<uint64_t>(gbase);
+  // (the builtin returns int: go through uint32_t so that the low half is not sign-extended over the high half)
+  const uint64_t gbase_uniform = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
+                                 ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(gbase_uniform), "v"(voff),
+               "s"(lds_base_uniform)
+               : "m0");
+}
 
-// Does query position q attend key position k?  Document ids are compared by the caller.
-__device__ __forceinline__ bool attend_positional(int kind, int q, int k, int window, int prefix) {
-  switch (kind) {
-    case MASK_CAUSAL:
-    case MASK_DOC_CAUSAL: return k <= q;
-    case MASK_SLIDING: return k <= q && q - k <= window;
-    case MASK_PREFIX: return k < prefix || k <= q;
-    default: return true;
+// Waits until at most N of this wave's vector-memory operations (the transfers above included) are outstanding;
+// they complete in issue order.  Leaves the LDS/scalar and export counters alone.
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 0xf) | ((N >> 4) << 14));
+}
+
+// f(integral_constant<int, I>) for I = I0, I0+1, ... < N while f returns true; false if some call returned false.
+template <int I, int N, class F>
+__device__ __forceinline__ bool static_while(F&& f) {
+  if constexpr (I < N) {
+    if (!f(std::integral_constant<int, I>{})) return false;
+    return static_while<I + 1, N>(f);
+  } else {
+    return true;
   }
 }
+
+// ---- mask logic (integer, shared by the tile classifier and the element predicate) -------------------------------
 
 // Class of the key tile [k0, k1) against query rows [q0, q1) for the positional part of the mask.
 // k1 and q1 are exclusive and already clipped to the sequence lengths.
@@ -167,9 +194,45 @@ struct TileLayout {
   }
 };
 
-template <int DQK_, int DV_, int RW_, int BN_, int NW_, uint32_t FEAT_>
+// Scheduling pipeline for the straight-line tile step (see fwd_kernel): instruction classes of
+// __builtin_amdgcn_sched_group_barrier.
+enum : int { SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400 };
+#ifndef FL_SCHED
+#define FL_SCHED 1
+#endif
+
+// Orders the step's instructions as: each first-product MFMA preceded by its K fragment read and followed by a
+// share of the exponential work; each second-product MFMA preceded by its two transposing V reads and followed
+// by a share of the next tile's row maximum.  NA / NB = MFMAs in the two products, VA / VB = vector ops to spread.
+template <int NA, int NB, int VA, int VB>
+__device__ __forceinline__ void sched_tile_step() {
+#if FL_SCHED == 1
+  __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 2, 0);
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+    if (i + 2 < NA) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, VA, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 4, 0);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+    if (i + 2 < NB) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 2, 0);
+    if (VB > 0) __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, VB, 0);
+  }
+#elif FL_SCHED == 2
+  __builtin_amdgcn_iglp_opt(2);
+#elif FL_SCHED == 3
+  __builtin_amdgcn_iglp_opt(3);
+#endif
+}
+
+template <int DQK_, int DV_, int RW_, int BN_, int NW_, uint32_t FEAT_, int NS_ = 4>
 struct FwdTraits {
   static constexpr int DQK = DQK_, DV = DV_, RW = RW_, BN = BN_, NW = NW_;
+  static constexpr int NS = NS_;  // K/V tiles resident in LDS (ring); transfers run NS - 1 tiles ahead of their use
+  static_assert(NS >= 2 && NS <= 8 && NS % 2 == 0, "ring depth (even: the two score buffers alternate with the slots)");
   static constexpr uint32_t FEAT = FEAT_;
   static constexpr int NT = NW * 64;
   static constexpr int BM = NW * RW;
@@ -178,29 +241,43 @@ struct FwdTraits {
   static constexpr int KS = DQK / 16;  // MFMA k-steps of the first product
   static constexpr int DVB = DV / 32;  // 32-wide blocks of the value dimension
   static constexpr int KBYTES = BN * DQK * 2, VBYTES = BN * DV * 2;
-  static constexpr int STAGE = KBYTES + VBYTES;
   static constexpr int K_CHUNKS = BN * DQK / 8, V_CHUNKS = BN * DV / 8;
   static constexpr int K_PER_T = K_CHUNKS / NT, V_PER_T = V_CHUNKS / NT;
   static_assert(K_CHUNKS % NT == 0 && V_CHUNKS % NT == 0, "tile must divide evenly over the threads");
   static_assert(RW % 32 == 0 && BN % 32 == 0 && DQK % 16 == 0 && DV % 32 == 0, "MFMA 32x32x16 blocking");
-  static constexpr int CLS_BYTES = kMaxKeyTiles * 2;
-  static constexpr int LDS_BYTES = 2 * STAGE + CLS_BYTES + 16;
+  static_assert(NW <= 8, "tile classes are packed two bits per wave into 16 bits");
+  // waves per SIMD the register budget is sized for
+  static constexpr int WAVES_PER_EU = (RW == 32) ? 2 : 1;
+  // LDS: K tiles [NS], V tiles [NS], 16 bytes of counters, then the tile list (4 bytes per key tile, sized at launch)
+  static constexpr int K_OFF = 0, V_OFF = NS * KBYTES, META_OFF = NS * (KBYTES + VBYTES), LIST_OFF = META_OFF + 16;
+  static constexpr int LDS_FIXED_BYTES = LIST_OFF;
 };
 
+// The main loop is software-pipelined over key tiles so that one wave keeps both the matrix pipe and the vector
+// ALU busy.  With ta, tb, tc three consecutive non-empty tiles, iteration i does
+//     region A   S(tb) = K(tb).Q^T on MFMA          ||   P(ta) = exp2(S(ta) - m), row sums, bf16 pack   (VALU)
+//     region B   O^T  += V(ta)^T.P(ta)^T on MFMA     ||   running max of S(tb)                            (VALU)
+//     rare       element mask of S(tb) on partial tiles; rescale of O, l when the maximum grew
+// while the global -> LDS transfers of K(tc) and V(tb), issued at the top of the iteration into the buffers that
+// iteration i-1 freed, are in flight; the barrier that ends the iteration publishes them.
 template <class T>
-__global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WAVES_PER_EU, T::WAVES_PER_EU)))
+void fwd_kernel(const KParams p) {
   constexpr int DQK = T::DQK, DV = T::DV, RW = T::RW, BN = T::BN, NW = T::NW, NT = T::NT, BM = T::BM;
   constexpr int QB = T::QB, KB = T::KB, KS = T::KS, DVB = T::DVB;
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kBias = FEAT & F_BIAS, kDoc = FEAT & F_DOC;
   constexpr bool kDiff = FEAT & F_DIFF, kGate = FEAT & F_GATE, kDump = FEAT & F_DUMP;
   constexpr bool kMod = kAlibi || kSoftcap || kBias;  // scores are transformed before the softmax
+  constexpr float kLog2e = 1.4426950408889634f;
   using LK = TileLayout<DQK>;
   using LV = TileLayout<DV>;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint16_t* cls = reinterpret_cast<uint16_t*>(smem + 2 * T::STAGE);
-  int* range = reinterpret_cast<int*>(smem + 2 * T::STAGE + T::CLS_BYTES);  // [0]=first, [1]=last+1 non-empty tile
+  // tile list: one entry per key tile that is not empty for the whole workgroup, in key order:
+  // bits 0-15 tile index, bits 16.. two class bits per wave
+  int* meta = reinterpret_cast<int*>(smem + T::META_OFF);  // [0] = number of list entries
+  uint32_t* tlist = reinterpret_cast<uint32_t*>(smem + T::LIST_OFF);
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
@@ -223,12 +300,7 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
   const int qw0 = q0 + wave * RW;     // first query row of this wave
   const int nk = p.n_ktiles;
 
-  // ---- classify every key tile for every wave -----------------------------------------------------------------
-  if (tid == 0) {
-    range[0] = nk;
-    range[1] = 0;
-  }
-  __syncthreads();
+  // ---- classify every key tile for every wave, then compact the non-empty ones into the tile list ---------------
   {
     const int64_t* dtab = kDoc ? p.doc_table + (int64_t)batch * p.doc_blocks * 2 : nullptr;
     int64_t qmn[NW], qmx[NW];
@@ -260,15 +332,27 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
         }
         c |= (unsigned)cw << (2 * w);
       }
-      cls[t] = (uint16_t)c;
-      if (c) {
-        atomicMin(&range[0], t);
-        atomicMax(&range[1], t + 1);
-      }
+      tlist[t] = (c << 16) | (unsigned)t;
     }
   }
   __syncthreads();
-  const int t_first = __builtin_amdgcn_readfirstlane(range[0]), t_end = __builtin_amdgcn_readfirstlane(range[1]);
+  if (wave == 0) {
+    // in-place compaction by one wave, 64 tiles at a time: an entry never moves to a higher index, and every chunk
+    // is read completely before it is written
+    int count = 0;
+    for (int base = 0; base < nk; base += 64) {
+      const int t = base + lane;
+      const uint32_t e = t < nk ? tlist[t] : 0u;
+      const bool keep = (e >> 16) != 0;
+      const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
+      const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+      if (keep) tlist[pos] = e;
+      count += __builtin_popcountll(m);
+    }
+    if (lane == 0) meta[0] = count;
+  }
+  __syncthreads();
+  const int n_list = __builtin_amdgcn_readfirstlane(meta[0]);
 
   // ---- per-lane constants ----------------------------------------------------------------------------------------
   int qrow[QB];  // query position owned by this lane in each query block
@@ -277,21 +361,24 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
 
   float slope_l2 = 0.f;  // ALiBi slope in log2 units
   if constexpr (kAlibi)
-    slope_l2 = p.alibi_heads > 0 ? exp2f(-8.0f * (float)(head + 1) / (float)p.alibi_heads) * 1.4426950408889634f : 0.f;
+    slope_l2 = p.alibi_heads > 0 ? exp2f(-8.0f * (float)(head + 1) / (float)p.alibi_heads) * kLog2e : 0.f;
   float cap_k1 = 0.f, cap_c = 0.f;
   if constexpr (kSoftcap) {
-    cap_k1 = p.scale / p.softcap * 2.0f * 1.4426950408889634f;  // exp2 argument of e^{2x/cap}
-    cap_c = p.softcap * 1.4426950408889634f;                    // cap in log2 units
+    cap_k1 = p.scale / p.softcap * 2.0f * kLog2e;  // exp2 argument of e^{2x/cap}
+    cap_c = p.softcap * kLog2e;                    // cap in log2 units
   }
   int64_t qdoc[QB];
   if constexpr (kDoc) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
-      qdoc[qb] = qrow[qb] < p.Lq ? p.doc_ids[(int64_t)batch * p.doc_stride + qrow[qb]] : 0;
+      qdoc[qb] = p.doc_ids[(int64_t)batch * p.doc_stride + min(qrow[qb], p.Lq - 1)];
   }
+  const float c2 = kMod ? 1.0f : p.scale_log2;  // s * c2 is the logit in log2 units
+  // The running maximum only moves when some row of the wave sees a score more than kTau (log2 units) above it,
+  // so exp2 arguments stay <= kTau and the accumulators are rescaled on few tiles.  Any m gives the same O / l.
+  constexpr float kTau = 8.0f;
 
   f32x16 ofin[kDiff ? DVB : 1][kDiff ? QB : 1];  // branch-0 result kept while branch 1 runs (diff only)
-
   f32x16 oacc[DVB][QB];
   float m_run[QB], l_run[QB];
 
@@ -306,12 +393,8 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        qf[qb][ks] = qrow[qb] < p.Lq
-                         ? *reinterpret_cast<const bf16x8*>(qptr + (int64_t)qrow[qb] * p.qs[2] + ks * 16 + 8 * h)
-                         : z;
-      }
+      for (int ks = 0; ks < KS; ++ks)
+        qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qptr + (int64_t)min(qrow[qb], p.Lq - 1) * p.qs[2] + ks * 16 + 8 * h);
 
 #pragma unroll
     for (int dvb = 0; dvb < DVB; ++dvb)
@@ -325,244 +408,362 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
       l_run[qb] = 0.f;
     }
 
-    // ---- global -> register -> LDS staging of one K/V tile ---------------------------------------------------
-    u32x4 kst[T::K_PER_T], vst[T::V_PER_T];
-    auto load_tile = [&](int t) {
-      const int k0 = t * BN;
+    // ---- global -> LDS, without passing through registers: each wave fills 1 KiB of the tile per transfer, lane l
+    // writing bytes [16 l, 16 l + 16) of that KiB from its own global address.  The LDS image is the swizzled tile, so
+    // lane (row, physical chunk) fetches the logical chunk that maps there (the swizzles are XORs, hence their own
+    // inverses).  The global address is a per-tile scalar base plus a per-lane byte offset that does not change from
+    // tile to tile; only the ragged last tile recomputes it, repeating the last key for rows past the end (those
+    // keys are masked, p = 0).
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;  // LDS byte address of the dynamic segment
+    unsigned koff[T::K_PER_T], voff[T::V_PER_T];
 #pragma unroll
-      for (int it = 0; it < T::K_PER_T; ++it) {
-        int id = it * NT + tid, row = id / LK::CPR, c = id % LK::CPR;
-        u32x4 z = {0, 0, 0, 0};
-        kst[it] = (k0 + row < p.Lk)
-                      ? *reinterpret_cast<const u32x4*>(kptr + (int64_t)(k0 + row) * p.ks[2] + c * 8)
-                      : z;
-      }
-#pragma unroll
-      for (int it = 0; it < T::V_PER_T; ++it) {
-        int id = it * NT + tid, row = id / LV::CPR, c = id % LV::CPR;
-        u32x4 z = {0, 0, 0, 0};
-        vst[it] = (k0 + row < p.Lk)
-                      ? *reinterpret_cast<const u32x4*>(vptr + (int64_t)(k0 + row) * p.vs[2] + c * 8)
-                      : z;
-      }
-    };
-    auto store_tile = [&](int buf) {
-      unsigned char* kb_ = smem + buf * T::STAGE;
-      unsigned char* vb_ = kb_ + T::KBYTES;
-#pragma unroll
-      for (int it = 0; it < T::K_PER_T; ++it) {
-        int id = it * NT + tid, row = id / LK::CPR, c = id % LK::CPR;
-        *reinterpret_cast<u32x4*>(kb_ + row * (DQK * 2) + LK::swz_k(row, c) * 16) = kst[it];
-      }
-#pragma unroll
-      for (int it = 0; it < T::V_PER_T; ++it) {
-        int id = it * NT + tid, row = id / LV::CPR, c = id % LV::CPR;
-        *reinterpret_cast<u32x4*>(vb_ + row * (DV * 2) + LV::swz_v(row, c) * 16) = vst[it];
-      }
-    };
-    // next tile >= t that is non-empty for at least one wave, or t_end
-    auto next_tile = [&](int t) {
-      while (t < t_end && __builtin_amdgcn_readfirstlane((int)cls[t]) == 0) ++t;
-      return t;
-    };
-
-    __syncthreads();  // previous branch (if any) is done with the LDS buffers
-    int t = t_first;
-    int buf = 0;
-    if (t < t_end) {
-      load_tile(t);
-      store_tile(0);
+    for (int it = 0; it < T::K_PER_T; ++it) {
+      const int id = it * NT + tid, row = id / LK::CPR, pc = id % LK::CPR;
+      koff[it] = (unsigned)(row * (int)p.ks[2] + LK::swz_k(row, pc) * 8) * 2u;
     }
-    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < T::V_PER_T; ++it) {
+      const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
+      voff[it] = (unsigned)(row * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
+    }
+    auto load_k = [&](int t, int slot) {
+      const bf16_t* base = kptr + (int64_t)t * BN * p.ks[2];
+      if (t * BN + BN <= p.Lk) {
+#pragma unroll
+        for (int it = 0; it < T::K_PER_T; ++it)
+          dma16(base, koff[it], __builtin_amdgcn_readfirstlane(lds0 + T::K_OFF + slot * T::KBYTES + (it * NT + wave * 64) * 16));
+      } else {
+#pragma unroll
+        for (int it = 0; it < T::K_PER_T; ++it) {
+          const int id = it * NT + tid, row = id / LK::CPR, pc = id % LK::CPR;
+          const unsigned off = (unsigned)(min(row, p.Lk - 1 - t * BN) * (int)p.ks[2] + LK::swz_k(row, pc) * 8) * 2u;
+          dma16(base, off, __builtin_amdgcn_readfirstlane(lds0 + T::K_OFF + slot * T::KBYTES + (it * NT + wave * 64) * 16));
+        }
+      }
+    };
+    auto load_v = [&](int t, int slot) {
+      const bf16_t* base = vptr + (int64_t)t * BN * p.vs[2];
+      if (t * BN + BN <= p.Lk) {
+#pragma unroll
+        for (int it = 0; it < T::V_PER_T; ++it)
+          dma16(base, voff[it], __builtin_amdgcn_readfirstlane(lds0 + T::V_OFF + slot * T::VBYTES + (it * NT + wave * 64) * 16));
+      } else {
+#pragma unroll
+        for (int it = 0; it < T::V_PER_T; ++it) {
+          const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
+          const unsigned off = (unsigned)(min(row, p.Lk - 1 - t * BN) * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
+          dma16(base, off, __builtin_amdgcn_readfirstlane(lds0 + T::V_OFF + slot * T::VBYTES + (it * NT + wave * 64) * 16));
+        }
+      }
+    };
+    // tile index / this wave's class of a tile-list entry
+    auto entry_tile = [&](uint32_t e) { return (int)(__builtin_amdgcn_readfirstlane(e) & 0xffffu); };
+    auto entry_class = [&](uint32_t e) { return (int)((__builtin_amdgcn_readfirstlane(e) >> (16 + 2 * wave)) & 3u); };
 
-    while (t < t_end) {
-      const int tn = next_tile(t + 1);
-      if (tn < t_end) load_tile(tn);
+    // ---- S^T = K . Q^T for one tile: A = K fragment from LDS, B = Q fragment ---------------------------------------
+    auto qk = [&](f32x16 (&s)[KB][QB], int buf) {
+      const unsigned char* kb_ = smem + T::K_OFF + buf * T::KBYTES;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const int row = kb * 32 + r;
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kb_ + row * (DQK * 2) + LK::swz_k(row, 2 * ks + h) * 16);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb)
+            s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], s[kb][qb], 0, 0, 0);
+        }
+    };
 
-      const int tclass = (__builtin_amdgcn_readfirstlane((int)cls[t]) >> (2 * wave)) & 3;
-      if (tclass != TILE_EMPTY) {
-        const unsigned char* kb_ = smem + buf * T::STAGE;
-        const unsigned char* vb_ = kb_ + T::KBYTES;
-        const int k0 = t * BN;
-
-        // ---- S^T = K . Q^T --------------------------------------------------------------------------------------
-        f32x16 s[KB][QB];
+    // ---- score modifications and element mask of one tile; afterwards s is in log2 units when kMod ----------------
+    // Register i of block (kb, qb) is key k0 + 32*kb + 8*(i/4) + 4*h + i%4 against query qrow[qb].
+    auto score_mods = [&](f32x16 (&s)[KB][QB], int t) {
+      const int k0 = t * BN;
+      if constexpr (kMod) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-          for (int qb = 0; qb < QB; ++qb)
+          for (int qb = 0; qb < QB; ++qb) {
+            const int kbase = k0 + 32 * kb + 4 * h;
+            const float rel0 = (float)(kbase - qrow[qb]);
+            float bv[16];
+            if constexpr (kBias) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
+              for (int i = 0; i < 16; ++i) bv[i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+              for (int nb = 0; nb < 2; ++nb) {
+                if (p.bias[nb] == nullptr) continue;
+                const bf16_t* bp = p.bias[nb] + (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] +
+                                   (int64_t)head * p.bs[nb][1] + (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            const int row = kb * 32 + r;
-            bf16x8 kf = *reinterpret_cast<const bf16x8*>(kb_ + row * (DQK * 2) + LK::swz_k(row, 2 * ks + h) * 16);
+                for (int g = 0; g < 4; ++g) {
+                  const int key = kbase + 8 * g;
+                  if (p.bias_vec[nb] && key + 3 < p.Lk) {
+                    bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bp + key);
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], s[kb][qb], 0, 0, 0);
-          }
-
-        // ---- score modifications; afterwards s is in log2 units when kMod -----------------------------------------
-        // Register i of block (kb, qb) is key k0 + 32*kb + 8*(i/4) + 4*h + i%4 against query qrow[qb].
-        if constexpr (kMod) {
+                    for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                  } else {
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) {
-              const int kbase = k0 + 32 * kb + 4 * h;
-              const float rel0 = (float)(kbase - qrow[qb]);
-              float bv[16];
-              if constexpr (kBias) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) bv[i] = 0.f;
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) {
-                  if (p.bias[nb] == nullptr) continue;
-                  const bf16_t* bp = p.bias[nb] + (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] +
-                                     (int64_t)head * p.bs[nb][1] +
-                                     (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
-#pragma unroll
-                  for (int g = 0; g < 4; ++g) {
-                    const int key = kbase + 8 * g;
-                    if (p.bias_vec[nb] && key + 3 < p.Lk) {
-                      bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bp + key);
-#pragma unroll
-                      for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
-                    } else {
-#pragma unroll
-                      for (int e = 0; e < 4; ++e)
-                        if (key + e < p.Lk) bv[4 * g + e] += (float)bp[(int64_t)(key + e) * p.bs[nb][3]];
-                    }
+                    for (int e = 0; e < 4; ++e)
+                      if (key + e < p.Lk) bv[4 * g + e] += (float)bp[(int64_t)(key + e) * p.bs[nb][3]];
                   }
                 }
               }
-#pragma unroll
-              for (int i = 0; i < 16; ++i) {
-                float x = s[kb][qb][i];
-                float tl2;
-                if constexpr (kSoftcap) {
-                  float e = fast_exp2(x * cap_k1);
-                  float rc = fast_rcp(e + 1.0f);
-                  tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
-                } else {
-                  tl2 = x * p.scale_log2;
-                }
-                if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
-                if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], 1.4426950408889634f, tl2);
-                s[kb][qb][i] = tl2;
-              }
             }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const float x = s[kb][qb][i];
+              float tl2;
+              if constexpr (kSoftcap) {
+                const float e = fast_exp2(x * cap_k1);
+                const float rc = fast_rcp(e + 1.0f);
+                tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
+              } else {
+                tl2 = x * p.scale_log2;
+              }
+              if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
+              if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
+              s[kb][qb][i] = tl2;
+            }
+          }
+      }
+    };
+    // Element mask of a tile that is not FULL for this wave: attend iff
+    // key < Lk && ((dmin <= key - q <= dmax) || key < pfx) [&& same document]; with key = kbase + off and off a
+    // compile-time constant per register, every test compares off with a per-lane bound (branch-free).
+    // A tile that is empty for this wave (but not for the workgroup) takes the same path and loses every score.
+    auto apply_mask = [&](f32x16 (&s)[KB][QB], int t) {
+      const int k0 = t * BN;
+      {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const int kbase = k0 + 32 * kb + 4 * h;
+          const int t_len = p.Lk - kbase;   // off < t_len   <=> key < Lk
+          const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
+          int64_t kdoc[16];
+          if constexpr (kDoc) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
+          }
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            const int rel = kbase - qrow[qb];
+            const int t_hi = p.dmax - rel;  // off <= t_hi  <=> key - q <= dmax
+            const int t_lo = p.dmin - rel;  // off >= t_lo  <=> key - q >= dmin
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int off = 8 * (i / 4) + (i % 4);
+              bool ok = (off < t_len) & (((off <= t_hi) & (off >= t_lo)) | (off < t_pfx));
+              if constexpr (kDoc) ok = ok & (kdoc[i] == qdoc[qb]);
+              s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
+            }
+          }
         }
-
-        // ---- element mask on partial tiles ------------------------------------------------------------------------
-        if (tclass == TILE_PARTIAL) {
+      }
+    };
+    auto dump_attended = [&](const f32x16 (&s)[KB][QB], int t) {
+      const int k0 = t * BN;
+      if constexpr (kDump) {
+        if (br == 0) {
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            int64_t kdoc[16];
-            if constexpr (kDoc) {
-#pragma unroll
-              for (int i = 0; i < 16; ++i) {
-                int key = k0 + 32 * kb + 8 * (i / 4) + 4 * h + (i % 4);
-                kdoc[i] = key < p.Lk ? p.doc_ids[(int64_t)batch * p.doc_stride + key] : 0;
-              }
-            }
+          for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
                 const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * h + (i % 4);
-                bool ok = key < p.Lk && attend_positional(p.mask_kind, qrow[qb], key, p.window, p.prefix);
-                if constexpr (kDoc) ok = ok && (kdoc[i] == qdoc[qb]);
-                s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
+                if (qrow[qb] < p.Lq && key < p.Lk && s[kb][qb][i] != -INFINITY)
+                  p.dump[(((int64_t)batch * p.Hq + head) * p.Lq + qrow[qb]) * p.Lk + key] = 1;
               }
-          }
         }
+      }
+    };
 
-        if constexpr (kDump) {
-          if (br == 0) {
+    // ---- running maximum: row maxima of one tile; the accumulators are rescaled when a maximum grew by more than kTau
+    auto row_max = [&](const f32x16 (&s)[KB][QB], float (&mx)[QB]) {
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+      for (int qb = 0; qb < QB; ++qb) {
+        float m = -INFINITY;
 #pragma unroll
-              for (int qb = 0; qb < QB; ++qb)
+        for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                  const int key = k0 + 32 * kb + 8 * (i / 4) + 4 * h + (i % 4);
-                  if (qrow[qb] < p.Lq && key < p.Lk && s[kb][qb][i] != -INFINITY)
-                    p.dump[(((int64_t)batch * p.Hq + head) * p.Lq + qrow[qb]) * p.Lk + key] = 1;
-                }
-          }
-        }
-
-        // ---- online softmax ---------------------------------------------------------------------------------------
-        const float c2 = kMod ? 1.0f : p.scale_log2;  // s * c2 is the logit in log2 units
-        bf16x8 pf[QB][2 * KB];
+          for (int i = 0; i < 16; ++i) m = __builtin_fmaxf(m, s[kb][qb][i]);
+        mx[qb] = xhalf_max(m);
+      }
+    };
+    auto rescale_if_grown = [&](const float (&mx)[QB]) {
+      bool grow = false;
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+        grow = grow | ((mx[qb] - m_run[qb]) * c2 > kTau);  // m_run = -inf before the first tile: always true
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-          float mx = -INFINITY;
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) mx = __builtin_fmaxf(mx, s[kb][qb][i]);
-          mx = xhalf_max(mx);
-          const float m_new = __builtin_fmaxf(m_run[qb], mx);
+          const float m_new = __builtin_fmaxf(m_run[qb], mx[qb]);
           const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // row fully masked so far
           const float alpha = fast_exp2((m_run[qb] - m_use) * c2);
-          const float mc = m_use * c2;
           m_run[qb] = m_new;
-          float rs = 0.f;
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb) {
-            float pv[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
-              rs += pv[i];
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-              for (int e = 0; e < 8; ++e) pf[qb][2 * kb + j][e] = (bf16_t)pv[8 * j + e];
-          }
-          l_run[qb] = l_run[qb] * alpha + rs;
+          l_run[qb] *= alpha;
 #pragma unroll
           for (int dvb = 0; dvb < DVB; ++dvb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[dvb][qb][i] *= alpha;
         }
-
-        // ---- O^T += V^T . P^T ----------------------------------------------------------------------------------------
-        // A operand slot j of lane (r, h) for 16-key chunk c is key 16c + 8*(j/4) + 4h + j%4, matching pf above.
-#pragma unroll
-        for (int c = 0; c < 2 * KB; ++c)
-#pragma unroll
-          for (int dvb = 0; dvb < DVB; ++dvb) {
-            bf16x8 vf;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              // transposing read: within each 16-lane group, lane i supplies row (key) i/4, 4 columns at 4*(i%4),
-              // and receives column i of the 4 rows.
-              const int i16 = lane % 16, g = (lane / 16) % 2;
-              const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
-              const int col = dvb * 32 + g * 16 + 4 * (i16 % 4);
-              const unsigned char* ap = vb_ + row * (DV * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
-              typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-              s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
-              bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
-            }
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-              oacc[dvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][c], oacc[dvb][qb], 0, 0, 0);
-          }
       }
+    };
 
-      if (tn < t_end) store_tile(buf ^ 1);
+    // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB]) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          float pv[16];
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
+            rs += pv[i];
+          }
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[qb][2 * kb + j][e] = (bf16_t)pv[8 * j + e];
+        }
+        l_run[qb] += rs;
+      }
+    };
+
+    // ---- O^T += V^T . P^T: A = V fragment through the transposing LDS read, B = P ---------------------------------------
+    // A operand slot j of lane (r, h) for 16-key chunk c is key 16c + 8*(j/4) + 4h + j%4, the key order of pf.
+    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf) {
+      const unsigned char* vb_ = smem + T::V_OFF + buf * T::VBYTES;
+#pragma unroll
+      for (int c = 0; c < 2 * KB; ++c)
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          bf16x8 vf;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            // within each 16-lane group, lane i supplies row (key) i/4, 4 columns at 4*(i%4), and receives column i
+            // of the 4 rows
+            const int i16 = lane % 16, g = (lane / 16) % 2;
+            const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
+            const int col = dvb * 32 + g * 16 + 4 * (i16 % 4);
+            const unsigned char* ap = vb_ + row * (DV * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
+            typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+            const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
+            const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
+          }
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb)
+            oacc[dvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][c], oacc[dvb][qb], 0, 0, 0);
+        }
+    };
+
+    __syncthreads();  // the previous branch (if any) is done with the LDS buffers
+    if (n_list > 0) {
+      constexpr int NS = T::NS;
+      constexpr int LPS = T::K_PER_T + T::V_PER_T;  // transfers per thread per step
+      // ent[j] = tile-list entry of list position pos + j (the last entry again past the end of the list).  Entries are
+      // read from LDS NS steps before they are needed, so the read latency never shows.
+      int pos = 0;
+      uint32_t ent[NS + 1];
+#pragma unroll
+      for (int j = 0; j <= NS; ++j) ent[j] = tlist[min(j, n_list - 1)];
+      // prologue: K of the first NS tiles and V of the first NS - 1 go to their ring slots; raw S of the first tile
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        if (j < n_list) load_k(entry_tile(ent[j]), j);
+#pragma unroll
+      for (int j = 0; j + 1 < NS; ++j)
+        if (j < n_list) load_v(entry_tile(ent[j]), j);
+      dma_wait<0>();
       __syncthreads();
-      t = tn;
-      buf ^= 1;
+      f32x16 s_a[KB][QB], s_b[KB][QB];
+      qk(s_a, 0);
+      score_mods(s_a, entry_tile(ent[0]));
+      __syncthreads();  // K slot 0 may be overwritten from here on
+
+      // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
+      // maxima, and the (rare) rescale.
+      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e) {
+        const int t = entry_tile(e);
+        if (entry_class(e) != TILE_FULL) apply_mask(sc, t);
+        dump_attended(sc, t);
+        float mx[QB];
+        row_max(sc, mx);
+        rescale_if_grown(mx);
+      };
+      // One pipeline step for list position pos with pos % NS == slot: `sc` holds the (score-modified, unmasked)
+      // scores of the current tile on entry and `sn` receives those of the next one.  K of list position j lives in K
+      // slot j % NS, V likewise.  The body after `settle` is one straight-line block in which the scheduler
+      // interleaves both MFMA groups with the exponentials.  The loop unrolls NS steps so that every slot index is a
+      // constant and the two score buffers swap roles without copies.
+      auto step = [&](f32x16 (&sc)[KB][QB], f32x16 (&sn)[KB][QB], auto slot_tag) {
+        constexpr int slot = decltype(slot_tag)::value;
+        // K slot `slot` held this tile's K and V slot `slot - 1` the previous tile's V: both were last read before the
+        // barrier that ended the previous step
+        const bool steady = pos + NS < n_list;
+        if (steady) load_k(entry_tile(ent[NS]), slot);
+        if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
+        settle(sc, ent[0]);
+        bf16x8 pf[QB][2 * KB];
+        qk(sn, (slot + 1) % NS);
+        softmax_p(sc, pf);
+        pv_mma(pf, slot);
+        score_mods(sn, entry_tile(ent[1]));
+        {
+          constexpr int NA = KS * KB * QB, NB = 2 * KB * DVB * QB;
+          constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp + add per score, one pack per two
+          sched_tile_step<NA, NB, (n_exp * 7 / 2 + NA - 1) / NA, 0>();
+        }
+        // the next step reads K and V transfers issued NS - 2 steps ago: later ones may stay in flight
+        if (steady) dma_wait<(NS - 2) * LPS>(); else dma_wait<0>();
+        __syncthreads();
+        ++pos;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) ent[j] = ent[j + 1];
+        ent[NS] = tlist[min(pos + NS, n_list - 1)];
+      };
+      int last_slot = 0;  // ring slot of the final tile; its scores are in s_a when the slot is even
+      bool more = true;
+      while (more) {
+        more = static_while<0, NS>([&](auto idx) {
+          constexpr int slot = decltype(idx)::value;
+          if (!(pos + 1 < n_list)) {
+            last_slot = slot;
+            return false;
+          }
+          if constexpr (slot % 2 == 0) step(s_a, s_b, idx); else step(s_b, s_a, idx);
+          return true;
+        });
+      }
+      // last tile: nothing left to prefetch
+      static_while<0, NS>([&](auto idx) {
+        constexpr int slot = decltype(idx)::value;
+        if (last_slot != slot) return true;
+        bf16x8 pf[QB][2 * KB];
+        if constexpr (slot % 2 == 0) {
+          settle(s_a, ent[0]);
+          softmax_p(s_a, pf);
+        } else {
+          settle(s_b, ent[0]);
+          softmax_p(s_b, pf);
+        }
+        pv_mma(pf, slot);
+        return false;
+      });
     }
 
     // ---- normalise this branch ---------------------------------------------------------------------------------
@@ -607,7 +808,7 @@ __global__ __launch_bounds__(T::NT) void fwd_kernel(const KParams p) {
           bf16x4 g4 = *reinterpret_cast<const bf16x4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            float sg = fast_rcp(1.0f + fast_exp2(-1.4426950408889634f * (float)g4[e]));
+            float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
             o4[e] = (bf16_t)(oacc[dvb][qb][4 * g + e] * sg);
           }
         } else {

@@ -26,6 +26,7 @@ HIPCC_FLAGS = [
     "-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-inline-asm", "-Wno-ignored-optimization-argument",
+    "-Wno-pass-failed", "-Rpass-analysis=kernel-resource-usage",
     f"-I{INCLUDE}", f"-I{CSRC}",
 ]
 
@@ -62,13 +63,33 @@ def _sources_digest() -> str:
     return h.hexdigest()[:16]
 
 
+def _resource_usage(log: str) -> list[str]:
+    """'kernel: VGPRs n, scratch n bytes/lane, occupancy n' lines from hipcc's kernel-resource-usage remarks."""
+    out, cur = [], {}
+    for line in log.splitlines():
+        m = re.search(r"remark:\s+(Function Name|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|Occupancy \[waves/SIMD\]): (\S+)", line)
+        if not m:
+            continue
+        key, val = m.group(1), m.group(2)
+        if key == "Function Name":
+            cur = {"name": val}
+        cur[key] = val
+        if key.startswith("Occupancy"):
+            out.append(f"{cur.get('name')}: VGPRs {cur.get('VGPRs')} AGPRs {cur.get('AGPRs')} "
+                       f"scratch {cur.get('ScratchSize [bytes/lane]')} B/lane occupancy {val}")
+    return out
+
+
 def _compile(args: tuple[list[str], Path]) -> str:
     cmd, out = args
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
+        log = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
         raise RuntimeError(f"hipcc failed for {out.name}:\n{' '.join(cmd)}\n{log}")
-    return log
+    usage = _resource_usage(r.stdout)
+    if usage:
+        out.with_suffix(".resources.txt").write_text("\n".join(usage) + "\n")
+    return "\n".join(usage)
 
 
 def build(force: bool = True, jobs: int | None = None, verbose: bool = False) -> Path:

@@ -111,12 +111,15 @@ __device__ __forceinline__ float xhalf_sum(float x) {
 // gbase + voff[l] and writes LDS bytes [lds_base + 16 l, +16).  gbase and lds_base are wave-uniform.  Written as asm
 // so that the compiler does not order later LDS reads of *other* buffers behind it with a vmcnt(0) wait; completion
 // is awaited explicitly (dma_wait) before the barrier that publishes the data.
-__device__ __forceinline__ void dma16(const void* gbase, unsigned voff, unsigned lds_base_uniform) {
-  // readfirstlane pins the (already uniform) base to scalar registers whatever the compiler's divergence analysis says
-  const uint64_t b = reinterpret_cast<uint64_t>(gbase);
-  // (the builtin returns int: go through uint32_t so that the low half is not sign-extended over the high half)
-  const uint64_t gbase_uniform = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
-                                 ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+// Pins an (already wave-uniform) pointer to scalar registers whatever the compiler's divergence analysis concluded.
+// readfirstlane returns int: each half goes through uint32_t so the low half is not sign-extended over the high one.
+__device__ __forceinline__ uint64_t uniform_ptr(const void* ptr) {
+  const uint64_t b = reinterpret_cast<uint64_t>(ptr);
+  return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
+         ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+}
+__device__ __forceinline__ void dma16(uint64_t gbase_uniform, unsigned voff, unsigned lds_base) {
+  const unsigned lds_base_uniform = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_base);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(gbase_uniform), "v"(voff),
                "s"(lds_base_uniform)
                : "m0");
@@ -197,6 +200,10 @@ struct TileLayout {
 // Scheduling pipeline for the straight-line tile step (see fwd_kernel): instruction classes of
 // __builtin_amdgcn_sched_group_barrier.
 enum : int { SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400 };
+// Every lambda of the kernel must be inlined: an outlined one would take its captures (the accumulators) by address
+// through scratch memory.
+#define FL_INLINE __attribute__((always_inline))
+
 #ifndef FL_SCHED
 #define FL_SCHED 1
 #endif
@@ -414,7 +421,9 @@ void fwd_kernel(const KParams p) {
     // inverses).  The global address is a per-tile scalar base plus a per-lane byte offset that does not change from
     // tile to tile; only the ragged last tile recomputes it, repeating the last key for rows past the end (those
     // keys are masked, p = 0).
-    const unsigned lds0 = (unsigned)(uintptr_t)smem;  // LDS byte address of the dynamic segment
+    // LDS byte addresses this wave's transfers of slot 0, first transfer, land at
+    const unsigned lds_k = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::K_OFF + wave * 1024);
+    const unsigned lds_v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::V_OFF + wave * 1024);
     unsigned koff[T::K_PER_T], voff[T::V_PER_T];
 #pragma unroll
     for (int it = 0; it < T::K_PER_T; ++it) {
@@ -426,42 +435,42 @@ void fwd_kernel(const KParams p) {
       const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
       voff[it] = (unsigned)(row * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
     }
-    auto load_k = [&](int t, int slot) {
-      const bf16_t* base = kptr + (int64_t)t * BN * p.ks[2];
+    auto load_k = [&](int t, int slot) FL_INLINE  {
+      const uint64_t base = uniform_ptr(kptr + (int64_t)t * BN * p.ks[2]);
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
         for (int it = 0; it < T::K_PER_T; ++it)
-          dma16(base, koff[it], __builtin_amdgcn_readfirstlane(lds0 + T::K_OFF + slot * T::KBYTES + (it * NT + wave * 64) * 16));
+          dma16(base, koff[it], lds_k + slot * T::KBYTES + it * NT * 16);
       } else {
 #pragma unroll
         for (int it = 0; it < T::K_PER_T; ++it) {
           const int id = it * NT + tid, row = id / LK::CPR, pc = id % LK::CPR;
           const unsigned off = (unsigned)(min(row, p.Lk - 1 - t * BN) * (int)p.ks[2] + LK::swz_k(row, pc) * 8) * 2u;
-          dma16(base, off, __builtin_amdgcn_readfirstlane(lds0 + T::K_OFF + slot * T::KBYTES + (it * NT + wave * 64) * 16));
+          dma16(base, off, lds_k + slot * T::KBYTES + it * NT * 16);
         }
       }
     };
-    auto load_v = [&](int t, int slot) {
-      const bf16_t* base = vptr + (int64_t)t * BN * p.vs[2];
+    auto load_v = [&](int t, int slot) FL_INLINE  {
+      const uint64_t base = uniform_ptr(vptr + (int64_t)t * BN * p.vs[2]);
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
         for (int it = 0; it < T::V_PER_T; ++it)
-          dma16(base, voff[it], __builtin_amdgcn_readfirstlane(lds0 + T::V_OFF + slot * T::VBYTES + (it * NT + wave * 64) * 16));
+          dma16(base, voff[it], lds_v + slot * T::VBYTES + it * NT * 16);
       } else {
 #pragma unroll
         for (int it = 0; it < T::V_PER_T; ++it) {
           const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
           const unsigned off = (unsigned)(min(row, p.Lk - 1 - t * BN) * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
-          dma16(base, off, __builtin_amdgcn_readfirstlane(lds0 + T::V_OFF + slot * T::VBYTES + (it * NT + wave * 64) * 16));
+          dma16(base, off, lds_v + slot * T::VBYTES + it * NT * 16);
         }
       }
     };
     // tile index / this wave's class of a tile-list entry
-    auto entry_tile = [&](uint32_t e) { return (int)(__builtin_amdgcn_readfirstlane(e) & 0xffffu); };
-    auto entry_class = [&](uint32_t e) { return (int)((__builtin_amdgcn_readfirstlane(e) >> (16 + 2 * wave)) & 3u); };
+    auto entry_tile = [&](uint32_t e) FL_INLINE  { return (int)(__builtin_amdgcn_readfirstlane(e) & 0xffffu); };
+    auto entry_class = [&](uint32_t e) FL_INLINE  { return (int)((__builtin_amdgcn_readfirstlane(e) >> (16 + 2 * wave)) & 3u); };
 
     // ---- S^T = K . Q^T for one tile: A = K fragment from LDS, B = Q fragment ---------------------------------------
-    auto qk = [&](f32x16 (&s)[KB][QB], int buf) {
+    auto qk = [&](f32x16 (&s)[KB][QB], int buf) FL_INLINE {
       const unsigned char* kb_ = smem + T::K_OFF + buf * T::KBYTES;
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
@@ -483,7 +492,7 @@ void fwd_kernel(const KParams p) {
 
     // ---- score modifications and element mask of one tile; afterwards s is in log2 units when kMod ----------------
     // Register i of block (kb, qb) is key k0 + 32*kb + 8*(i/4) + 4*h + i%4 against query qrow[qb].
-    auto score_mods = [&](f32x16 (&s)[KB][QB], int t) {
+    auto score_mods = [&](f32x16 (&s)[KB][QB], int t) FL_INLINE {
       const int k0 = t * BN;
       if constexpr (kMod) {
 #pragma unroll
@@ -538,7 +547,7 @@ void fwd_kernel(const KParams p) {
     // key < Lk && ((dmin <= key - q <= dmax) || key < pfx) [&& same document]; with key = kbase + off and off a
     // compile-time constant per register, every test compares off with a per-lane bound (branch-free).
     // A tile that is empty for this wave (but not for the workgroup) takes the same path and loses every score.
-    auto apply_mask = [&](f32x16 (&s)[KB][QB], int t) {
+    auto apply_mask = [&](f32x16 (&s)[KB][QB], int t) FL_INLINE {
       const int k0 = t * BN;
       {
 #pragma unroll
@@ -568,7 +577,7 @@ void fwd_kernel(const KParams p) {
         }
       }
     };
-    auto dump_attended = [&](const f32x16 (&s)[KB][QB], int t) {
+    auto dump_attended = [&](const f32x16 (&s)[KB][QB], int t) FL_INLINE {
       const int k0 = t * BN;
       if constexpr (kDump) {
         if (br == 0) {
@@ -587,7 +596,7 @@ void fwd_kernel(const KParams p) {
     };
 
     // ---- running maximum: row maxima of one tile; the accumulators are rescaled when a maximum grew by more than kTau
-    auto row_max = [&](const f32x16 (&s)[KB][QB], float (&mx)[QB]) {
+    auto row_max = [&](const f32x16 (&s)[KB][QB], float (&mx)[QB]) FL_INLINE {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         float m = -INFINITY;
@@ -598,7 +607,7 @@ void fwd_kernel(const KParams p) {
         mx[qb] = xhalf_max(m);
       }
     };
-    auto rescale_if_grown = [&](const float (&mx)[QB]) {
+    auto rescale_if_grown = [&](const float (&mx)[QB]) FL_INLINE {
       bool grow = false;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
@@ -620,7 +629,9 @@ void fwd_kernel(const KParams p) {
     };
 
     // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
-    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB]) {
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB]) FL_INLINE {
+      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+      const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
@@ -629,14 +640,19 @@ void fwd_kernel(const KParams p) {
         for (int kb = 0; kb < KB; ++kb) {
           float pv[16];
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
-            rs += pv[i];
-          }
+          for (int i = 0; i < 16; ++i) pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < 2; ++j) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[qb][2 * kb + j][e] = (bf16_t)pv[8 * j + e];
+            // the row sum adds up the rounded weights, the very numbers the second product uses (v_dot2 with ones:
+            // two weights per instruction)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              const bf16x2 pr = {pf[qb][2 * kb + j][e], pf[qb][2 * kb + j][e + 1]};
+              rs = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, rs, false);
+            }
+          }
         }
         l_run[qb] += rs;
       }
@@ -644,7 +660,7 @@ void fwd_kernel(const KParams p) {
 
     // ---- O^T += V^T . P^T: A = V fragment through the transposing LDS read, B = P ---------------------------------------
     // A operand slot j of lane (r, h) for 16-key chunk c is key 16c + 8*(j/4) + 4h + j%4, the key order of pf.
-    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf) {
+    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf) FL_INLINE {
       const unsigned char* vb_ = smem + T::V_OFF + buf * T::VBYTES;
 #pragma unroll
       for (int c = 0; c < 2 * KB; ++c)
@@ -697,7 +713,7 @@ void fwd_kernel(const KParams p) {
 
       // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
       // maxima, and the (rare) rescale.
-      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e) {
+      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e) FL_INLINE {
         const int t = entry_tile(e);
         if (entry_class(e) != TILE_FULL) apply_mask(sc, t);
         dump_attended(sc, t);
@@ -710,7 +726,7 @@ void fwd_kernel(const KParams p) {
       // slot j % NS, V likewise.  The body after `settle` is one straight-line block in which the scheduler
       // interleaves both MFMA groups with the exponentials.  The loop unrolls NS steps so that every slot index is a
       // constant and the two score buffers swap roles without copies.
-      auto step = [&](f32x16 (&sc)[KB][QB], f32x16 (&sn)[KB][QB], auto slot_tag) {
+      auto step = [&](f32x16 (&sc)[KB][QB], f32x16 (&sn)[KB][QB], auto slot_tag) FL_INLINE {
         constexpr int slot = decltype(slot_tag)::value;
         // K slot `slot` held this tile's K and V slot `slot - 1` the previous tile's V: both were last read before the
         // barrier that ended the previous step
@@ -739,7 +755,7 @@ void fwd_kernel(const KParams p) {
       int last_slot = 0;  // ring slot of the final tile; its scores are in s_a when the slot is even
       bool more = true;
       while (more) {
-        more = static_while<0, NS>([&](auto idx) {
+        more = static_while<0, NS>([&](auto idx) FL_INLINE  {
           constexpr int slot = decltype(idx)::value;
           if (!(pos + 1 < n_list)) {
             last_slot = slot;
@@ -750,7 +766,7 @@ void fwd_kernel(const KParams p) {
         });
       }
       // last tile: nothing left to prefetch
-      static_while<0, NS>([&](auto idx) {
+      static_while<0, NS>([&](auto idx) FL_INLINE  {
         constexpr int slot = decltype(idx)::value;
         if (last_slot != slot) return true;
         bf16x8 pf[QB][2 * KB];

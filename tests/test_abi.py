@@ -124,8 +124,12 @@ def test_workspace_size_for_document_masks(lib):
 
 
 def test_too_many_keys_is_an_error_not_a_fault(lib):
-    p = good_params(B=1, Hq=1, Hkv=1, L=64 * 4096 + 64, D=64)
+    # the tile list (4 bytes per key tile) must fit in LDS next to the K/V ring
+    p = good_params(B=1, Hq=1, Hkv=1, L=1 << 26, D=64)
     assert rc(lib, p) == -2 and "maximum" in _ffi.last_error()
+    p = good_params(B=1, Hq=1, Hkv=1, L=1 << 20, D=64)
+    assert rc(lib, p) == 0, _ffi.last_error()
+    assert _ffi.plan(p)["lds_bytes"] <= 160 * 1024
 
 
 def test_front_end_refuses_cpu_and_fp32_tensors(lib):

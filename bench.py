@@ -33,12 +33,17 @@ def parse_args():
     return ap.parse_args()
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 256 MiB copy's readings);
+# commands and raw values: profiles/fwd_kernel_d128_cfg1_counters.md
+MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 269.1e6, "cfg1/sliding_window": 308.4e6}
+
+
 def event_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
 def time_launches(fn, iters: int, warmup: int = 3):
-    """Mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
+    """Trimmed mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
     current stream (the stream the kernels are launched on)."""
     for _ in range(warmup):
         fn()
@@ -48,8 +53,9 @@ def time_launches(fn, iters: int, warmup: int = 3):
         fn()
         b.record()
     torch.cuda.synchronize()
-    ts = [a.elapsed_time(b) for a, b in pairs]
-    return statistics.fmean(ts), statistics.median(ts)
+    ts = sorted(a.elapsed_time(b) for a, b in pairs)
+    keep = ts[: max(1, int(len(ts) * 0.9))]  # drop the slowest tenth: one-off host hiccups land inside an event pair
+    return statistics.fmean(keep), statistics.median(ts)
 
 
 def cpu_baseline(threads_hint: int = 0) -> dict:
@@ -142,7 +148,8 @@ def main():
     dv = variants[dom.name]
     roofline = {"bound": "mfma", "kernel": f"fl::fwd_kernel ({dom.name})", "achieved": dv["tflops"],
                 "peak": W.PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dv["tflops"] / W.PEAK_BF16_TFLOPS,
-                "traffic": None, "launch_ms": dv["ms"], "flops_per_launch": dom.flops}
+                "traffic": MEASURED_HBM_BYTES.get(dom.name), "traffic_unit": "bytes/launch (rocprofv3, see profiles/)",
+                "launch_ms": dv["ms"], "flops_per_launch": dom.flops}
 
     others = {}
     if not args.no_other_configs:

@@ -292,14 +292,23 @@ void fwd_kernel(const KParams p) {
 
   // ---- workgroup -> (batch, head, query tile).  Consecutive workgroup ids land on different XCDs, so ids are
   // regrouped to give every XCD a contiguous run of (batch, head) pairs: their K/V stay in that XCD's L2.
-  // Within a run the query tiles are visited from the last (longest under a causal mask) to the first.
-  int wg = blockIdx.x;
+  // Within a run, heads are taken two at a time and their query tiles dealt from the last (longest under a causal
+  // mask) to the first, alternating between the two heads: the workgroups still running when the grid drains are
+  // the short ones, and an XCD works on the K/V of two heads at a time.
+  int bh, qt;
   {
-    const int total = gridDim.x;
-    if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+    const int nbh = p.B * p.Hq, nq = p.n_qtiles;
+    int i = blockIdx.x, run = nbh, base = 0;
+    if (nbh % 8 == 0) {
+      run = nbh / 8;
+      base = (i % 8) * run;
+      i /= 8;
+    }
+    const int g = i / (2 * nq), rem = i % (2 * nq);
+    const int gg = min(2, run - 2 * g);
+    qt = nq - 1 - rem / gg;
+    bh = base + 2 * g + rem % gg;
   }
-  const int qt = p.n_qtiles - 1 - (wg % p.n_qtiles);
-  const int bh = wg / p.n_qtiles;
   const int head = bh % p.Hq, batch = bh / p.Hq;
   const int kvh = head / p.group;
 
@@ -735,6 +744,10 @@ void fwd_kernel(const KParams p) {
         if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
         settle(sc, ent[0]);
         bf16x8 pf[QB][2 * KB];
+        // Raised issue priority while this wave has matrix work: of the two waves sharing a SIMD, the one that is in
+        // its MFMA phase wins the issue port, which drives the pair into opposite phases (one on the matrix pipe while
+        // the other does vector work) instead of both stalling on each other.
+        __builtin_amdgcn_s_setprio(3);
         qk(sn, (slot + 1) % NS);
         softmax_p(sc, pf);
         pv_mma(pf, slot);
@@ -744,6 +757,7 @@ void fwd_kernel(const KParams p) {
           constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp + add per score, one pack per two
           sched_tile_step<NA, NB, (n_exp * 7 / 2 + NA - 1) / NA, 0>();
         }
+        __builtin_amdgcn_s_setprio(0);
         // the next step reads K and V transfers issued NS - 2 steps ago: later ones may stay in flight
         if (steady) dma_wait<(NS - 2) * LPS>(); else dma_wait<0>();
         __syncthreads();

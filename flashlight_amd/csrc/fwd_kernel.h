@@ -70,6 +70,8 @@ struct KParams {
   int64_t bs[2][4];
   int32_t bdiv[2];
   int32_t bias_vec[2];  // rows of this bias may be read 4 keys (8 bytes) at a time
+  int32_t bias_lds;     // index of the bias operand staged through LDS (16-byte aligned rows, Lk % 8 == 0), or -1
+  int32_t bias_row;     // index of a row-broadcast bias operand staged through LDS as single rows, or -1
   const bf16_t* gate;
   int64_t gs[3];
   float lambda;
@@ -197,6 +199,15 @@ struct TileLayout {
   }
 };
 
+// Staged bias tile of one wave: [RW rows][BN keys] bf16, 16-byte chunks XOR-swizzled with the row so that the 8-byte
+// reads of 32 consecutive rows at one key offset spread over the banks.
+template <int BN>
+struct BiasLayout {
+  static constexpr int CPR = BN / 8;                         // chunks per row
+  static constexpr int RPW = (CPR >= 16) ? 1 : (16 / CPR);   // rows per 256-byte bank window
+  __device__ static __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row / RPW) & (CPR - 1)); }
+};
+
 // Scheduling pipeline for the straight-line tile step (see fwd_kernel): instruction classes of
 // __builtin_amdgcn_sched_group_barrier.
 enum : int { SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400 };
@@ -254,9 +265,24 @@ struct FwdTraits {
   static_assert(RW % 32 == 0 && BN % 32 == 0 && DQK % 16 == 0 && DV % 32 == 0, "MFMA 32x32x16 blocking");
   static_assert(NW <= 8, "tile classes are packed two bits per wave into 16 bits");
   // waves per SIMD the register budget is sized for
+#ifdef FL_WPE
+  static constexpr int WAVES_PER_EU = FL_WPE;
+#else
   static constexpr int WAVES_PER_EU = (RW == 32) ? 2 : 1;
-  // LDS: K tiles [NS], V tiles [NS], 16 bytes of counters, then the tile list (4 bytes per key tile, sized at launch)
-  static constexpr int K_OFF = 0, V_OFF = NS * KBYTES, META_OFF = NS * (KBYTES + VBYTES), LIST_OFF = META_OFF + 16;
+#endif
+  // One dense bias operand is staged through LDS like K and V: per ring slot a [BM][BN] bf16 tile, every wave
+  // transferring (and later reading) only its own RW rows.
+  static constexpr int BBYTES = (FEAT & F_BIAS) ? BM * BN * 2 : 0;
+  static constexpr int B_PER_T = (FEAT & F_BIAS) ? RW * BN / 8 / 64 : 0;  // 16-byte transfers per lane per tile
+  static_assert(!(FEAT & F_BIAS) || ((RW * BN / 8) % 64 == 0 && NS == 2), "staged bias: whole transfers, ring of two");
+  // LDS: K tiles [NS], V tiles [NS], bias tiles [NS], 16 bytes of counters, then the tile list (4 bytes per key tile,
+  // sized at launch)
+  // A second, row-broadcast operand (query stride 0, e.g. a key-padding bias) is staged as one row of BN keys per wave
+  // and slot; the transfer is a whole 1 KiB wave transfer whose lanes repeat the row.
+  static constexpr int RBYTES = (FEAT & F_BIAS) ? NW * 1024 : 0;
+  static constexpr int R_PER_T = (FEAT & F_BIAS) ? 1 : 0;
+  static constexpr int K_OFF = 0, V_OFF = NS * KBYTES, B_OFF = NS * (KBYTES + VBYTES), R_OFF = B_OFF + NS * BBYTES,
+                       META_OFF = R_OFF + NS * RBYTES, LIST_OFF = META_OFF + 16;
   static constexpr int LDS_FIXED_BYTES = LIST_OFF;
 };
 
@@ -389,10 +415,31 @@ void fwd_kernel(const KParams p) {
     for (int qb = 0; qb < QB; ++qb)
       qdoc[qb] = p.doc_ids[(int64_t)batch * p.doc_stride + min(qrow[qb], p.Lq - 1)];
   }
-  const float c2 = kMod ? 1.0f : p.scale_log2;  // s * c2 is the logit in log2 units
+  // With dense biases as the only score modification the modified scores stay in natural units (s = qk * scale + bias)
+  // and the factor log2(e) rides in the exponential's multiply-add; other modifications produce log2 units directly.
+  constexpr bool kNatural = kBias && !kSoftcap && !kAlibi;
+  const float c2 = kNatural ? kLog2e : (kMod ? 1.0f : p.scale_log2);  // s * c2 is the logit in log2 units
   // The running maximum only moves when some row of the wave sees a score more than kTau (log2 units) above it,
   // so exp2 arguments stay <= kTau and the accumulators are rescaled on few tiles.  Any m gives the same O / l.
   constexpr float kTau = 8.0f;
+
+  // Gate logits of this lane's output elements, fetched before the key loop when they fit the register budget so that
+  // their latency is not paid in the epilogue.
+  constexpr bool kGateEarly = kGate && DV <= 32;
+  bf16x4 gpre[kGateEarly ? DVB : 1][kGateEarly ? QB : 1][4];
+  if constexpr (kGateEarly) {
+    if (p.gate) {
+      const bf16_t* gp = p.gate + (int64_t)batch * p.gs[0] + (int64_t)head * p.gs[1];
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            gpre[dvb][qb][g] = *reinterpret_cast<const bf16x4*>(gp + (int64_t)min(qrow[qb], p.Lq - 1) * p.gs[2] +
+                                                                32 * dvb + 8 * g + 4 * h);
+    }
+  }
 
   f32x16 ofin[kDiff ? DVB : 1][kDiff ? QB : 1];  // branch-0 result kept while branch 1 runs (diff only)
   f32x16 oacc[DVB][QB];
@@ -474,6 +521,59 @@ void fwd_kernel(const KParams p) {
         }
       }
     };
+    // Staged bias operand: this wave's rows [qw0, qw0 + RW) x the tile's BN keys, lane -> (row, physical chunk) of the
+    // wave's LDS image; rows past Lq repeat the last row (their results are never stored).
+    using LB = BiasLayout<BN>;
+    const int nbl = kBias ? p.bias_lds : -1;
+    const bool stage_bias = kBias && nbl >= 0;
+    const bf16_t* bptr = nullptr;
+    const unsigned lds_b = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::B_OFF + wave * (RW * BN * 2));
+    unsigned boff[T::B_PER_T > 0 ? T::B_PER_T : 1];
+    if constexpr (kBias) {
+      if (stage_bias) {
+        bptr = p.bias[nbl] + (int64_t)(batch / p.bdiv[nbl]) * p.bs[nbl][0] + (int64_t)head * p.bs[nbl][1];
+#pragma unroll
+        for (int it = 0; it < T::B_PER_T; ++it) {
+          const int id = it * 64 + lane, row = id / LB::CPR, pc = id % LB::CPR;
+          boff[it] = (unsigned)(min(qw0 + row, p.Lq - 1) * (int)p.bs[nbl][2] + LB::swz(row, pc) * 8) * 2u;
+        }
+      }
+    }
+    const int nbr = kBias ? p.bias_row : -1;
+    const bf16_t* rptr = nullptr;
+    const unsigned lds_r = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::R_OFF + wave * 1024);
+    if constexpr (kBias) {
+      if (nbr >= 0) rptr = p.bias[nbr] + (int64_t)(batch / p.bdiv[nbr]) * p.bs[nbr][0] + (int64_t)head * p.bs[nbr][1];
+    }
+    bool any_direct = false;
+    if constexpr (kBias) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) any_direct = any_direct || (p.bias[nb] != nullptr && nb != nbr && nb != nbl);
+    }
+    auto load_b = [&](int t, int slot) FL_INLINE {
+      if constexpr (kBias) {
+        if (nbr >= 0) {
+          // lanes repeat the row's BN / 8 chunks; chunks past Lk repeat the last one
+          const int last_chunk = (min(p.Lk - t * BN, BN)) / 8 - 1;
+          dma16(uniform_ptr(rptr + (int64_t)t * BN), (unsigned)min(lane % LB::CPR, last_chunk) * 16u, lds_r + slot * T::RBYTES);
+        }
+        if (!stage_bias) return;
+        const uint64_t base = uniform_ptr(bptr + (int64_t)t * BN);
+        if (t * BN + BN <= p.Lk) {
+#pragma unroll
+          for (int it = 0; it < T::B_PER_T; ++it) dma16(base, boff[it], lds_b + slot * T::BBYTES + it * 1024);
+        } else {
+          const int last_chunk = (p.Lk - t * BN) / 8 - 1;  // Lk % 8 == 0 whenever a bias is staged
+#pragma unroll
+          for (int it = 0; it < T::B_PER_T; ++it) {
+            const int id = it * 64 + lane, row = id / LB::CPR, pc = id % LB::CPR;
+            const unsigned off =
+                (unsigned)(min(qw0 + row, p.Lq - 1) * (int)p.bs[nbl][2] + min(LB::swz(row, pc), last_chunk) * 8) * 2u;
+            dma16(base, off, lds_b + slot * T::BBYTES + it * 1024);
+          }
+        }
+      }
+    };
     // tile index / this wave's class of a tile-list entry
     auto entry_tile = [&](uint32_t e) FL_INLINE  { return (int)(__builtin_amdgcn_readfirstlane(e) & 0xffffu); };
     auto entry_class = [&](uint32_t e) FL_INLINE  { return (int)((__builtin_amdgcn_readfirstlane(e) >> (16 + 2 * wave)) & 3u); };
@@ -499,9 +599,9 @@ void fwd_kernel(const KParams p) {
         }
     };
 
-    // ---- score modifications and element mask of one tile; afterwards s is in log2 units when kMod ----------------
+    // ---- score modifications of one tile; afterwards s * c2 is the logit in log2 units ---------------------------------
     // Register i of block (kb, qb) is key k0 + 32*kb + 8*(i/4) + 4*h + i%4 against query qrow[qb].
-    auto score_mods = [&](f32x16 (&s)[KB][QB], int t) FL_INLINE {
+    auto score_mods = [&](f32x16 (&s)[KB][QB], int t, int bslot) FL_INLINE {
       const int k0 = t * BN;
       if constexpr (kMod) {
 #pragma unroll
@@ -514,22 +614,46 @@ void fwd_kernel(const KParams p) {
             if constexpr (kBias) {
 #pragma unroll
               for (int i = 0; i < 16; ++i) bv[i] = 0.f;
-#pragma unroll
-              for (int nb = 0; nb < 2; ++nb) {
-                if (p.bias[nb] == nullptr) continue;
-                const bf16_t* bp = p.bias[nb] + (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] +
-                                   (int64_t)head * p.bs[nb][1] + (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
+              if (nbr >= 0) {
+                // row-broadcast operand: keys 32 kb + 8 g + 4 h .. + 4 of this wave's staged row
+                const unsigned char* bl = smem + T::R_OFF + bslot * T::RBYTES + wave * 1024 + 8 * h;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                  const int key = kbase + 8 * g;
-                  if (p.bias_vec[nb] && key + 3 < p.Lk) {
-                    bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bp + key);
+                  const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bl + (4 * kb + g) * 16);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
-                  } else {
+                  for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                }
+              }
+              if (nbl >= 0) {
+                // staged tile: the same keys of row 32 qb + r from this wave's LDS image
+                const int row = 32 * qb + r;
+                const unsigned char* bl = smem + T::B_OFF + bslot * T::BBYTES + wave * (RW * BN * 2) + row * (BN * 2) + 8 * h;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                      if (key + e < p.Lk) bv[4 * g + e] += (float)bp[(int64_t)(key + e) * p.bs[nb][3]];
+                for (int g = 0; g < 4; ++g) {
+                  const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bl + LB::swz(row, 4 * kb + g) * 16);
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                }
+              }
+              if (any_direct) {
+                // operands that cannot be staged (unaligned rows, ragged key count, a third dense operand): read from
+                // global memory where they are used
+                for (int nb = 0; nb < 2; ++nb) {
+                  if (p.bias[nb] == nullptr || nb == nbr || nb == nbl) continue;
+                  const bf16_t* bp = p.bias[nb] + (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] +
+                                     (int64_t)head * p.bs[nb][1] + (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
+#pragma unroll
+                  for (int g = 0; g < 4; ++g) {
+                    const int key = kbase + 8 * g;
+                    if (p.bias_vec[nb] && key + 3 < p.Lk) {
+                      bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bp + key);
+#pragma unroll
+                      for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                    } else {
+#pragma unroll
+                      for (int e = 0; e < 4; ++e)
+                        if (key + e < p.Lk) bv[4 * g + e] += (float)bp[(int64_t)(key + e) * p.bs[nb][3]];
+                    }
                   }
                 }
               }
@@ -538,15 +662,19 @@ void fwd_kernel(const KParams p) {
             for (int i = 0; i < 16; ++i) {
               const float x = s[kb][qb][i];
               float tl2;
-              if constexpr (kSoftcap) {
-                const float e = fast_exp2(x * cap_k1);
-                const float rc = fast_rcp(e + 1.0f);
-                tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
+              if constexpr (kNatural) {
+                tl2 = __builtin_fmaf(x, p.scale, bv[i]);  // natural units: one operation per score
               } else {
-                tl2 = x * p.scale_log2;
+                if constexpr (kSoftcap) {
+                  const float e = fast_exp2(x * cap_k1);
+                  const float rc = fast_rcp(e + 1.0f);
+                  tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
+                } else {
+                  tl2 = x * p.scale_log2;
+                }
+                if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
+                if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
               }
-              if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
-              if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
               s[kb][qb][i] = tl2;
             }
           }
@@ -699,7 +827,7 @@ void fwd_kernel(const KParams p) {
     __syncthreads();  // the previous branch (if any) is done with the LDS buffers
     if (n_list > 0) {
       constexpr int NS = T::NS;
-      constexpr int LPS = T::K_PER_T + T::V_PER_T;  // transfers per thread per step
+      constexpr int LPS = T::K_PER_T + T::V_PER_T + T::B_PER_T + T::R_PER_T;  // transfers per thread per step
       // ent[j] = tile-list entry of list position pos + j (the last entry again past the end of the list).  Entries are
       // read from LDS NS steps before they are needed, so the read latency never shows.
       int pos = 0;
@@ -709,7 +837,10 @@ void fwd_kernel(const KParams p) {
       // prologue: K of the first NS tiles and V of the first NS - 1 go to their ring slots; raw S of the first tile
 #pragma unroll
       for (int j = 0; j < NS; ++j)
-        if (j < n_list) load_k(entry_tile(ent[j]), j);
+        if (j < n_list) {
+          load_k(entry_tile(ent[j]), j);
+          load_b(entry_tile(ent[j]), j);
+        }
 #pragma unroll
       for (int j = 0; j + 1 < NS; ++j)
         if (j < n_list) load_v(entry_tile(ent[j]), j);
@@ -717,7 +848,7 @@ void fwd_kernel(const KParams p) {
       __syncthreads();
       f32x16 s_a[KB][QB], s_b[KB][QB];
       qk(s_a, 0);
-      score_mods(s_a, entry_tile(ent[0]));
+      score_mods(s_a, entry_tile(ent[0]), 0);
       __syncthreads();  // K slot 0 may be overwritten from here on
 
       // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
@@ -740,7 +871,10 @@ void fwd_kernel(const KParams p) {
         // K slot `slot` held this tile's K and V slot `slot - 1` the previous tile's V: both were last read before the
         // barrier that ended the previous step
         const bool steady = pos + NS < n_list;
-        if (steady) load_k(entry_tile(ent[NS]), slot);
+        if (steady) {
+          load_k(entry_tile(ent[NS]), slot);
+          load_b(entry_tile(ent[NS]), slot);  // the bias of this step's tile was consumed at the end of the previous step
+        }
         if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
         settle(sc, ent[0]);
         bf16x8 pf[QB][2 * KB];
@@ -751,7 +885,7 @@ void fwd_kernel(const KParams p) {
         qk(sn, (slot + 1) % NS);
         softmax_p(sc, pf);
         pv_mma(pf, slot);
-        score_mods(sn, entry_tile(ent[1]));
+        score_mods(sn, entry_tile(ent[1]), (slot + 1) % NS);
         {
           constexpr int NA = KS * KB * QB, NB = 2 * KB * DVB * QB;
           constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp + add per score, one pack per two
@@ -835,7 +969,9 @@ void fwd_kernel(const KParams p) {
         const int dv = 32 * dvb + 8 * g + 4 * h;
         bf16x4 o4;
         if (kGate && gptr) {
-          bf16x4 g4 = *reinterpret_cast<const bf16x4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
+          bf16x4 g4;
+          if constexpr (kGateEarly) g4 = gpre[dvb][qb][g];
+          else g4 = *reinterpret_cast<const bf16x4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));

@@ -253,6 +253,30 @@ def test_evoformer_bias_layouts():
         assert_parity(out, ref, name)
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_evoformer_bias_staged_and_direct_paths(D):
+    # S = 104: the key count is a multiple of 8 (bias rows travel through LDS) but not of any key tile or query block,
+    # so the last staged tile is ragged in both directions.  Operand pairs cover: row-broadcast + dense, two dense
+    # (the second one is read directly), two row-broadcast, and a dense operand whose rows start 2 bytes off a 16-byte
+    # boundary (read directly), each with the sigmoid gate.
+    g = torch.Generator().manual_seed(170 + D)
+    mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(DEV)
+    B, N, S, H = 1, 3, 104, 2
+    Q, K, V, G = mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D)
+    wide = mk(B, 1, H, S, S + 8)
+    cases = {
+        "mask + pair": [mk(B, N, 1, 1, S), mk(B, 1, H, S, S)],
+        "two dense": [mk(B, 1, H, S, S), mk(B, N, H, S, S)],
+        "two masks": [mk(B, N, 1, 1, S), mk(B, 1, 1, 1, S)],
+        "misaligned rows": [wide[..., 1:S + 1]],
+        "padded rows": [wide[..., 8:S + 8]],
+    }
+    for name, biases in cases.items():
+        out = A.attention_reference(Q, K, V, biases, gate=G)
+        ref = O.attention_evoformer(*f32(Q, K, V), [b.float() for b in biases], gate=G.float())
+        assert_parity(out, ref, f"D={D} {name}")
+
+
 def test_front_end_errors_on_gpu_tensors():
     q, k, v = qkv(1, 4, 2, 64, 64)
     with pytest.raises(ValueError, match="enable_gqa"):

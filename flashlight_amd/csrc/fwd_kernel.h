@@ -342,59 +342,90 @@ void fwd_kernel(const KParams p) {
   const int qw0 = q0 + wave * RW;     // first query row of this wave
   const int nk = p.n_ktiles;
 
-  // ---- classify every key tile for every wave, then compact the non-empty ones into the tile list ---------------
-  {
-    const int64_t* dtab = kDoc ? p.doc_table + (int64_t)batch * p.doc_blocks * 2 : nullptr;
-    int64_t qmn[NW], qmx[NW];
-    if constexpr (kDoc) {
+  // ---- which key tiles this workgroup visits ------------------------------------------------------------------------
+  // Positional masks attend one contiguous range of key tiles, [t_lo, t_lo + n_list): list position i is tile t_lo + i
+  // and its class for this wave is computed where it is needed.  Document masks can attend scattered tiles: every key
+  // tile is classified for every wave and the non-empty ones are compacted into the LDS tile list.
+  int n_list = 0, t_lo = 0;
+  if constexpr (kDoc) {
+    {
+      const int64_t* dtab = kDoc ? p.doc_table + (int64_t)batch * p.doc_blocks * 2 : nullptr;
+      int64_t qmn[NW], qmx[NW];
+      if constexpr (kDoc) {
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        int a = q0 + w * RW, b = min(a + RW, p.Lq);
-        qmn[w] = 0;
-        qmx[w] = 0;
-        if (a < b) doc_range(dtab, a, b, qmn[w], qmx[w]);
-      }
-    }
-    for (int t = tid; t < nk; t += NT) {
-      const int k0 = t * BN, k1 = min(k0 + BN, p.Lk);
-      int64_t kmn = 0, kmx = 0;
-      if constexpr (kDoc) doc_range(dtab, k0, k1, kmn, kmx);
-      unsigned c = 0;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        int a = q0 + w * RW, b = min(a + RW, p.Lq);
-        int cw = TILE_EMPTY;
-        if (a < b) {
-          cw = classify_positional(p.mask_kind, a, b, k0, k1, p.window, p.prefix);
-          if constexpr (kDoc) {
-            if (kmx < qmn[w] || kmn > qmx[w]) cw = TILE_EMPTY;
-            else if (!(kmn == kmx && qmn[w] == qmx[w] && kmn == qmn[w]) && cw == TILE_FULL) cw = TILE_PARTIAL;
-          }
-          if (cw == TILE_FULL && k0 + BN > p.Lk) cw = TILE_PARTIAL;  // ragged tail: keys >= Lk are masked
+        for (int w = 0; w < NW; ++w) {
+          int a = q0 + w * RW, b = min(a + RW, p.Lq);
+          qmn[w] = 0;
+          qmx[w] = 0;
+          if (a < b) doc_range(dtab, a, b, qmn[w], qmx[w]);
         }
-        c |= (unsigned)cw << (2 * w);
       }
-      tlist[t] = (c << 16) | (unsigned)t;
+      for (int t = tid; t < nk; t += NT) {
+        const int k0 = t * BN, k1 = min(k0 + BN, p.Lk);
+        int64_t kmn = 0, kmx = 0;
+        if constexpr (kDoc) doc_range(dtab, k0, k1, kmn, kmx);
+        unsigned c = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+          int a = q0 + w * RW, b = min(a + RW, p.Lq);
+          int cw = TILE_EMPTY;
+          if (a < b) {
+            cw = classify_positional(p.mask_kind, a, b, k0, k1, p.window, p.prefix);
+            if constexpr (kDoc) {
+              if (kmx < qmn[w] || kmn > qmx[w]) cw = TILE_EMPTY;
+              else if (!(kmn == kmx && qmn[w] == qmx[w] && kmn == qmn[w]) && cw == TILE_FULL) cw = TILE_PARTIAL;
+            }
+            if (cw == TILE_FULL && k0 + BN > p.Lk) cw = TILE_PARTIAL;  // ragged tail: keys >= Lk are masked
+          }
+          c |= (unsigned)cw << (2 * w);
+        }
+        tlist[t] = (c << 16) | (unsigned)t;
+      }
     }
-  }
-  __syncthreads();
-  if (wave == 0) {
-    // in-place compaction by one wave, 64 tiles at a time: an entry never moves to a higher index, and every chunk
-    // is read completely before it is written
-    int count = 0;
-    for (int base = 0; base < nk; base += 64) {
-      const int t = base + lane;
-      const uint32_t e = t < nk ? tlist[t] : 0u;
-      const bool keep = (e >> 16) != 0;
-      const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
-      const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-      if (keep) tlist[pos] = e;
-      count += __builtin_popcountll(m);
+    __syncthreads();
+    if (wave == 0) {
+      // in-place compaction by one wave, 64 tiles at a time: an entry never moves to a higher index, and every chunk
+      // is read completely before it is written
+      int count = 0;
+      for (int base = 0; base < nk; base += 64) {
+        const int t = base + lane;
+        const uint32_t e = t < nk ? tlist[t] : 0u;
+        const bool keep = (e >> 16) != 0;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
+        const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+        if (keep) tlist[pos] = e;
+        count += __builtin_popcountll(m);
+      }
+      if (lane == 0) meta[0] = count;
     }
-    if (lane == 0) meta[0] = count;
+    __syncthreads();
+    n_list = __builtin_amdgcn_readfirstlane(meta[0]);
+  } else {
+    const int q1 = min(q0 + BM, p.Lq);
+    int hi_key = p.Lk - 1, lo_key = 0;  // first / last key position some row of the workgroup may attend
+    if (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_SLIDING) hi_key = min(hi_key, q1 - 1);
+    if (p.mask_kind == MASK_PREFIX) hi_key = min(hi_key, max(q1, p.prefix) - 1);
+    if (p.mask_kind == MASK_SLIDING) lo_key = max(0, q0 - p.window);
+    t_lo = lo_key / BN;
+    n_list = hi_key >= lo_key ? hi_key / BN - t_lo + 1 : 0;
   }
-  __syncthreads();
-  const int n_list = __builtin_amdgcn_readfirstlane(meta[0]);
+  // tile-list entry of list position i (the last entry again past the end): bits 0-15 tile index, two class bits per
+  // wave from bit 16 on (only this wave's are filled in when the entry is computed rather than read)
+  auto list_entry = [&](int i) FL_INLINE -> uint32_t {
+    if constexpr (kDoc) {
+      return tlist[min(i, n_list - 1)];
+    } else {
+      const int t = t_lo + min(i, n_list - 1);
+      const int a = qw0, b = min(qw0 + RW, p.Lq);
+      int cw = TILE_EMPTY;
+      if (a < b) {
+        const int k0 = t * BN, k1 = min(k0 + BN, p.Lk);
+        cw = classify_positional(p.mask_kind, a, b, k0, k1, p.window, p.prefix);
+        if (cw == TILE_FULL && k0 + BN > p.Lk) cw = TILE_PARTIAL;  // ragged tail: keys >= Lk are masked
+      }
+      return ((uint32_t)cw << (16 + 2 * wave)) | (uint32_t)t;
+    }
+  };
 
   // ---- per-lane constants ----------------------------------------------------------------------------------------
   int qrow[QB];  // query position owned by this lane in each query block
@@ -833,7 +864,7 @@ void fwd_kernel(const KParams p) {
       int pos = 0;
       uint32_t ent[NS + 1];
 #pragma unroll
-      for (int j = 0; j <= NS; ++j) ent[j] = tlist[min(j, n_list - 1)];
+      for (int j = 0; j <= NS; ++j) ent[j] = list_entry(j);
       // prologue: K of the first NS tiles and V of the first NS - 1 go to their ring slots; raw S of the first tile
 #pragma unroll
       for (int j = 0; j < NS; ++j)
@@ -898,7 +929,7 @@ void fwd_kernel(const KParams p) {
         ++pos;
 #pragma unroll
         for (int j = 0; j < NS; ++j) ent[j] = ent[j + 1];
-        ent[NS] = tlist[min(pos + NS, n_list - 1)];
+        ent[NS] = list_entry(pos + NS);
       };
       int last_slot = 0;  // ring slot of the final tile; its scores are in s_a when the slot is even
       bool more = true;

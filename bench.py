@@ -42,7 +42,7 @@ def event_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def time_launches(fn, iters: int, warmup: int = 3):
+def time_launches(fn, iters: int, warmup: int = 20):
     """Trimmed mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
     current stream (the stream the kernels are launched on)."""
     for _ in range(warmup):
@@ -56,6 +56,19 @@ def time_launches(fn, iters: int, warmup: int = 3):
     ts = sorted(a.elapsed_time(b) for a, b in pairs)
     keep = ts[: max(1, int(len(ts) * 0.9))]  # drop the slowest tenth: one-off host hiccups land inside an event pair
     return statistics.fmean(keep), statistics.median(ts)
+
+
+def time_back_to_back(fn, iters: int, warmup: int = 10) -> float:
+    """Average duration (ms) of `iters` launches of `fn` queued back to back between one pair of events."""
+    for _ in range(warmup):
+        fn()
+    a, b = event_pair()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
 
 
 def cpu_baseline(threads_hint: int = 0) -> dict:
@@ -139,9 +152,10 @@ def main():
     # per-launch durations of each variant, HIP events on the launch stream
     variants = {}
     for w in cfg1:
-        mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(20, args.steps))
+        mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(50, args.steps))
         tf = w.flops / mean_ms / 1e9
         variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
+                            "ms_back_to_back": time_back_to_back(lambda w=w: w.call(tens), iters=max(50, args.steps), warmup=20),
                             "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
                             "hbm_floor_GBps_at_this_time": w.min_bytes / mean_ms / 1e6}
     dom = max(cfg1, key=lambda w: variants[w.name]["ms"])  # the launch that dominates the step
@@ -158,13 +172,36 @@ def main():
             if w.config == 1:
                 continue
             t = w.make(dev)
-            mean_ms, med_ms = time_launches(lambda: w.call(t), iters=20)
+            mean_ms = time_back_to_back(lambda: w.call(t), iters=100, warmup=50)
             tf = w.flops / mean_ms / 1e9
-            others[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf,
+            others[w.name] = {"ms": mean_ms, "timing": "100 launches back to back after 50 warm-up launches", "tflops": tf,
                               "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS, "unmasked_flops": w.flops,
                               "min_bytes": w.min_bytes, "GBps_on_min_bytes": w.min_bytes / mean_ms / 1e6}
             del t
             torch.cuda.empty_cache()
+
+    # What the matrix pipe alone sustains on this part (same MFMA instruction, operands in registers, nothing else
+    # running), on N(0,1) operands like the benchmark's and on zeros, and the forward itself on all-zero inputs: the
+    # part lowers its clock under data-dependent power, so these put the roofline fraction in context.
+    context = {}
+    if not args.no_other_configs:
+        n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+        sink = torch.empty(n_cu * 512, dtype=torch.float32, device=dev)
+        g = torch.Generator().manual_seed(7)
+        ops = {"randn_operands": torch.randn(1 << 23, generator=g).to(torch.bfloat16).to(dev),
+               "zero_operands": torch.zeros(1 << 23, dtype=torch.bfloat16, device=dev)}
+        for tag, x in ops.items():
+            flops = [0.0]
+
+            def run(x=x):
+                flops[0] = _ffi.probe_mfma_rate(x, 600, n_cu, sink)
+            ms = time_back_to_back(run, iters=100, warmup=30)
+            context["mfma_only_" + tag + "_TFLOPs"] = flops[0] / ms / 1e9
+        tens = cfg1[0].make(dev)
+        zeros = {k: torch.zeros_like(v) for k, v in tens.items()}
+        ms = time_back_to_back(lambda: cfg1[0].call(zeros), iters=100, warmup=30)
+        context["vanilla_on_zero_inputs_TFLOPs"] = cfg1[0].flops / ms / 1e9
+        del tens, zeros, ops
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -181,7 +218,7 @@ def main():
                    "seed": cfg1[0].seed, "unmasked_flops_per_step": step_flops},
         "pct_mfma_peak": 100 * step_flops / wall_ms / 1e9 / W.PEAK_BF16_TFLOPS,
         "peak_used_TFLOPs": W.PEAK_BF16_TFLOPS,
-        "variants": variants, "roofline": roofline, "other_configs": others,
+        "variants": variants, "roofline": roofline, "other_configs": others, "power_context": context,
         "device": torch.cuda.get_device_name(0),
     }
     if not args.no_cpu_baseline:

@@ -77,6 +77,8 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_plan.argtypes = [C.POINTER(FlAttnParams), C.POINTER(C.c_int64)]
     lib.fl_attn_fwd.restype = C.c_int
     lib.fl_attn_fwd.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
+    lib.fl_probe_mfma_rate.restype = C.c_int
+    lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
         raise RuntimeError(f"{p}: ABI version {lib.fl_version()} != expected {ABI_VERSION}")
     if lib.fl_params_sizeof() != C.sizeof(FlAttnParams):
@@ -250,3 +252,19 @@ def plan(p: FlAttnParams) -> dict:
     _check(lib.fl_attn_plan(C.byref(p), out))
     return {"rows_per_workgroup": out[0], "keys_per_tile": out[1], "threads": out[2], "workgroups": out[3],
             "lds_bytes": out[4], "features": out[5]}
+
+
+def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink: torch.Tensor) -> float:
+    """Launches the MFMA-only rate probe on the current stream (measurement aid, include/flashlight_amd.h) and returns
+    the FLOPs of the launch.  `operands`: bf16 device tensor (multiple of 8 elements, 16-byte aligned) the per-lane
+    fragments are read from; `sink`: float32 device tensor of n_workgroups * 512 elements."""
+    if operands.dtype != torch.bfloat16 or not operands.is_cuda or not operands.is_contiguous() or operands.numel() % 8:
+        raise ValueError("operands must be a contiguous bf16 device tensor with a multiple of 8 elements")
+    if sink.dtype != torch.float32 or sink.numel() < n_workgroups * 512 or sink.device != operands.device:
+        raise ValueError("sink must be a float32 tensor of n_workgroups * 512 elements on the operands' device")
+    stream = torch.cuda.current_stream(operands.device).cuda_stream
+    rc = load_library().fl_probe_mfma_rate(operands.data_ptr(), operands.numel() // 8, int(iters), int(n_workgroups),
+                                           sink.data_ptr(), C.c_void_p(stream))
+    if rc != 0:
+        raise FlashlightError(rc, "fl_probe_mfma_rate rejected its arguments" if rc < 0 else "probe launch failed")
+    return float(n_workgroups) * 8 * iters * 32 * 32768.0

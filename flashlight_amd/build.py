@@ -111,7 +111,7 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
             tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_NAME={name}", f"-DFL_INST_ARGS={args}", "-c",
                            str(CSRC / "instance_unit.hip"), "-o", str(o)], o))
     # the instance table is host data only: compiling it for the device would reference the host launchers
-    for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("api.hip", [])):
+    for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("api.hip", []), ("probe.hip", [])):
         o = objdir / (Path(src).stem + ".o")
         objs.append(o)
         if not o.exists():

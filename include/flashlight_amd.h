@@ -132,6 +132,15 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream);
  * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
 int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
 
+/* Measurement aid with no counterpart in the reference: launches a kernel that does nothing but issue
+ * v_mfma_f32_32x32x16_bf16 (the instruction both products of the forward are built from) on operand fragments read
+ * once from `operands`, so that the matrix-pipe rate this part sustains on given data can be put next to the
+ * forward's.  One workgroup of 512 threads per compute unit, two waves per SIMD; every lane reads 12 16-byte
+ * fragments (8 A, 4 B) at 16-byte index (thread * 12 + j) % n_fragments and issues iters * 32 MFMAs; one float per
+ * thread is written to `sink` (n_workgroups * 512 floats).  Work = n_workgroups * 8 * iters * 32 * 32768 FLOP.
+ * Returns 0, or a negative code for bad arguments (see fl_last_error()). */
+int fl_probe_mfma_rate(const void* operands, int64_t n_fragments, int iters, int n_workgroups, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -142,3 +142,13 @@ def test_front_end_refuses_cpu_and_fp32_tensors(lib):
         attention_pytorch_alibi(q, q, q, score_mod=lambda a, b: None)
     with pytest.raises(TypeError):
         attention_pytorch_alibi(q, q, q)
+
+
+def test_probe_rejects_bad_arguments_without_a_gpu(lib):
+    # the measurement aid checks its arguments on the host before it launches anything
+    assert lib.fl_probe_mfma_rate(None, 1, 1, 1, None, None) == -5
+    buf = (C.c_char * 64)()
+    addr = C.addressof(buf)
+    aligned = (addr + 15) // 16 * 16
+    assert lib.fl_probe_mfma_rate(C.c_void_p(aligned), 0, 1, 1, C.c_void_p(aligned), None) == -5
+    assert lib.fl_probe_mfma_rate(C.c_void_p(aligned + 2), 1, 1, 1, C.c_void_p(aligned), None) == -7

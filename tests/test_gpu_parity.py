@@ -290,3 +290,14 @@ def test_front_end_errors_on_gpu_tensors():
     q48 = torch.randn(1, 2, 64, 48, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
         A.attention_pytorch(q48, q48, q48)
+
+
+def test_mfma_rate_probe_runs_and_sums_products():
+    # 8 x 4 fragment pairs of ones: every accumulator element ends at 16 (k) * 8 (A fragments) * iters per B fragment
+    iters, wgs = 3, 2
+    ones = torch.ones(1 << 12, dtype=torch.bfloat16, device=DEV)
+    sink = torch.zeros(wgs * 512, dtype=torch.float32, device=DEV)
+    flops = _ffi.probe_mfma_rate(ones, iters, wgs, sink)
+    torch.cuda.synchronize()
+    assert flops == wgs * 8 * iters * 32 * 32768
+    assert torch.all(sink == 16.0 * 8 * iters * 4 * 16)

@@ -222,8 +222,8 @@ enum : int { SG_VALU = 0x2, SG_MFMA = 0x8, SG_DS_READ = 0x100, SG_TRANS = 0x400 
 // Orders the step's instructions as: each first-product MFMA preceded by its K fragment read and followed by a
 // share of the exponential work; each second-product MFMA preceded by its two transposing V reads and followed
 // by a share of the next tile's row maximum.  NA / NB = MFMAs in the two products, VA / VB = vector ops to spread.
-template <int NA, int NB, int VA, int VB>
-__device__ __forceinline__ void sched_tile_step() {
+template <int NA, int VA>
+__device__ __forceinline__ void sched_first_product() {
 #if FL_SCHED == 1
   __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 2, 0);
 #pragma unroll
@@ -232,6 +232,11 @@ __device__ __forceinline__ void sched_tile_step() {
     if (i + 2 < NA) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
     __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, VA, 0);
   }
+#endif
+}
+template <int NB, int VB>
+__device__ __forceinline__ void sched_second_product() {
+#if FL_SCHED == 1
   __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 4, 0);
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
@@ -239,10 +244,6 @@ __device__ __forceinline__ void sched_tile_step() {
     if (i + 2 < NB) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 2, 0);
     if (VB > 0) __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, VB, 0);
   }
-#elif FL_SCHED == 2
-  __builtin_amdgcn_iglp_opt(2);
-#elif FL_SCHED == 3
-  __builtin_amdgcn_iglp_opt(3);
 #endif
 }
 
@@ -763,6 +764,27 @@ void fwd_kernel(const KParams p) {
       }
     };
 
+    // ---- A operand of O^T += V^T . P^T for 16-key chunk c and value block dvb, through the transposing LDS read.
+    // Slot j of lane (r, h) is key 16c + 8*(j/4) + 4h + j%4, the key order of the packed weights.
+    auto v_frag = [&](int buf, int c, int dvb) FL_INLINE -> bf16x8 {
+      const unsigned char* vb_ = smem + T::V_OFF + buf * T::VBYTES;
+      bf16x8 vf;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // within each 16-lane group, lane i supplies row (key) i/4, 4 columns at 4*(i%4), and receives column i
+        // of the 4 rows
+        const int i16 = lane % 16, g = (lane / 16) % 2;
+        const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
+        const int col = dvb * 32 + g * 16 + 4 * (i16 % 4);
+        const unsigned char* ap = vb_ + row * (DV * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
+        typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+        const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
+        const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
+      }
+      return vf;
+    };
     // ---- running maximum: row maxima of one tile; the accumulators are rescaled when a maximum grew by more than kTau
     auto row_max = [&](const f32x16 (&s)[KB][QB], float (&mx)[QB]) FL_INLINE {
 #pragma unroll
@@ -775,8 +797,8 @@ void fwd_kernel(const KParams p) {
         mx[qb] = xhalf_max(m);
       }
     };
-    auto rescale_if_grown = [&](const float (&mx)[QB]) FL_INLINE {
-      bool grow = false;
+    auto rescale_if_grown = [&](const float (&mx)[QB], bool force) FL_INLINE {
+      bool grow = force;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb)
         grow = grow | ((mx[qb] - m_run[qb]) * c2 > kTau);  // m_run = -inf before the first tile: always true
@@ -785,7 +807,10 @@ void fwd_kernel(const KParams p) {
         for (int qb = 0; qb < QB; ++qb) {
           const float m_new = __builtin_fmaxf(m_run[qb], mx[qb]);
           const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // row fully masked so far
-          const float alpha = fast_exp2((m_run[qb] - m_use) * c2);
+          // before the first update the reference is 0 (see softmax_p); the clamp keeps 0 * inf out of accumulators
+          // whose contents have underflowed to nothing
+          const float m_old = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
+          const float alpha = __builtin_fminf(fast_exp2((m_old - m_use) * c2), 0x1p126f);
           m_run[qb] = m_new;
           l_run[qb] *= alpha;
 #pragma unroll
@@ -797,7 +822,7 @@ void fwd_kernel(const KParams p) {
     };
 
     // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
-    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB]) FL_INLINE {
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB], float (&rsum)[QB]) FL_INLINE {
       typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
       const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
 #pragma unroll
@@ -822,33 +847,63 @@ void fwd_kernel(const KParams p) {
             }
           }
         }
-        l_run[qb] += rs;
+        rsum[qb] = rs;
       }
+    };
+    // Tiles that need no element mask skip the row maximum altogether: their weights are formed against the running
+    // reference m_run as it stands, and the row sums (needed anyway) tell whether that was safe.  A lane whose sum
+    // is not <= kBig (a weight overflowed, or NaN), or whose sum and running sum are both < kTiny (the tile may have
+    // underflowed with nothing to be negligible against), sends the wave through the exact path: row maxima, new
+    // reference, weights again.  Any reference gives the same O / l; fp32 sums keep their relative precision.
+    // ALiBi moves the scores by a large, steady amount from tile to tile, which would send most tiles through the
+    // exact path after the fact: kernels with ALiBi take the exact path up front instead.
+    constexpr float kBig = 0x1p24f, kTiny = 0x1p-24f;
+    constexpr bool kFastRef = !kAlibi;
+    auto weights_checked = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB], bool check, auto in_loop,
+                               bf16x8 (&vfirst)[DVB], int vslot) FL_INLINE {
+      float rs[QB];
+      softmax_p(s, pf, rs);
+      if constexpr (decltype(in_loop)::value) {
+        // inside the pipelined step the exponentials share a block with the first product's MFMAs (issued by the
+        // caller just before): interleave them
+        constexpr int NA = KS * KB * QB;
+        constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp per score, one pack and one dot2 per two
+        sched_first_product<NA, (n_exp * 3 + NA - 1) / NA>();
+      }
+      if constexpr (decltype(in_loop)::value) {
+        // the second product's first V fragments are fetched here, ahead of the branch below, so that their LDS
+        // latency runs under the exponentials
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          vfirst[dvb] = v_frag(vslot, 0, dvb);
+        }
+      }
+      if (check) {
+        bool bad = false;
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) bad = bad | !(rs[qb] <= kBig) | ((rs[qb] < kTiny) & (l_run[qb] < kTiny));
+        if (__builtin_amdgcn_ballot_w64(bad) != 0) {
+          float mx[QB];
+          row_max(s, mx);
+          rescale_if_grown(mx, true);
+          softmax_p(s, pf, rs);
+        }
+      }
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) l_run[qb] += rs[qb];
     };
 
     // ---- O^T += V^T . P^T: A = V fragment through the transposing LDS read, B = P ---------------------------------------
     // A operand slot j of lane (r, h) for 16-key chunk c is key 16c + 8*(j/4) + 4h + j%4, the key order of pf.
-    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf) FL_INLINE {
-      const unsigned char* vb_ = smem + T::V_OFF + buf * T::VBYTES;
+    // `first` holds the fragments of key chunk 0 when the caller has fetched them ahead (HAVE_FIRST)
+    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf, const bf16x8 (&first)[DVB], auto have_first) FL_INLINE {
 #pragma unroll
       for (int c = 0; c < 2 * KB; ++c)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
           bf16x8 vf;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            // within each 16-lane group, lane i supplies row (key) i/4, 4 columns at 4*(i%4), and receives column i
-            // of the 4 rows
-            const int i16 = lane % 16, g = (lane / 16) % 2;
-            const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
-            const int col = dvb * 32 + g * 16 + 4 * (i16 % 4);
-            const unsigned char* ap = vb_ + row * (DV * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
-            typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
-            const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
-            const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
-          }
+          if (decltype(have_first)::value && c == 0) vf = first[dvb];
+          else vf = v_frag(buf, c, dvb);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb)
             oacc[dvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][c], oacc[dvb][qb], 0, 0, 0);
@@ -886,11 +941,14 @@ void fwd_kernel(const KParams p) {
       // maxima, and the (rare) rescale.
       auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e) FL_INLINE {
         const int t = entry_tile(e);
-        if (entry_class(e) != TILE_FULL) apply_mask(sc, t);
+        const bool full = entry_class(e) == TILE_FULL;
+        if (!full || !kFastRef) {
+          if (!full) apply_mask(sc, t);
+          float mx[QB];
+          row_max(sc, mx);
+          rescale_if_grown(mx, false);
+        }
         dump_attended(sc, t);
-        float mx[QB];
-        row_max(sc, mx);
-        rescale_if_grown(mx);
       };
       // One pipeline step for list position pos with pos % NS == slot: `sc` holds the (score-modified, unmasked)
       // scores of the current tile on entry and `sn` receives those of the next one.  K of list position j lives in K
@@ -914,13 +972,15 @@ void fwd_kernel(const KParams p) {
         // the other does vector work) instead of both stalling on each other.
         __builtin_amdgcn_s_setprio(3);
         qk(sn, (slot + 1) % NS);
-        softmax_p(sc, pf);
-        pv_mma(pf, slot);
+        bf16x8 vfirst[DVB];
+        weights_checked(sc, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::true_type{}, vfirst, slot);
+        pv_mma(pf, slot, vfirst, std::true_type{});
         score_mods(sn, entry_tile(ent[1]), (slot + 1) % NS);
         {
-          constexpr int NA = KS * KB * QB, NB = 2 * KB * DVB * QB;
-          constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp + add per score, one pack per two
-          sched_tile_step<NA, NB, (n_exp * 7 / 2 + NA - 1) / NA, 0>();
+          // the next tile's score modifications (if any) go under the second product's MFMAs
+          constexpr int NB = 2 * KB * DVB * QB;
+          constexpr int mod_ops = (kSoftcap ? 4 : (kMod ? 1 : 0)) + (kAlibi ? 2 : 0) + (kBias ? 3 : 0);
+          sched_second_product<NB, (16 * KB * QB * mod_ops + NB - 1) / NB>();
         }
         __builtin_amdgcn_s_setprio(0);
         // the next step reads K and V transfers issued NS - 2 steps ago: later ones may stay in flight
@@ -949,14 +1009,15 @@ void fwd_kernel(const KParams p) {
         constexpr int slot = decltype(idx)::value;
         if (last_slot != slot) return true;
         bf16x8 pf[QB][2 * KB];
+        bf16x8 vfirst[DVB];
         if constexpr (slot % 2 == 0) {
           settle(s_a, ent[0]);
-          softmax_p(s_a, pf);
+          weights_checked(s_a, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot);
         } else {
           settle(s_b, ent[0]);
-          softmax_p(s_b, pf);
+          weights_checked(s_b, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot);
         }
-        pv_mma(pf, slot);
+        pv_mma(pf, slot, vfirst, std::false_type{});
         return false;
       });
     }

@@ -301,3 +301,25 @@ def test_mfma_rate_probe_runs_and_sums_products():
     torch.cuda.synchronize()
     assert flops == wgs * 8 * iters * 32 * 32768
     assert torch.all(sink == 16.0 * 8 * iters * 4 * 16)
+
+
+@pytest.mark.parametrize("D,offsets", [
+    (128, [-2600.0, -2000.0, 400.0, 2600.0, -800.0, 3000.0, -3000.0, 0.0]),   # logits jump by hundreds of nats per tile
+    (128, [-3000.0] * 8),                                                       # every logit far below zero
+    (64, [0.0, 1500.0, -1500.0, 30.0, -30.0, 2500.0, 2500.0, -2500.0]),
+])
+def test_reference_free_weights_survive_extreme_logit_ranges(D, offsets):
+    # Unmasked tiles form their weights against the running reference without looking at the row maximum first and
+    # fall back to the exact path when a row sum overflows or underflows.  Keys of the j-th block of 64 carry the
+    # offset offsets[j] along the direction every query points in, so whole tiles sit hundreds of nats above or below
+    # whatever came before; the result must still match the fp32 oracle.
+    S = 64 * len(offsets)
+    g = torch.Generator().manual_seed(18)
+    q = torch.randn(1, 2, S, D, generator=g)
+    k = torch.randn(1, 2, S, D, generator=g)
+    v = torch.randn(1, 2, S, D, generator=g)
+    q[..., 0] = 16.0
+    k[..., 0] = torch.tensor(offsets).repeat_interleave(64) / 16.0
+    q, k, v = (t.bfloat16().to(DEV) for t in (q, k, v))
+    assert_parity(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v)), "vanilla")
+    assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(*f32(q, k, v), enable_gqa=True), "causal")

@@ -716,32 +716,34 @@ void fwd_kernel(const KParams p) {
     // key < Lk && ((dmin <= key - q <= dmax) || key < pfx) [&& same document]; with key = kbase + off and off a
     // compile-time constant per register, every test compares off with a per-lane bound (branch-free).
     // A tile that is empty for this wave (but not for the workgroup) takes the same path and loses every score.
+    // With off = key - kbase a compile-time constant per register, the positional predicate is lo <= off <= hi for
+    // per-lane bounds: every mask is one interval of key - q cut at Lk; the prefix-LM mask is the union of two
+    // intervals that both start at -inf, i.e. again one (dmin is far below any offset unless a window is set).
     auto apply_mask = [&](f32x16 (&s)[KB][QB], int t) FL_INLINE {
       const int k0 = t * BN;
-      {
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          const int kbase = k0 + 32 * kb + 4 * h;
-          const int t_len = p.Lk - kbase;   // off < t_len   <=> key < Lk
-          const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
-          int64_t kdoc[16];
-          if constexpr (kDoc) {
+      for (int kb = 0; kb < KB; ++kb) {
+        const int kbase = k0 + 32 * kb + 4 * h;
+        const int t_len = p.Lk - kbase;   // off < t_len   <=> key < Lk
+        const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
+        int64_t kdoc[16];
+        if constexpr (kDoc) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-              kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
-          }
+          for (int i = 0; i < 16; ++i)
+            kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
+        }
 #pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            const int rel = kbase - qrow[qb];
-            const int t_hi = p.dmax - rel;  // off <= t_hi  <=> key - q <= dmax
-            const int t_lo = p.dmin - rel;  // off >= t_lo  <=> key - q >= dmin
+        for (int qb = 0; qb < QB; ++qb) {
+          const int rel = kbase - qrow[qb];
+          // off <= hi <=> key < Lk && (key - q <= dmax || key < pfx);  off >= lo <=> key - q >= dmin
+          const int hi = min(t_len - 1, max(p.dmax - rel, t_pfx - 1));
+          const int lo = p.dmin - rel;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int off = 8 * (i / 4) + (i % 4);
-              bool ok = (off < t_len) & (((off <= t_hi) & (off >= t_lo)) | (off < t_pfx));
-              if constexpr (kDoc) ok = ok & (kdoc[i] == qdoc[qb]);
-              s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
-            }
+          for (int i = 0; i < 16; ++i) {
+            const int off = 8 * (i / 4) + (i % 4);
+            bool ok = (off <= hi) & (off >= lo);
+            if constexpr (kDoc) ok = ok & (kdoc[i] == qdoc[qb]);
+            s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
           }
         }
       }

@@ -65,6 +65,9 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   // to instances of that shape (the default is the first listed instance that fits).
   int want_rw = 0, want_bn = 0, want_nw = 0, want_ns = 0;
   if (const char* e = std::getenv("FL_TILE")) std::sscanf(e, "%dx%dx%dx%d", &want_rw, &want_bn, &want_nw, &want_ns);
+  // keys one workgroup of 128 query rows visits: the window plus its own rows for a sliding window, else up to Lk
+  const int64_t visited = p->mask_kind == FL_MASK_SLIDING ? std::min<int64_t>(p->Lk, (int64_t)p->window + 128) : p->Lk;
+  const bool short_loop = p->mask_kind == FL_MASK_SLIDING && visited <= 640;
   for (int i = 0; i < fl::kNumInstances; ++i) {
     const fl::Instance& in = fl::kInstances[i];
     if (in.dqk != p->Dqk || in.dv != p->Dv) continue;
@@ -72,7 +75,9 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
     const uint32_t extra = in.feat & ~want;
     if (extra & ~kOptionalFeatures) continue;
     if (want_rw && (in.rw != want_rw || in.bn != want_bn || in.nw != want_nw || (want_ns && in.ns != want_ns))) continue;
-    const int n = __builtin_popcount(extra);
+    // fewer unused features first; among equals the listed order, except that a short key loop prefers the small
+    // workgroup
+    const int n = 2 * __builtin_popcount(extra) + ((in.nw == 2) == short_loop ? 0 : 1);
     if (n < best_extra) {
       best = &in;
       best_extra = n;

@@ -24,8 +24,8 @@ import torch
 def parse_args():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the eager CPU timing (about 20 s)")
     ap.add_argument("--no-other-configs", action="store_true", help="only run the configuration the metric is quoted on")
     ap.add_argument("--calibrate-copy", action="store_true",

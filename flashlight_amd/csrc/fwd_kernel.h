@@ -410,6 +410,31 @@ void fwd_kernel(const KParams p) {
     t_lo = lo_key / BN;
     n_list = hi_key >= lo_key ? hi_key / BN - t_lo + 1 : 0;
   }
+  // This wave's tile classes for a positional mask, as index ranges: tiles outside [e_lo, e_hi] are EMPTY for its
+  // rows [a, b), tiles inside [f_lo, f_hi] FULL, the rest PARTIAL (the same closed forms as classify_positional,
+  // solved for the tile index; the ragged last tile is never FULL because keys >= Lk are masked; a tile may be
+  // called PARTIAL where it is in fact EMPTY or FULL, never the other way round).
+  int e_lo = 0, e_hi = -1, f_lo = 0, f_hi = -1;
+  if constexpr (!kDoc) {
+    const int a = qw0, b = min(qw0 + RW, p.Lq);
+    if (a < b) {
+      const int last = nk - 1, whole = p.Lk / BN - 1;  // last tile; last tile that lies entirely below Lk
+      e_hi = last;
+      f_hi = whole;
+      if (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_SLIDING) {
+        e_hi = min(last, (b - 1) / BN);
+        f_hi = min(whole, (a + 1) / BN - 1);
+      }
+      if (p.mask_kind == MASK_SLIDING) {
+        e_lo = max(0, a - p.window) / BN;
+        f_lo = b - 1 - p.window > 0 ? (b - 1 - p.window + BN - 1) / BN : 0;
+      }
+      if (p.mask_kind == MASK_PREFIX) {
+        e_hi = min(last, (max(p.prefix, b) + BN - 1) / BN - 1);
+        f_hi = min(whole, max(p.prefix / BN, (a + 1) / BN) - 1);
+      }
+    }
+  }
   // tile-list entry of list position i (the last entry again past the end): bits 0-15 tile index, two class bits per
   // wave from bit 16 on (only this wave's are filled in when the entry is computed rather than read)
   auto list_entry = [&](int i) FL_INLINE -> uint32_t {
@@ -417,13 +442,7 @@ void fwd_kernel(const KParams p) {
       return tlist[min(i, n_list - 1)];
     } else {
       const int t = t_lo + min(i, n_list - 1);
-      const int a = qw0, b = min(qw0 + RW, p.Lq);
-      int cw = TILE_EMPTY;
-      if (a < b) {
-        const int k0 = t * BN, k1 = min(k0 + BN, p.Lk);
-        cw = classify_positional(p.mask_kind, a, b, k0, k1, p.window, p.prefix);
-        if (cw == TILE_FULL && k0 + BN > p.Lk) cw = TILE_PARTIAL;  // ragged tail: keys >= Lk are masked
-      }
+      const int cw = (t < e_lo || t > e_hi) ? TILE_EMPTY : ((t >= f_lo && t <= f_hi) ? TILE_FULL : TILE_PARTIAL);
       return ((uint32_t)cw << (16 + 2 * wave)) | (uint32_t)t;
     }
   };
@@ -523,8 +542,12 @@ void fwd_kernel(const KParams p) {
       const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
       voff[it] = (unsigned)(row * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
     }
+    // scalar base addresses; one key tile is less than 2^31 bytes from start to end (checked on the host)
+    const uint64_t kbase = uniform_ptr(kptr), vbase = uniform_ptr(vptr);
+    const uint32_t k_tile_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(BN * (uint32_t)p.ks[2] * 2u));
+    const uint32_t v_tile_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(BN * (uint32_t)p.vs[2] * 2u));
     auto load_k = [&](int t, int slot) FL_INLINE  {
-      const uint64_t base = uniform_ptr(kptr + (int64_t)t * BN * p.ks[2]);
+      const uint64_t base = kbase + (uint64_t)(uint32_t)t * k_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
         for (int it = 0; it < T::K_PER_T; ++it)
@@ -539,7 +562,7 @@ void fwd_kernel(const KParams p) {
       }
     };
     auto load_v = [&](int t, int slot) FL_INLINE  {
-      const uint64_t base = uniform_ptr(vptr + (int64_t)t * BN * p.vs[2]);
+      const uint64_t base = vbase + (uint64_t)(uint32_t)t * v_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
         for (int it = 0; it < T::V_PER_T; ++it)

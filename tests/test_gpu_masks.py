@@ -58,6 +58,26 @@ def test_document_masks_bit_exact(S):
             assert np.array_equal(got[0, 0], want) and np.array_equal(got[0, 1], want), f"{kind}/{tag} S={S}"
 
 
+@pytest.mark.parametrize("Lq,Lk", [(100, 300), (300, 100), (129, 64), (64, 129), (1, 200), (513, 190)])
+def test_unmasked_and_causal_bit_exact_with_unequal_lengths(Lq, Lk):
+    # the causal mask is top-left aligned (query i and key j compare as positions i and j): rows past the last key see
+    # all keys
+    g = torch.Generator().manual_seed(Lq * 1000 + Lk)
+    q = torch.randn(1, 2, Lq, 64, generator=g).bfloat16().to(DEV)
+    k, v = (torch.randn(1, 2, Lk, 64, generator=g).bfloat16().to(DEV) for _ in range(2))
+    # (the sliding-window and prefix-LM masks are defined for Lq == Lk only, like the reference's mask builders)
+    for kind, kws in (("none", [{}]), ("causal", [{}])):
+        for kw in kws:
+            dump = torch.zeros(1, 2, Lq, Lk, dtype=torch.uint8, device=DEV)
+            _ffi.attn_fwd(q, k, v, mask_kind=KIND[kind], window=kw.get("window", 0), prefix=kw.get("prefix", 0),
+                          attended_dump=dump)
+            torch.cuda.synchronize()
+            got = dump.cpu().numpy().astype(bool)
+            want = M.attend_matrix(kind, Lq, Lk, **kw)
+            for h in range(2):
+                assert np.array_equal(got[0, h], want), f"{kind} {kw} Lq={Lq} Lk={Lk}: {np.argwhere(got[0, h] != want)[:5]}"
+
+
 def test_d128_instance_bit_exact():
     for kind, kw in (("causal", {}), ("sliding", {"window": 100}), ("prefix", {"prefix": 70})):
         got = attended_bitmap(kind, 300, D=128, **kw)

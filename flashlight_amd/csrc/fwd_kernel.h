@@ -319,9 +319,10 @@ void fwd_kernel(const KParams p) {
 
   // ---- workgroup -> (batch, head, query tile).  Consecutive workgroup ids land on different XCDs, so ids are
   // regrouped to give every XCD a contiguous run of (batch, head) pairs: their K/V stay in that XCD's L2.
-  // Within a run, heads are taken two at a time and their query tiles dealt from the last (longest under a causal
-  // mask) to the first, alternating between the two heads: the workgroups still running when the grid drains are
-  // the short ones, and an XCD works on the K/V of two heads at a time.
+  // Under masks whose work grows with the query position (causal, prefix-LM, causal documents) heads are taken four
+  // at a time and their query tiles dealt from the last (longest) to the first, round-robin over the four heads: the
+  // workgroups still running when the grid drains are the short ones.  Under the other masks every query tile costs
+  // the same, and heads are taken one at a time (HBM then sees each K/V tile once).
   int bh, qt;
   {
     const int nbh = p.B * p.Hq, nq = p.n_qtiles;
@@ -331,10 +332,11 @@ void fwd_kernel(const KParams p) {
       base = (i % 8) * run;
       i /= 8;
     }
-    const int g = i / (2 * nq), rem = i % (2 * nq);
-    const int gg = min(2, run - 2 * g);
+    const int G = (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || p.mask_kind == MASK_DOC_CAUSAL) ? 4 : 1;
+    const int g = i / (G * nq), rem = i % (G * nq);
+    const int gg = min(G, run - G * g);
     qt = nq - 1 - rem / gg;
-    bh = base + 2 * g + rem % gg;
+    bh = base + G * g + rem % gg;
   }
   const int head = bh % p.Hq, batch = bh / p.Hq;
   const int kvh = head / p.group;

@@ -35,7 +35,7 @@ def parse_args():
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 256 MiB copy's readings);
 # commands and raw values: profiles/fwd_kernel_d128_cfg1_counters.md
-MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 269.1e6, "cfg1/sliding_window": 308.4e6}
+MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 410.6e6, "cfg1/sliding_window": 311.4e6}
 
 
 def event_pair():

@@ -5,7 +5,7 @@ from typing import Optional
 
 import torch
 
-from .. import _ffi
+from .. import _ffi, ops
 
 
 def check_heads(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, enable_gqa: bool) -> None:
@@ -34,4 +34,4 @@ def grouped_view(out: torch.Tensor, key: torch.Tensor, enable_gqa: bool) -> torc
 
 def run(query, key, value, *, scale: Optional[float], enable_gqa: bool, **kw) -> torch.Tensor:
     check_heads(query, key, value, enable_gqa)
-    return _ffi.attn_fwd(query, key, value, scale=scale, **kw)
+    return ops.dispatch(query, key, value, scale=scale, **kw)

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .. import _ffi
+from .. import _ffi, ops
 
 
 def diffattn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale=None, lambda_full=0.2, **kwargs) -> torch.Tensor:
@@ -13,8 +13,8 @@ def diffattn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale=None, lamb
 
     `is_causal=True` (not in the reference, which swallows extra keywords) masks k > q in both softmaxes."""
     causal = bool(kwargs.get("is_causal", False))
-    return _ffi.attn_fwd(q, k, v, scale=scale, diff=True, lambda_full=float(lambda_full),
-                         mask_kind=_ffi.MASK_CAUSAL if causal else _ffi.MASK_NONE)
+    return ops.dispatch(q, k, v, scale=scale, diff=True, lambda_full=float(lambda_full),
+                        mask_kind=_ffi.MASK_CAUSAL if causal else _ffi.MASK_NONE)
 
 
 def make_input(config, attention_name="diffattn"):

@@ -6,7 +6,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from .. import _ffi
+from .. import _ffi, ops
 
 N = 256  # number of MSA rows in the reference's benchmark inputs (evoformer.py:39)
 
@@ -66,10 +66,10 @@ def attention_reference(q_input: torch.Tensor, k_input: torch.Tensor, v_input: t
         raise ValueError("biases need equally long query and key sequences")
     kb = [_as_kernel_bias(b, lead, H, S) for b in bl]
 
-    out = torch.empty((*lead, S, H, Dv), dtype=torch.bfloat16, device=q_input.device)
-    _ffi.attn_fwd(heads_first(q_input), heads_first(k_input), heads_first(v_input), scale=sm_scale, biases=kb,
-                  gate=None if gate is None else heads_first(gate), out=heads_first(out))
-    return out
+    # the result comes back as the [prod(*), H, S, Dv] view of a buffer in [prod(*), S, H, Dv] memory order
+    out = ops.dispatch(heads_first(q_input), heads_first(k_input), heads_first(v_input), scale=sm_scale, biases=kb,
+                       gate=None if gate is None else heads_first(gate), seq_major_out=True)
+    return out.transpose(1, 2).reshape(*lead, S, H, Dv)
 
 
 def make_input(config, attention_name="ipa"):

@@ -1,0 +1,90 @@
+"""The variant functions under `torch.compile`: one `flashlight_amd::attn_fwd` node per call, no graph break
+(the reference's callers wrap the same functions in `torch.compile`, benchmarks/run_flex_variants.py:118-124)."""
+import pytest
+import torch
+
+import flashlight_amd.attention_variants as A
+import flashlight_amd.ops  # noqa: F401  (registers the operator)
+
+BF = torch.bfloat16
+
+
+class _Stop(Exception):
+    pass
+
+
+def _trace(fn, *args, **kwargs):
+    """Compiles `fn` with a backend that records the FX graph and refuses to run it (tracing needs no GPU)."""
+    graphs = []
+
+    def backend(gm, example_inputs):
+        graphs.append(gm)
+
+        def run(*a):
+            raise _Stop
+        return run
+
+    torch._dynamo.reset()
+    with pytest.raises(_Stop):
+        torch.compile(fn, backend=backend, fullgraph=True)(*args, **kwargs)
+    assert len(graphs) == 1, "one graph, no break"
+    return [n for n in graphs[0].graph.nodes if n.op == "call_function" and n.target is torch.ops.flashlight_amd.attn_fwd.default]
+
+
+def _qkv(B=1, Hq=4, Hkv=2, S=64, D=64):
+    g = torch.Generator().manual_seed(0)
+    return (torch.randn(B, Hq, S, D, generator=g).to(BF), torch.randn(B, Hkv, S, D, generator=g).to(BF),
+            torch.randn(B, Hkv, S, D, generator=g).to(BF))
+
+
+CASES = {
+    "vanilla": lambda q, k, v: A.attention_pytorch(q, k, v, enable_gqa=True),
+    "causal": lambda q, k, v: A.attention_pytorch_causal(q, k, v, enable_gqa=True),
+    "sliding": lambda q, k, v: A.attention_pytorch_sliding_window(q, k, v, window_size=16, enable_gqa=True),
+    "prefix": lambda q, k, v: A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=8, enable_gqa=True),
+    "alibi": lambda q, k, v: A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(q.size(-3)), enable_gqa=True),
+    "softcap": lambda q, k, v: A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(30.0), enable_gqa=True),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_variant_traces_into_one_operator(name):
+    nodes = _trace(CASES[name], *_qkv())
+    assert len(nodes) == 1
+    assert tuple(nodes[0].meta["example_value"].shape) == (1, 4, 64, 64)
+
+
+def test_document_diff_and_evoformer_trace():
+    q, k, v = _qkv()
+    ids = torch.arange(64).div(20, rounding_mode="floor")[None]
+    assert len(_trace(lambda q, k, v, ids: A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True), q, k, v, ids)) == 1
+    qd, kd, _ = _qkv(Hq=4, Hkv=4)
+    vd = torch.randn(1, 2, 64, 128).to(BF)
+    nodes = _trace(lambda q, k, v: A.diffattn(q, k, v, lambda_full=0.5, is_causal=True), qd, kd, vd)
+    assert len(nodes) == 1 and tuple(nodes[0].meta["example_value"].shape) == (1, 2, 64, 128)
+    Q, K, V, G = (torch.randn(1, 3, 40, 2, 32).to(BF) for _ in range(4))
+    pair, mask = torch.randn(1, 1, 2, 40, 40).to(BF), torch.randn(1, 3, 1, 1, 40).to(BF)
+    nodes = _trace(lambda Q, K, V, m, p, G: A.attention_reference(Q, K, V, [m, p], gate=G), Q, K, V, mask, pair, G)
+    assert len(nodes) == 1
+    # [prod(*), H, S, D] view of a [prod(*), S, H, D] buffer
+    val = nodes[0].meta["example_value"]
+    assert tuple(val.shape) == (3, 2, 40, 32) and val.stride() == (40 * 2 * 32, 32, 2 * 32, 1)
+
+
+@pytest.mark.gpu
+def test_compiled_equals_eager_on_gpu():
+    dev = "cuda"
+    q, k, v = (t.to(dev) for t in _qkv(B=2, Hq=8, Hkv=2, S=300, D=64))
+    for name, fn in CASES.items():
+        torch._dynamo.reset()
+        got = torch.compile(fn, backend="aot_eager", fullgraph=True)(q, k, v)
+        assert torch.equal(got, fn(q, k, v)), name
+    Q, K, V, G = (torch.randn(1, 3, 104, 2, 32, device=dev).to(BF) for _ in range(4))
+    pair, mask = torch.randn(1, 1, 2, 104, 104, device=dev).to(BF), torch.randn(1, 3, 1, 1, 104, device=dev).to(BF)
+    fn = lambda Q, K, V, m, p, G: A.attention_reference(Q, K, V, [m, p], gate=G)
+    torch._dynamo.reset()
+    got = torch.compile(fn, backend="aot_eager", fullgraph=True)(Q, K, V, mask, pair, G)
+    want = fn(Q, K, V, mask, pair, G)
+    assert got.shape == want.shape and torch.equal(got, want)
+    torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd.default,
+                          (q, k, v, -1.0, 1, 0, 0, None, 0, 0.0, None, 1, None, 1, None, False, 0.0, False))

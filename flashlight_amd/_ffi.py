@@ -53,6 +53,7 @@ class FlashlightError(RuntimeError):
 
 
 _lib: Optional[C.CDLL] = None
+_MAX_DV_DIFF = 128  # widest value slab of a differential-attention kernel instance
 
 
 def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
@@ -166,6 +167,16 @@ def attn_fwd(
         out = torch.empty((B, Hq, Lq, Dv), dtype=torch.bfloat16, device=q.device)
     elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != torch.bfloat16 or out.device != q.device:
         raise ValueError("out has the wrong shape, dtype or device")
+    if diff and Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None:
+        # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,
+        # so wide values go in slabs of _MAX_DV_DIFF columns, one launch each, through strided views of v and out
+        # (the reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38).
+        for c in range(0, Dv, _MAX_DV_DIFF):
+            attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
+                     doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
+                     gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
+                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
+        return out
 
     p = FlAttnParams()
     p.q, p.k, p.v, p.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()

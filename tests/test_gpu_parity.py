@@ -157,11 +157,15 @@ def test_reference_script_gqa():                   # tests/test_gqa.py:69-96 (ba
     assert_script_tolerance(out, O.attention_vanilla(*f32(q, k, v), enable_gqa=True, q_block=1024), "gqa")
 
 
-def test_reference_script_diffattn():              # tests/test_diffattn.py:20-41 uses head_dim 128 / value dim 256,
-    # which has no kernel instance yet; the benchmark's head_dim 64 / value dim 128 shape is checked instead
+def test_reference_script_diffattn():              # tests/test_diffattn.py:20-41: head_dim 128, value dim 256
+    # (batch 4 instead of 16 to keep the fp32 oracle small); the 256 value columns go through two launches
+    q, k, v = qkv(4, 16, 16, 1024, 128, Dv=256, seed=7, lo_hi=(-9, 9))
+    v = v[:, :8].contiguous()
+    assert_script_tolerance(A.diffattn(q, k, v), O.diff_attention(*f32(q, k, v)), "diffattn 128/256")
+    # the benchmark's other shape: head_dim 64, value dim 128 (diff_attn.py:33-38 with nheads = 32)
     q, k, v = qkv(4, 16, 16, 1024, 64, Dv=128, seed=7, lo_hi=(-9, 9))
     v = v[:, :8].contiguous()
-    assert_script_tolerance(A.diffattn(q, k, v), O.diff_attention(*f32(q, k, v)), "diffattn")
+    assert_script_tolerance(A.diffattn(q, k, v), O.diff_attention(*f32(q, k, v)), "diffattn 64/128")
 
 
 def test_reference_script_evoformer():             # tests/test_evoattn.py:21-71 (randn inputs, batch 2)

@@ -18,6 +18,7 @@ LIB_PATH = Path(os.environ.get("FL_LIB") or Path(__file__).resolve().parent / LI
 
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING, MASK_PREFIX_LM, MASK_DOCUMENT, MASK_DOCUMENT_CAUSAL = range(6)
 FL_BF16 = 0
+FL_F32 = 1
 ABI_VERSION = 1
 
 
@@ -40,7 +41,8 @@ class FlAttnParams(C.Structure):
         ("dtype", C.c_int32),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
         ("attended_dump", C.c_void_p),
-        ("reserved", C.c_int32 * 8),
+        ("bias_dtype", C.c_int32 * 2),
+        ("reserved", C.c_int32 * 6),
     ]
 
 
@@ -141,8 +143,8 @@ def attn_fwd(
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
-    `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, broadcastable to [B/batch_div, Hq, Lq, Lk]
-    (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
+    `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, bf16 or fp32, broadcastable to
+    [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -202,7 +204,10 @@ def attn_fwd(
     if len(biases) > 2:
         raise ValueError("at most two additive biases are supported")
     for i, (b, div) in enumerate(biases):
-        _require_gpu_bf16(f"bias[{i}]", b)
+        if b.dtype == torch.float32 and b.is_cuda:
+            p.bias_dtype[i] = FL_F32
+        else:
+            _require_gpu_bf16(f"bias[{i}]", b)
         if b.dim() != 4:
             raise ValueError(f"bias[{i}] must be 4-D, got {tuple(b.shape)}")
         want = (B // div, Hq, Lq, Lk)

@@ -14,3 +14,4 @@ from .prefix_lm import attention_pytorch_prefix_lm, get_prefix_lm_mask  # noqa: 
 from .document_mask import attention_pytorch_document_mask, create_document_id  # noqa: F401
 from .diff_attn import diffattn  # noqa: F401
 from .evoformer import attention_reference  # noqa: F401
+from .ipa import invariant_point_attention  # noqa: F401

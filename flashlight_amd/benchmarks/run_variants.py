@@ -148,10 +148,11 @@ def write_results_csv(rows: List[tuple], path: str) -> None:
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer"), default="variants",
+    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer", "ipa"), default="variants",
                     help="variants: run_flex_variants.py; diffattn: run_diff_attn.py (model dim 2048, head dims 64 and "
                          "128, published FLOP estimate 8 B S^2 H D); evoformer: run_evoformer.py (N_seq = S = 256, 4 "
-                         "heads, mask bias + pair bias, FLOPs 4 B 256 S^2 H D)")
+                         "heads, mask bias + pair bias, FLOPs 4 B 256 S^2 H D); ipa: invariant point attention of "
+                         "tests/test_ipa.py at 12 heads x (16 scalar + 4 query/key points + 8 value points)")
     ap.add_argument("--filter", type=str, nargs="+", default=[], help="keywords of variants to benchmark")
     ap.add_argument("--batch_size", type=int, nargs="+", default=DEFAULTS["batch_sizes"])
     ap.add_argument("--seqlen", type=int, nargs="+", default=DEFAULTS["seq_lengths"])
@@ -164,7 +165,7 @@ def parse_args(argv=None):
     if a.dim is None:
         a.dim = DEFAULTS["model_dim"] if a.suite == "variants" else 2048
     if a.headdim is None:
-        a.headdim = DEFAULTS["head_dims"] if a.suite == "variants" else [64, 128]
+        a.headdim = DEFAULTS["head_dims"] if a.suite == "variants" else [16] if a.suite == "ipa" else [64, 128]
     return a
 
 
@@ -201,6 +202,8 @@ def main(argv=None) -> List[tuple]:
 
 def _run_other_suite(args) -> List[tuple]:
     """run_diff_attn.py:42-82 / run_evoformer.py:40-82 with this package's kernels as the only implementation."""
+    import torch
+
     from flashlight_amd import attention_variants as A
     from flashlight_amd._ffi import FlashlightError
 
@@ -213,6 +216,19 @@ def _run_other_suite(args) -> List[tuple]:
                 flops = 8 * batch * seqlen ** 2 * nheads * headdim  # the reference's estimate ("double vanilla"); 6 is exact
                 inputs = A.diff_attn.make_input(config)
                 name, fn = "diffattn", lambda: A.diffattn(*inputs)
+            elif args.suite == "ipa":
+                # not swept by the reference (tests/test_ipa.py runs one shape once): AlphaFold's structure-module head
+                # layout, 12 heads of 16 scalar channels, 4 query/key points and 8 value points, `seqlen` residues;
+                # FLOPs count both products over the channels that carry data (16 + 12 and 16 + 24), launch and the
+                # concatenation of scalar and point channels included in the time
+                nheads, c, pq, pv = 12, 16, 4, 8
+                config = (batch, seqlen, nheads, c, 1, args.dropout_p)
+                flops = 2 * batch * nheads * seqlen ** 2 * ((c + 3 * pq) + (c + 3 * pv))
+                mk = lambda *shape: torch.randn(*shape, dtype=torch.bfloat16, device="cuda")  # noqa: E731
+                inputs = (mk(batch, nheads, seqlen, c), mk(batch, nheads, seqlen, c), mk(batch, nheads, seqlen, c),
+                          mk(batch, nheads, seqlen, pq, 3), mk(batch, nheads, seqlen, pq, 3),
+                          mk(batch, nheads, seqlen, pv, 3), mk(batch, nheads, seqlen, seqlen))
+                name, fn = "ipa", lambda: A.invariant_point_attention(*inputs, c_hidden=c, no_qk_points=pq)
             else:
                 seqlen, nheads = 256, 4
                 config = (batch, seqlen, nheads, headdim, 1, args.dropout_p)

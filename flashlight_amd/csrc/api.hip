@@ -131,7 +131,7 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if ((rc = check_strides("q", p->q_strides, 8)) || (rc = check_strides("k", p->k_strides, 8)) ||
       (rc = check_strides("v", p->v_strides, 8)) || (rc = check_strides("o", p->o_strides, 4)))
     return rc;
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < 6; ++i)
     if (p->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
 
   switch (p->mask_kind) {
@@ -157,7 +157,11 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if (!(p->softcap >= 0.f) || !std::isfinite(p->softcap)) return fail(FL_ERR_ARG, "softcap must be finite and >= 0");
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb]) continue;
-    if (reinterpret_cast<uintptr_t>(p->bias[nb]) % 2) return fail(FL_ERR_ALIGN, "bias[%d] must be 2-byte aligned", nb);
+    if (p->bias_dtype[nb] != FL_BF16 && p->bias_dtype[nb] != FL_F32)
+      return fail(FL_ERR_UNSUPPORTED, "bias_dtype[%d]=%d is not supported (bf16 or fp32)", nb, p->bias_dtype[nb]);
+    const int esz = p->bias_dtype[nb] == FL_F32 ? 4 : 2;
+    if (reinterpret_cast<uintptr_t>(p->bias[nb]) % esz)
+      return fail(FL_ERR_ALIGN, "bias[%d] must be %d-byte aligned", nb, esz);
     if (p->bias_batch_div[nb] <= 0) return fail(FL_ERR_ARG, "bias_batch_div[%d] must be >= 1", nb);
     for (int i = 0; i < 4; ++i)
       if (p->bias_strides[nb][i] < 0) return fail(FL_ERR_STRIDE, "bias[%d]: negative stride", nb);
@@ -278,7 +282,10 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   for (int nb = 0; nb < 2; ++nb) {
     kp.bias[nb] = static_cast<const fl::bf16_t*>(p->bias[nb]);
     kp.bdiv[nb] = p->bias[nb] ? p->bias_batch_div[nb] : 1;
-    bool vec = p->bias[nb] && p->bias_strides[nb][3] == 1 && reinterpret_cast<uintptr_t>(p->bias[nb]) % 8 == 0;
+    kp.bias_f32[nb] = p->bias[nb] && p->bias_dtype[nb] == FL_F32;
+    // four consecutive keys of a row in one load: 8 bytes of bf16 or 16 bytes of fp32
+    bool vec = p->bias[nb] && p->bias_strides[nb][3] == 1 &&
+               reinterpret_cast<uintptr_t>(p->bias[nb]) % (kp.bias_f32[nb] ? 16 : 8) == 0;
     for (int i = 0; i < 4; ++i) {
       kp.bs[nb][i] = p->bias_strides[nb][i];
       if (i < 3 && p->bias_strides[nb][i] % 4 != 0) vec = false;
@@ -292,7 +299,7 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   kp.bias_row = -1;
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb] || p->bias_strides[nb][3] != 1 || reinterpret_cast<uintptr_t>(p->bias[nb]) % 16 != 0) continue;
-    if (p->Lk % 8 != 0) continue;
+    if (p->Lk % 8 != 0 || kp.bias_f32[nb]) continue;
     bool ok = true;
     for (int i = 0; i < 3; ++i) ok = ok && p->bias_strides[nb][i] % 8 == 0;
     // per-lane byte offsets inside one (batch, head) slice are 32-bit

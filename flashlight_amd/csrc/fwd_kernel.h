@@ -69,7 +69,8 @@ struct KParams {
   const bf16_t* bias[2];
   int64_t bs[2][4];
   int32_t bdiv[2];
-  int32_t bias_vec[2];  // rows of this bias may be read 4 keys (8 bytes) at a time
+  int32_t bias_vec[2];  // rows of this bias may be read 4 keys at a time (8-byte pieces of bf16, 16-byte of fp32)
+  int32_t bias_f32[2];  // elements are fp32 instead of bf16 (such an operand is never staged through LDS)
   int32_t bias_lds;     // index of the bias operand staged through LDS (16-byte aligned rows, Lk % 8 == 0), or -1
   int32_t bias_row;     // index of a row-broadcast bias operand staged through LDS as single rows, or -1
   const bf16_t* gate;
@@ -697,8 +698,26 @@ void fwd_kernel(const KParams p) {
                 // global memory where they are used
                 for (int nb = 0; nb < 2; ++nb) {
                   if (p.bias[nb] == nullptr || nb == nbr || nb == nbl) continue;
-                  const bf16_t* bp = p.bias[nb] + (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] +
-                                     (int64_t)head * p.bs[nb][1] + (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
+                  const int64_t boff = (int64_t)(batch / p.bdiv[nb]) * p.bs[nb][0] + (int64_t)head * p.bs[nb][1] +
+                                       (int64_t)min(qrow[qb], p.Lq - 1) * p.bs[nb][2];
+                  if (p.bias_f32[nb]) {
+                    const float* fp = reinterpret_cast<const float*>(p.bias[nb]) + boff;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                      const int key = kbase + 8 * g;
+                      if (p.bias_vec[nb] && key + 3 < p.Lk) {
+                        const f32x4 b4 = *reinterpret_cast<const f32x4*>(fp + key);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) bv[4 * g + e] += b4[e];
+                      } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                          if (key + e < p.Lk) bv[4 * g + e] += fp[(int64_t)(key + e) * p.bs[nb][3]];
+                      }
+                    }
+                    continue;
+                  }
+                  const bf16_t* bp = p.bias[nb] + boff;
 #pragma unroll
                   for (int g = 0; g < 4; ++g) {
                     const int key = kbase + 8 * g;

@@ -43,7 +43,7 @@ enum fl_mask_kind {
                                  benchmarks/run_flex_variants.py:86) */
 };
 
-enum fl_dtype { FL_BF16 = 0 };
+enum fl_dtype { FL_BF16 = 0, FL_F32 = 1 };
 
 /* error codes (negative) */
 #define FL_ERR_NULL (-1)
@@ -80,9 +80,10 @@ typedef struct fl_attn_params {
   int32_t alibi_heads;
   float softcap;
 
-  /* Optional additive biases (evoformer.py:26-27), bf16, logical shape [B, Hq, Lq, Lk] with
-   * strides in elements over (batch / bias_batch_div, head, q, k); a stride of 0 broadcasts; the k
-   * stride must be 1 (or 0 when Lk == 1). */
+  /* Optional additive biases (evoformer.py:26-27; the dense fp32 tensor `score_mod(L, S)` of alibi.py:26),
+   * logical shape [B, Hq, Lq, Lk] with strides in elements over (batch / bias_batch_div, head, q, k); a
+   * stride of 0 broadcasts; the k stride must be 1 (or 0 when Lk == 1).  bias_dtype (below) selects bf16
+   * (default) or fp32 elements per operand. */
   const void* bias[2];
   int64_t bias_strides[2][4];
   int32_t bias_batch_div[2];
@@ -106,7 +107,9 @@ typedef struct fl_attn_params {
    * for every (q, k) pair it attends (after tile skipping and the element predicate). */
   uint8_t* attended_dump;
 
-  int32_t reserved[8]; /* must be 0 */
+  int32_t bias_dtype[2]; /* enum fl_dtype of bias[0], bias[1]: FL_BF16 or FL_F32 */
+
+  int32_t reserved[6]; /* must be 0 */
 } fl_attn_params;
 
 /* ABI version of the loaded library (FL_ABI_VERSION it was built with). */

@@ -15,6 +15,10 @@ How each function is pinned (tests/test_oracle_pinned.py) without running the re
   diff-attn          difference of two SDPA calls; lambda = 0 == branch 0; equal branches == (1 - lambda) * SDPA
   Evoformer          SDPA on transposed inputs with the summed bias as float mask; zero bias == vanilla
   gate               elementwise sigmoid written with math.exp in a loop
+  dense score_mod    SDPA with the callable's tensor as float mask (with and without GQA)
+  IPA                pure-Python loops over queries, keys and points with math.exp at N <= 6; zero points == SDPA with
+                     the pair bias as float mask; a common translation of query and key points changes nothing;
+                     two keys at distances d1, d2 get weights in the ratio exp(w (d1^2 - d2^2))
 The committed fixtures under tests/golden/ were produced by tests/golden/make_golden.py from those library
 routines (never from this package), so they pin it from outside as well.
 """
@@ -30,6 +34,7 @@ from .attention import (  # noqa: F401
     attention_vanilla,
     attention_vanilla_nogqa,
     diff_attention,
+    invariant_point_attention,
     tanh_softcap,
 )
 from .masks import (  # noqa: F401

@@ -136,18 +136,27 @@ def attention_alibi(query, key, value, score_mod=None, attn_mask=None, dropout_p
                     enable_gqa=False, *, softcap=None, honor_causal=False, q_block=None):
     """attention_variants/alibi.py:13-33 with score_mod = generate_alibi_bias_pytorch(Hq) (alibi.py:11): adds
     slope_h * (k - q) to the scaled scores, no mask (is_causal is ignored by the reference).  `score_mod` here is the
-    number of heads the slopes are generated for (None = query heads).  Extensions: softcap (applied to the scaled
+    number of heads the slopes are generated for (None = query heads), or a callable (L, S) -> dense tensor.  Extensions: softcap (applied to the scaled
     score before the bias), honor_causal (mask k > q with -inf when is_causal is set)."""
     hq = query.size(1)
-    slopes = alibi_slopes(hq if score_mod is None else int(score_mod), device=query.device).to(torch.float32)
     q, k, v = _group(query, key, value, enable_gqa)
+    masked = (lambda qi, ki: ki > qi) if (honor_causal and is_causal) else None
+    if callable(score_mod):
+        # any other callable: its dense result is converted to the scores' dtype and, under GQA, viewed as
+        # [Hkv, G, L, S] (alibi.py:26-29)
+        dense = score_mod(query.size(-2), key.size(-2)).to(q.dtype)
+        if enable_gqa:
+            dense = dense.view(q.size(1), q.size(2), query.size(-2), key.size(-2))
+        return _softmax_attention(q, k, v, _default_scale(query, scale), softcap=softcap, masked=masked, fill=NEG_INF,
+                                  bias=lambda qi, ki: dense if dense.size(-2) == 1 else dense[..., qi.view(-1), :],
+                                  q_block=q_block)
+    slopes = alibi_slopes(hq if score_mod is None else int(score_mod), device=query.device).to(torch.float32)
     head_shape = (q.size(1), q.size(2), 1, 1) if enable_gqa else (hq, 1, 1)  # alibi.py:27-28
 
     def bias(qi, ki):
         rel = (ki.to(torch.int32) - qi.to(torch.int32))
         return (slopes.view(-1, 1, 1) * rel).to(q.dtype).reshape(*head_shape[:-2], qi.numel(), ki.numel())
 
-    masked = (lambda qi, ki: ki > qi) if (honor_causal and is_causal) else None
     return _softmax_attention(q, k, v, _default_scale(query, scale), bias=bias, softcap=softcap, masked=masked,
                               fill=NEG_INF, q_block=q_block)
 
@@ -204,3 +213,24 @@ def attention_evoformer(q_input, k_input, v_input, biases: Sequence[torch.Tensor
     if gate is not None:
         out = out * torch.sigmoid(gate.to(out.dtype))
     return out
+
+
+# ---- invariant point attention ------------------------------------------------------------------------------------------------
+
+def invariant_point_attention(q_scalar, k_scalar, v_scalar, q_points, k_points, v_points, pair_bias, frames=None,
+                              mask=None, c_hidden=64, no_qk_points=8):
+    """tests/test_ipa.py:57-125.  Scalars [*, H, N, C], points [*, H, N, P, X].  The frame transforms and the mask are
+    commented out in the reference (test_ipa.py:84-86, 111-112, 122), so `frames` and `mask` are unused.  Returns the
+    two aggregations (output_scalar [*, H, N, C], output_points [*, N, H, Pv, X]) of test_ipa.py:117-122 instead of
+    their sum (test_ipa.py:125), which does not broadcast for general sizes."""
+    content = torch.matmul(q_scalar / (c_hidden ** 0.5), k_scalar.transpose(-1, -2))     # test_ipa.py:88-100
+    diff = q_points.unsqueeze(-3) - k_points.unsqueeze(-4)                               # [*, H, Nq, Nk, P, X]
+    dist_sq = (diff ** 2).sum(dim=-1)                                                    # test_ipa.py:102-105
+    weight = -0.5 * (9.0 / (2 * no_qk_points)) ** 0.5                                    # test_ipa.py:107
+    logits = content + dist_sq.sum(dim=-1) * weight
+    if pair_bias is not None:
+        logits = logits + pair_bias                                                      # test_ipa.py:110
+    attn = torch.softmax(logits, dim=-1)
+    out_scalar = torch.matmul(attn, v_scalar)                                            # test_ipa.py:118
+    out_points = torch.einsum('...hij,...hjpv->...ihpv', attn, v_points)                 # test_ipa.py:122
+    return out_scalar, out_points

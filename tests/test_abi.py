@@ -96,6 +96,10 @@ def test_plan_reports_launch_shape(lib):
     (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 0)), -5, "bias_batch_div"),
     (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 1),
                 p.bias_strides[0].__setitem__(3, 2)), -3, "key stride"),
+    (lambda p: (p.bias.__setitem__(1, 0x60000), p.bias_batch_div.__setitem__(1, 1),
+                p.bias_dtype.__setitem__(1, 2)), -4, "bias_dtype"),
+    (lambda p: (p.bias.__setitem__(0, 0x60002), p.bias_batch_div.__setitem__(0, 1),
+                p.bias_dtype.__setitem__(0, _ffi.FL_F32)), -7, "4-byte aligned"),
     (lambda p: setattr(p, "gate", 0x70004), -7, "gate"),
 ])
 def test_invalid_arguments_are_rejected_without_a_launch(lib, mutate, code, word):
@@ -138,7 +142,9 @@ def test_front_end_refuses_cpu_and_fp32_tensors(lib):
     q = torch.randn(1, 2, 16, 64)
     with pytest.raises(NotImplementedError, match="no CPU path"):
         attention_pytorch_causal(q.bfloat16(), q.bfloat16(), q.bfloat16())
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError, match="no CPU path"):
+        attention_pytorch_alibi(q.bfloat16(), q.bfloat16(), q.bfloat16(), score_mod=lambda a, b: torch.zeros(a, b))
+    with pytest.raises(TypeError, match="return a tensor"):
         attention_pytorch_alibi(q, q, q, score_mod=lambda a, b: None)
     with pytest.raises(TypeError):
         attention_pytorch_alibi(q, q, q)

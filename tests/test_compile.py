@@ -71,6 +71,21 @@ def test_document_diff_and_evoformer_trace():
     assert tuple(val.shape) == (3, 2, 40, 32) and val.stride() == (40 * 2 * 32, 32, 2 * 32, 1)
 
 
+def test_dense_score_mod_and_ipa_trace():
+    q, k, v = _qkv(Hq=4, Hkv=4)
+    dense = torch.randn(4, 64, 64)
+    nodes = _trace(lambda q, k, v, d: A.attention_pytorch_alibi(q, k, v, score_mod=lambda l, s: d, is_causal=True), q, k, v, dense)
+    assert len(nodes) == 1 and nodes[0].args[10].meta["example_value"].dtype == torch.float32  # bias0 stays fp32
+    r = lambda *s: torch.randn(*s).to(BF)  # noqa: E731
+    args = (r(2, 4, 48, 16), r(2, 4, 48, 16), r(2, 4, 48, 16), r(2, 4, 48, 4, 3), r(2, 4, 48, 4, 3), r(2, 4, 48, 8, 3),
+            r(2, 4, 48, 48))
+    nodes = _trace(lambda *a: A.invariant_point_attention(*a, c_hidden=16, no_qk_points=4), *args)
+    assert len(nodes) == 1
+    # scalar and point channels of q/k padded from 28 to 32, of v from 40 to 64
+    assert tuple(nodes[0].args[0].meta["example_value"].shape) == (2, 4, 48, 32)
+    assert tuple(nodes[0].meta["example_value"].shape) == (2, 4, 48, 64)
+
+
 @pytest.mark.gpu
 def test_compiled_equals_eager_on_gpu():
     dev = "cuda"

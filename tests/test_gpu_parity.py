@@ -327,3 +327,82 @@ def test_reference_free_weights_survive_extreme_logit_ranges(D, offsets):
     q, k, v = (t.bfloat16().to(DEV) for t in (q, k, v))
     assert_parity(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v)), "vanilla")
     assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(*f32(q, k, v), enable_gqa=True), "causal")
+
+
+# ---- dense score_mod and invariant point attention -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("gqa", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_dense_score_mod_matches_the_in_kernel_alibi_and_the_oracle(D, gqa):
+    # an untagged callable that returns the reference's dense fp32 ALiBi tensor (alibi.py:5-9) must give what the
+    # in-kernel ALiBi term gives; S = 333 leaves the fp32 rows unaligned for vector loads on odd rows
+    B, Hq, Hkv, S = 2, 8, (2 if gqa else 8), 333
+    q, k, v = qkv(B, Hq, Hkv, S, D, seed=5)
+    dense = lambda l, s: A.alibi_bias(Hq, l, s, device=DEV)  # noqa: E731
+    out = A.attention_pytorch_alibi(q, k, v, score_mod=dense, enable_gqa=gqa)
+    tagged = A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(Hq), enable_gqa=gqa)
+    ref = O.attention_alibi(*f32(q, k, v), score_mod=Hq, enable_gqa=gqa)
+    assert out.shape == tagged.shape == ref.shape
+    assert_parity(out, ref, "dense fp32")
+    assert (out.float() - tagged.float()).abs().max().item() <= 2e-2  # one bf16 step of an output near 2
+    # 16-byte aligned fp32 rows (vector loads), bf16 tensor through the staged path, and is_causal
+    S = 256
+    q, k, v = qkv(B, Hq, Hkv, S, D, seed=6)
+    g = torch.Generator().manual_seed(8)
+    t32 = torch.randn(Hq, S, S, generator=g).to(DEV)
+    for t in (t32, t32.bfloat16(), t32[:, :1], t32[:, :1].bfloat16(), t32[:1]):
+        full = t.expand(Hq, S, S).contiguous()
+        # under GQA the reference views the tensor as [Hkv, G, L, S], which needs every element; without GQA the
+        # size-1 axes broadcast
+        given = full if gqa else t
+        out = A.attention_pytorch_alibi(q, k, v, score_mod=lambda l, s: given, enable_gqa=gqa, is_causal=True)
+        ref = O.attention_alibi(*f32(q, k, v), score_mod=lambda l, s: full.float(), enable_gqa=gqa, is_causal=True,
+                                honor_causal=True)
+        assert_parity(out, ref, f"dense {t.dtype} {tuple(t.shape)}")
+
+
+def _ipa_inputs(B, H, N, C, P, Pv, X, seed, spread=1.0, centre=0.0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g)  # noqa: E731
+    t = dict(q_scalar=mk(B, H, N, C), k_scalar=mk(B, H, N, C), v_scalar=mk(B, H, N, C),
+             q_points=mk(B, H, N, P, X) * spread + centre, k_points=mk(B, H, N, P, X) * spread + centre,
+             v_points=mk(B, H, N, Pv, X), pair_bias=mk(B, H, N, N))
+    return {n: x.bfloat16().to(DEV) for n, x in t.items()}
+
+
+@pytest.mark.parametrize("shape", [
+    dict(B=2, H=8, N=64, C=16, P=4, Pv=8, X=4),    # tests/test_ipa.py:141-157: Dqk = 32, Dv = 48 -> 64
+    dict(B=1, H=12, N=384, C=16, P=4, Pv=8, X=3),  # AlphaFold's structure module: Dqk = 28 -> 32, Dv = 40 -> 64
+    dict(B=2, H=4, N=203, C=32, P=8, Pv=12, X=3),  # Dqk = 56 -> 64, Dv = 68 -> 128, ragged length
+    dict(B=1, H=2, N=130, C=64, P=8, Pv=8, X=3),   # Dqk = 88 -> 128, Dv = 88 -> 128
+])
+def test_invariant_point_attention(shape):
+    t = _ipa_inputs(**shape, seed=61)
+    o_s, o_p = A.invariant_point_attention(**t, c_hidden=shape["C"], no_qk_points=shape["P"])
+    r_s, r_p = O.invariant_point_attention(**{n: x.float() for n, x in t.items()}, c_hidden=shape["C"],
+                                           no_qk_points=shape["P"])
+    assert o_s.shape == r_s.shape and o_p.shape == r_p.shape
+    # the reference's own bar (tests/test_ipa.py:195) and this suite's
+    torch.testing.assert_close(o_s.float(), r_s, atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(o_p.float(), r_p, atol=1e-2, rtol=1e-2)
+    assert_parity(o_s, r_s, "scalar")
+    assert_parity(o_p, r_p, "points")
+
+
+def test_invariant_point_attention_far_from_the_origin_and_broadcast_bias():
+    # point clouds centred 40 units from the origin: |q|^2 + |k|^2 - 2 q.k loses nothing as long as the inputs enter
+    # the product unrounded and the key term stays fp32; pair bias shared by the batch; extra leading axis; no bias
+    t = _ipa_inputs(B=2, H=4, N=96, C=16, P=4, Pv=8, X=3, seed=67, spread=0.5, centre=40.0)
+    t["pair_bias"] = t["pair_bias"][:1]
+    o_s, o_p = A.invariant_point_attention(**t, c_hidden=16, no_qk_points=4)
+    r_s, r_p = O.invariant_point_attention(**{n: x.double() for n, x in t.items()}, c_hidden=16, no_qk_points=4)
+    assert_parity(o_s, r_s, "scalar, far")
+    assert_parity(o_p, r_p, "points, far")
+    t5 = {n: x.unsqueeze(0) for n, x in _ipa_inputs(B=2, H=2, N=40, C=16, P=4, Pv=8, X=3, seed=68).items()}
+    t5["pair_bias"] = None
+    o_s, o_p = A.invariant_point_attention(**t5, c_hidden=16, no_qk_points=4)
+    r_s, r_p = O.invariant_point_attention(**{n: None if x is None else x.float() for n, x in t5.items()}, c_hidden=16,
+                                           no_qk_points=4)
+    assert o_s.shape == r_s.shape == (1, 2, 2, 40, 16) and o_p.shape == r_p.shape == (1, 2, 40, 2, 8, 3)
+    assert_parity(o_s, r_s, "scalar, 5-D")
+    assert_parity(o_p, r_p, "points, 5-D")

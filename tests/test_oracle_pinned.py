@@ -151,3 +151,92 @@ def test_row_blocks_do_not_change_results():
                lambda **kw: O.attention_alibi(q, k, v, score_mod=2, softcap=3.0, **kw)):
         assert torch.equal(fn(), fn(q_block=50))
         assert torch.allclose(fn(), fn(q_block=16), atol=1e-6)
+
+
+# ---- dense score_mod (alibi.py:26-29 with an arbitrary callable) -----------------------------------------------------------
+
+@pytest.mark.parametrize("gqa", [False, True])
+def test_dense_score_mod_against_sdpa(gqa):
+    g = torch.Generator().manual_seed(31)
+    N, Hq, Hkv, L, E = 2, 4, (2 if gqa else 4), 9, 8
+    q = torch.randn(N, Hq, L, E, generator=g, dtype=torch.float64)
+    k = torch.randn(N, Hkv, L, E, generator=g, dtype=torch.float64)
+    v = torch.randn(N, Hkv, L, E, generator=g, dtype=torch.float64)
+    dense = torch.randn(Hq, L, L, generator=g, dtype=torch.float64)
+    out = O.attention_alibi(q, k, v, score_mod=lambda l, s: dense, enable_gqa=gqa)
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=dense, enable_gqa=gqa)
+    if gqa:
+        assert tuple(out.shape) == (N, Hkv, Hq // Hkv, L, E)
+    assert (out.reshape(N, Hq, L, E) - ref).abs().max().item() < 1e-12
+
+
+# ---- invariant point attention (tests/test_ipa.py:57-125) ------------------------------------------------------------------
+
+def _ipa_inputs(seed, B=1, H=2, N=5, C=4, P=3, Pv=2, X=3, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=dtype)  # noqa: E731
+    return dict(q_scalar=r(B, H, N, C), k_scalar=r(B, H, N, C), v_scalar=r(B, H, N, C), q_points=r(B, H, N, P, X),
+                k_points=r(B, H, N, P, X), v_points=r(B, H, N, Pv, X), pair_bias=r(B, H, N, N))
+
+
+def test_ipa_bruteforce_loops():
+    a = _ipa_inputs(41, B=2, H=2, N=6, C=4, P=3, Pv=2, X=3)
+    c_hidden, P = 4, 3
+    o_s, o_p = O.invariant_point_attention(**a, c_hidden=c_hidden, no_qk_points=P)
+    B, H, N, C = a["q_scalar"].shape
+    Pv, X = a["v_points"].shape[-2:]
+    assert tuple(o_s.shape) == (B, H, N, C) and tuple(o_p.shape) == (B, N, H, Pv, X)
+    for b in range(B):
+        for h in range(H):
+            for i in range(N):
+                logits = []
+                for j in range(N):
+                    dot = sum(float(a["q_scalar"][b, h, i, c]) * float(a["k_scalar"][b, h, j, c]) for c in range(C))
+                    d2 = 0.0
+                    for p in range(P):
+                        for x in range(X):
+                            d2 += (float(a["q_points"][b, h, i, p, x]) - float(a["k_points"][b, h, j, p, x])) ** 2
+                    logits.append(dot / math.sqrt(c_hidden) - 0.5 * math.sqrt(9.0 / (2 * P)) * d2 +
+                                  float(a["pair_bias"][b, h, i, j]))
+                m = max(logits)
+                wts = [math.exp(x - m) for x in logits]
+                z = sum(wts)
+                for c in range(C):
+                    want = sum(wts[j] / z * float(a["v_scalar"][b, h, j, c]) for j in range(N))
+                    assert abs(float(o_s[b, h, i, c]) - want) < 1e-10
+                for p in range(Pv):
+                    for x in range(X):
+                        want = sum(wts[j] / z * float(a["v_points"][b, h, j, p, x]) for j in range(N))
+                        assert abs(float(o_p[b, i, h, p, x]) - want) < 1e-10
+
+
+def test_ipa_identities():
+    a = _ipa_inputs(43, B=2, H=3, N=7, C=8, P=4, Pv=3, X=4)
+    # no points: plain attention with the pair bias as float mask and scale 1/sqrt(c_hidden)
+    z = dict(a, q_points=torch.zeros_like(a["q_points"]), k_points=torch.zeros_like(a["k_points"]))
+    o_s, o_p = O.invariant_point_attention(**z, c_hidden=16, no_qk_points=4)
+    ref = F.scaled_dot_product_attention(a["q_scalar"], a["k_scalar"], a["v_scalar"], attn_mask=a["pair_bias"],
+                                         scale=1 / 4.0)
+    assert (o_s - ref).abs().max().item() < 1e-12
+    vp = a["v_points"].flatten(-2)
+    refp = F.scaled_dot_product_attention(a["q_scalar"], a["k_scalar"], vp, attn_mask=a["pair_bias"], scale=1 / 4.0)
+    assert (o_p.transpose(1, 2).flatten(-2) - refp).abs().max().item() < 1e-12
+    # distances only see differences: moving every query and key point by the same vector changes nothing
+    shift = torch.tensor([0.7, -1.3, 2.1, 0.4], dtype=torch.float64)
+    s = dict(a, q_points=a["q_points"] + shift, k_points=a["k_points"] + shift)
+    o1 = O.invariant_point_attention(**a, c_hidden=16, no_qk_points=4)
+    o2 = O.invariant_point_attention(**s, c_hidden=16, no_qk_points=4)
+    assert (o1[0] - o2[0]).abs().max().item() < 1e-10 and (o1[1] - o2[1]).abs().max().item() < 1e-10
+    # one query at the origin, two keys at distances d1 and d2, nothing else: weights in the ratio exp(w (d1^2 - d2^2))
+    for P in (1, 4, 8):
+        w = -0.5 * math.sqrt(9.0 / (2 * P))
+        d1, d2 = 0.5, 1.25
+        qp = torch.zeros(1, 1, 1, 1, 3, dtype=torch.float64)
+        kp = torch.zeros(1, 1, 2, 1, 3, dtype=torch.float64)
+        kp[0, 0, 0, 0, 0], kp[0, 0, 1, 0, 2] = d1, d2
+        zero = torch.zeros(1, 1, 1, 2, dtype=torch.float64)
+        vs = torch.tensor([[1.0, 0.0], [0.0, 1.0]], dtype=torch.float64).view(1, 1, 2, 2)
+        o_s, _ = O.invariant_point_attention(zero[..., :1, :], torch.zeros(1, 1, 2, 2, dtype=torch.float64), vs, qp, kp,
+                                             torch.zeros(1, 1, 2, 1, 3, dtype=torch.float64), None, c_hidden=2,
+                                             no_qk_points=P)
+        assert abs(float(o_s[0, 0, 0, 0] / o_s[0, 0, 0, 1]) - math.exp(w * (d1 * d1 - d2 * d2))) < 1e-12

@@ -1,0 +1,662 @@
+"""Graph rewrite: eager attention written out in PyTorch -> one fused launch.
+
+The reference turns `torch.compile(fn)` of an eager attention function (matmul -> score modifications -> softmax ->
+matmul, attention_variants/*.py) into one generated kernel by patching TorchInductor
+(`from monkeypatch.fusion import ...`, tests/test_causal.py:14-17).  This module is the counterpart for callers who
+keep their own eager functions: `torch.compile(fn, backend=flashlight_amd.fusion.backend, dynamic=False)` captures the
+function with Dynamo, finds every region of that shape in the FX graph and replaces it by a call into the hand-written
+kernel (`flashlight_amd::attn_fwd`); whatever else the function does keeps running as ordinary eager PyTorch.
+
+What a region may contain, from the first matmul to the second:
+  q @ k.transpose(-2, -1)  [* scale | / scale]  [cap * tanh(x / cap)]  {+ bias | masked_fill / where(mask, fill, x)}*
+  -> softmax(dim=-1) [-> type_as / to] -> @ v
+with q/k/v of any rank >= 3 (leading axes are batch; `query.view(N, Hkv, G, L, E)` with `key.unsqueeze(2)` is
+grouped-query attention) and masks/biases broadcastable to the scores.
+
+Masks and biases are recognised by what they compute, not by how they were written:
+  * a mask that depends on no graph input is evaluated once at compile time and compared with the closed forms of the
+    kernel's positional masks (causal, sliding window, prefix-LM); anything else becomes a constant additive -inf bias;
+  * a mask that depends on one integer [N, L] input is probed with random ids and compared with the document
+    predicates (same document, optionally k <= q); anything else stays in the graph and is converted to an additive
+    bias at run time;
+  * a constant bias equal to 2^(-8 (h + 1) / H) * (k - q) is ALiBi and is computed inside the kernel; other biases are
+    passed to the kernel's bias operands (fp32 or bf16).
+Regions that do not fit (a softmax whose weights are used elsewhere, dropout with p > 0, ...) are left untouched.
+"""
+from __future__ import annotations
+
+import math
+import operator
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+import torch.fx as fx
+
+from . import _ffi, ops
+
+__all__ = ["backend", "fuse_attention", "fused_attention"]
+
+_NEG_INF = float("-inf")
+
+
+# ---- node helpers ------------------------------------------------------------------------------------------------------
+
+def _name(n: Any) -> Optional[str]:
+    """Canonical operation name of a call node: 'matmul' for torch.matmul / operator.matmul / Tensor.matmul, ..."""
+    if not isinstance(n, fx.Node):
+        return None
+    if n.op == "call_method":
+        s = n.target
+    elif n.op == "call_function":
+        s = getattr(n.target, "__name__", str(n.target))
+    else:
+        return None
+    s = s.strip("_") if s.startswith("__") else s
+    return {"imatmul": "matmul", "truediv": "div", "itruediv": "div", "iadd": "add", "imul": "mul", "add_": "add",
+            "mul_": "mul", "div_": "div", "masked_fill_": "masked_fill", "bmm": "matmul", "isub": "sub"}.get(s, s)
+
+
+def _val(n: fx.Node):
+    v = n.meta.get("example_value", n.meta.get("val"))
+    if v is None:
+        raise _NoMatch(f"no example value recorded for {n.name}")
+    return v
+
+
+def _is_number(x) -> bool:
+    return isinstance(x, (int, float)) and not isinstance(x, bool)
+
+
+class _NoMatch(Exception):
+    pass
+
+
+def _arg(n: fx.Node, i: int, kw: str, default=None):
+    if len(n.args) > i:
+        return n.args[i]
+    return n.kwargs.get(kw, default)
+
+
+def _is_last2_transpose(n: Any) -> Optional[fx.Node]:
+    """Returns x when n is x with its last two axes swapped."""
+    nm = _name(n)
+    if nm == "transpose":
+        d0, d1 = _arg(n, 1, "dim0"), _arg(n, 2, "dim1")
+        nd = _val(n.args[0]).dim()
+        if isinstance(d0, int) and isinstance(d1, int) and {d0 % nd, d1 % nd} == {nd - 1, nd - 2}:
+            return n.args[0]
+    if nm == "permute":
+        dims = n.args[1:] if len(n.args) > 2 else tuple(_arg(n, 1, "dims"))
+        nd = len(dims)
+        want = list(range(nd - 2)) + [nd - 1, nd - 2]
+        if [d % nd for d in dims] == want:
+            return n.args[0]
+    if n.op == "call_function" and n.target is getattr and n.args[1] == "mT":
+        return n.args[0]
+    return None
+
+
+def _depends_on(n: Any, target: fx.Node, memo: Dict[fx.Node, bool]) -> bool:
+    if not isinstance(n, fx.Node):
+        return False
+    if n is target:
+        return True
+    if n in memo:
+        return memo[n]
+    memo[n] = False
+    r = any(_depends_on(a, target, memo) for a in n.all_input_nodes)
+    memo[n] = r
+    return r
+
+
+def _placeholders_of(n: fx.Node) -> List[fx.Node]:
+    seen, out, stack = set(), [], [n]
+    while stack:
+        x = stack.pop()
+        if x in seen:
+            continue
+        seen.add(x)
+        if x.op == "placeholder":
+            out.append(x)
+        stack.extend(x.all_input_nodes)
+    return out
+
+
+def _evaluate(n: Any, env: Dict[fx.Node, Any], gm: fx.GraphModule):
+    """Runs the subgraph that produces `n` eagerly; `env` maps placeholders (and already computed nodes) to values."""
+    if isinstance(n, (tuple, list)):
+        return type(n)(_evaluate(x, env, gm) for x in n)
+    if isinstance(n, dict):
+        return {k: _evaluate(v, env, gm) for k, v in n.items()}
+    if isinstance(n, slice):
+        return slice(_evaluate(n.start, env, gm), _evaluate(n.stop, env, gm), _evaluate(n.step, env, gm))
+    if not isinstance(n, fx.Node):
+        return n
+    if n in env:
+        return env[n]
+    if n.op == "placeholder":
+        raise _NoMatch(f"subgraph reads graph input {n.name}")
+    args, kwargs = _evaluate(n.args, env, gm), _evaluate(n.kwargs, env, gm)
+    if n.op == "call_function":
+        r = n.target(*args, **kwargs)
+    elif n.op == "call_method":
+        r = getattr(args[0], n.target)(*args[1:], **kwargs)
+    elif n.op == "get_attr":
+        r = gm
+        for part in n.target.split("."):
+            r = getattr(r, part)
+    elif n.op == "call_module":
+        r = gm.get_submodule(n.target)(*args, **kwargs)
+    else:
+        raise _NoMatch(f"cannot evaluate {n.op}")
+    env[n] = r
+    return r
+
+
+def _try_evaluate(n: fx.Node, gm: fx.GraphModule):
+    """Value of a subgraph without graph inputs, or None when it cannot be computed at compile time."""
+    try:
+        return _evaluate(n, {}, gm)
+    except Exception:
+        return None
+
+
+# ---- what the positional masks look like (True = masked) ---------------------------------------------------------------------
+
+def _idx(L: int, S: int, device):
+    return torch.arange(L, device=device).view(L, 1), torch.arange(S, device=device).view(1, S)
+
+
+def _classify_constant_mask(m: torch.Tensor, L: int, S: int):
+    """m: bool, broadcastable to [..., L, S], True = masked.  Returns (mask_kind, window, prefix) when it equals one of the
+    kernel's positional masks on every leading index, else None."""
+    if m.dim() < 2:
+        m = m.reshape((1,) * (2 - m.dim()) + tuple(m.shape))
+    if m.size(-2) not in (1, L) or m.size(-1) not in (1, S):
+        return None
+    m = m.reshape(-1, m.size(-2), m.size(-1))
+    if m.size(0) > 1 and not bool((m == m[:1]).all()):
+        return None
+    m = m[0].expand(L, S)
+    q, k = _idx(L, S, m.device)
+    if not bool(m.any()):
+        return _ffi.MASK_NONE, 0, 0
+    if bool((m == (k > q)).all()):
+        return _ffi.MASK_CAUSAL, 0, 0
+    if L == S:
+        w = int((~m[L - 1]).sum().item()) - 1
+        if w >= 0 and bool((m == ((q < k) | ((q - k) > w))).all()):
+            return _ffi.MASK_SLIDING, w, 0
+        p = int((~m[0]).sum().item())
+        if p >= 1 and bool((m == (k > torch.clamp(q, min=p - 1))).all()):
+            return _ffi.MASK_PREFIX_LM, 0, p
+    return None
+
+
+def _classify_document_mask(node: fx.Node, ids_ph: fx.Node, invert: bool, L: int, S: int, gm: fx.GraphModule):
+    """Probes the mask subgraph, a function of one integer [N, L] input, with random ids.  Returns MASK_DOCUMENT or
+    MASK_DOCUMENT_CAUSAL when its output equals that predicate for every probe, else None."""
+    ex = _val(ids_ph)
+    if L != S or ex.dim() != 2 or ex.size(1) != L or ex.dtype not in (torch.int64, torch.int32):
+        return None
+    N, dev = ex.size(0), ex.device
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    probes = [torch.randint(0, 3, (N, L), generator=g).sort(dim=1).values,
+              torch.randint(-5, 7, (N, L), generator=g),
+              torch.zeros(N, L, dtype=torch.int64)]
+    q, k = _idx(L, S, dev)
+    verdict = None
+    for ids in probes:
+        ids = ids.to(device=dev, dtype=ex.dtype)
+        try:
+            m = _evaluate(node, {ids_ph: ids}, gm)
+        except Exception:  # the subgraph needs something a probe cannot give it
+            return None
+        if not isinstance(m, torch.Tensor) or m.dtype != torch.bool:
+            return None
+        if invert:
+            m = ~m
+        if m.dim() < 3 or m.size(0) not in (1, N):
+            return None
+        same = ids.unsqueeze(2) != ids.unsqueeze(1)                                  # [N, L, S], True = masked
+        lead = (N,) + (1,) * (m.dim() - 3)
+        ok_doc = bool((m == same.view(*lead, L, S)).all())
+        ok_causal = bool((m == (same | (k > q)).view(*lead, L, S)).all())
+        got = _ffi.MASK_DOCUMENT if ok_doc else _ffi.MASK_DOCUMENT_CAUSAL if ok_causal else None
+        if ok_doc and ok_causal:  # a probe that cannot tell the two apart
+            continue
+        if got is None or (verdict is not None and verdict != got):
+            return None
+        verdict = got
+    return verdict
+
+
+def _is_alibi(b: torch.Tensor, H: int, L: int, S: int) -> bool:
+    """b broadcastable to [H, L, S] (or [Hkv, G, L, S]) and equal to 2^(-8 (h + 1) / H) (k - q) (alibi.py:5-9)."""
+    if b.numel() != H * L * S:
+        return False
+    b = b.reshape(H, L, S).to(torch.float32)
+    slopes = torch.exp2(-8.0 * torch.arange(1, H + 1, device=b.device, dtype=torch.float32) / H)
+    q, k = _idx(L, S, b.device)
+    want = slopes.view(H, 1, 1) * (k - q).to(torch.float32)
+    return bool(((b - want).abs() <= 1e-5 * want.abs() + 1e-6).all())
+
+
+# ---- the run-time side: what the replacement node calls -----------------------------------------------------------------------
+
+def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...], L: int, S: int):
+    """Maps a tensor broadcastable to the scores [*lead, *heads, L, S] onto the kernel's ([Nb, H|1, L|1, S], batch divisor)
+    form (batch index = flat_batch // divisor), copying only when the broadcast pattern has no such form."""
+    nl, nh = len(lead), len(heads)
+    nd = nl + nh + 2
+    if b.dim() > nd:
+        raise ValueError(f"bias of shape {tuple(b.shape)} has more axes than the scores")
+    b = b.reshape((1,) * (nd - b.dim()) + tuple(b.shape))
+    for got, want in zip(b.shape, (*lead, *heads, L, S)):
+        if got not in (1, want):
+            raise ValueError(f"bias of shape {tuple(b.shape)} does not broadcast to the scores {(*lead, *heads, L, S)}")
+    if b.dtype == torch.bool:
+        raise TypeError("boolean biases are masks; use masked_fill / where")
+    if b.dtype not in (torch.bfloat16, torch.float32):
+        b = b.to(torch.float32)
+    if b.size(-1) != S:
+        b = b.expand(*b.shape[:-1], S)
+    hs = tuple(b.shape[nl:nl + nh])
+    if not (all(h == 1 for h in hs) or hs == tuple(heads)):  # e.g. full over kv heads, broadcast over the group
+        b = b.expand(*b.shape[:nl], *heads, *b.shape[nl + nh:])
+        hs = tuple(heads)
+    H = math.prod(hs)
+    bl = tuple(b.shape[:nl])
+    split = nl
+    while split > 0 and bl[split - 1] == 1:
+        split -= 1
+    if any(bl[i] != lead[i] for i in range(split)):
+        b = b.expand(*lead, *b.shape[nl:])
+        bl, split = tuple(lead), nl
+    div = math.prod(lead[split:]) if split < nl else 1
+    nb = math.prod(bl[:split]) if split else 1
+    return b.reshape(nb, H, b.shape[-2], S), int(div)
+
+
+def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: Optional[torch.Tensor],
+                    biases: Sequence[torch.Tensor], masks: Sequence[torch.Tensor], *, scale: float, mask_kind: int,
+                    window: int, prefix: int, alibi_heads: int, softcap: float, gqa: bool,
+                    mask_invert: Sequence[bool] = (), diff_lambda: Optional[float] = None) -> torch.Tensor:
+    """Target of the replacement node.  q [*lead, H, L, E] (or [N, Hkv, G, L, E] with `gqa`), k/v likewise with S keys;
+    `biases` are added to the scaled scores, `masks` (bool, True = masked unless the matching `mask_invert` entry is
+    set) are those the rewrite could not map to a positional or document mask.  Returns what the eager region
+    returned: [*q.shape[:-1], Ev].  With `diff_lambda` q and k hold the heads of both softmax branches (first half,
+    second half) and the result is branch 0 minus diff_lambda times branch 1."""
+    L, S = q.size(-2), k.size(-2)
+    result_shape = (*q.shape[:-1], v.size(-1))
+    if gqa:
+        lead, heads = (q.size(0),), (q.size(1), q.size(2))
+        q4 = q.reshape(q.size(0), -1, L, q.size(-1))
+        k4, v4 = k.squeeze(2), v.squeeze(2)
+    else:
+        if q.dim() == 3:
+            q = q.unsqueeze(1)
+        lead, heads = tuple(q.shape[:-3]), (q.size(-3),)
+
+        def like_q(t):  # key/value with missing or size-1 leading axes broadcast like matmul operands do
+            if t.dim() == 3 and len(lead) == 1:
+                t = t.unsqueeze(1)
+            t = t.reshape((1,) * (q.dim() - t.dim()) + tuple(t.shape))
+            return t if tuple(t.shape[:-3]) == lead else t.expand(*lead, *t.shape[-3:])
+
+        q4, k4, v4 = (t.reshape(-1, *t.shape[-3:]) for t in (q, like_q(k), like_q(v)))
+    kb = [_kernel_bias(b, lead, heads, L, S) for b in biases]
+    for i, m in enumerate(masks):
+        if i < len(mask_invert) and mask_invert[i]:
+            m = ~m
+        add = torch.zeros(m.shape, dtype=torch.bfloat16, device=m.device).masked_fill_(m, _NEG_INF)
+        kb.append(_kernel_bias(add, lead, heads, L, S))
+    while len(kb) > 2:  # the kernel takes two operands: fold the rest into the last one
+        (b1, d1), (b2, d2) = kb[-2], kb[-1]
+        if d1 != d2:  # different batch groupings: give both one row per flat batch index
+            b1, b2 = (b.repeat_interleave(d, dim=0) if d > 1 else b for b, d in ((b1, d1), (b2, d2)))
+            d1 = 1
+        kb[-2:] = [(b1.float() + b2.float(), d1)]
+    if diff_lambda is None:
+        out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
+                           alibi_heads=alibi_heads, softcap=softcap, biases=kb)
+        return out.reshape(result_shape)
+    out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
+                       alibi_heads=alibi_heads, softcap=softcap, biases=kb, diff=True, lambda_full=float(diff_lambda))
+    return out.reshape(*result_shape[:-3], result_shape[-3] // 2, *result_shape[-2:])
+
+
+# ---- matching ----------------------------------------------------------------------------------------------------------------
+
+class _Region:
+    def __init__(self):
+        self.nodes: List[fx.Node] = []      # interior nodes to delete, consumer first
+        self.q = self.k = self.v = None
+        self.scale = 1.0
+        self.softcap = 0.0
+        self.biases: List[fx.Node] = []
+        self.masks: List[Tuple[fx.Node, bool]] = []   # (mask node, invert)
+        self.out: Optional[fx.Node] = None
+
+
+def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
+    """Walks from the softmax input up to the q k^T matmul, recording what each step does to the scores."""
+    nm = _name(n)
+    if nm is None:
+        raise _NoMatch("scores do not come from a matmul")
+    if nm in ("to", "type_as", "float", "contiguous", "clone"):
+        r.nodes.append(n)
+        return _peel_scores(n.args[0], r, qk_memo, mods_below)
+    if nm == "matmul":
+        a, b = n.args[0], n.args[1]
+        kt = _is_last2_transpose(b)
+        if kt is None:
+            raise _NoMatch("second matmul operand is not a transposed key")
+        r.nodes.append(n)
+        if len(b.users) == 1:
+            r.nodes.append(b)
+        r.q, r.k = a, kt
+        return
+    if nm in ("where",):
+        cond, a, b = n.args[0], n.args[1], n.args[2]
+        if isinstance(b, fx.Node) and _is_number(a) and a <= -1e9:
+            r.masks.append((cond, False))
+            inner = b
+        elif isinstance(a, fx.Node) and _is_number(b) and b <= -1e9:
+            r.masks.append((cond, True))
+            inner = a
+        else:
+            raise _NoMatch("where() is not a mask fill")
+        r.nodes.append(n)
+        mods_below.append("mask")
+        return _peel_scores(inner, r, qk_memo, mods_below)
+    if nm == "masked_fill":
+        inner, cond, fill = n.args[0], _arg(n, 1, "mask"), _arg(n, 2, "value")
+        if not (_is_number(fill) and fill <= -1e9):
+            raise _NoMatch("masked_fill value is not a large negative number")
+        r.masks.append((cond, False))
+        r.nodes.append(n)
+        mods_below.append("mask")
+        return _peel_scores(inner, r, qk_memo, mods_below)
+    if nm == "add":
+        a, b = n.args[0], n.args[1]
+        if _is_number(a) or _is_number(b):
+            raise _NoMatch("scalar added to the scores")
+        a_has = _contains_qk(a, qk_memo)
+        inner, bias = (a, b) if a_has else (b, a)
+        if not a_has and not _contains_qk(b, qk_memo):
+            raise _NoMatch("add without a score operand")
+        r.biases.append(bias)
+        r.nodes.append(n)
+        mods_below.append("bias")
+        return _peel_scores(inner, r, qk_memo, mods_below)
+    if nm in ("mul", "div"):
+        a, b = n.args[0], n.args[1]
+        if nm == "mul" and _is_number(a):
+            a, b = b, a
+        if not _is_number(b) or not isinstance(a, fx.Node):
+            raise _NoMatch("scores multiplied by a tensor")
+        c = float(b) if nm == "mul" else 1.0 / float(b)
+        if _name(a) == "tanh":  # cap * tanh(x / cap)
+            t_in = a.args[0]
+            nm2 = _name(t_in)
+            if nm2 not in ("div", "mul") or not _is_number(t_in.args[1]):
+                raise _NoMatch("tanh argument is not scores / cap")
+            inv = 1.0 / float(t_in.args[1]) if nm2 == "div" else float(t_in.args[1])
+            if not (c > 0 and abs(c * inv - 1.0) < 1e-6):
+                raise _NoMatch("tanh soft-cap with mismatched constants")
+            if r.softcap or "softcap" in mods_below:
+                raise _NoMatch("two soft-caps")
+            r.softcap = c
+            r.nodes += [n, a, t_in]
+            mods_below.append("softcap")
+            return _peel_scores(t_in.args[0], r, qk_memo, mods_below)
+        if not c > 0:
+            raise _NoMatch("non-positive scale")
+        r.scale *= c
+        r.nodes.append(n)
+        mods_below.append("scale")
+        return _peel_scores(a, r, qk_memo, mods_below)
+    raise _NoMatch(f"unsupported operation on the scores: {nm}")
+
+
+def _contains_qk(n: Any, memo: Dict[fx.Node, bool]) -> bool:
+    """True when `n` is reached from a (x @ transposed y) matmul through score-chain operations only."""
+    if not isinstance(n, fx.Node):
+        return False
+    if n in memo:
+        return memo[n]
+    nm = _name(n)
+    memo[n] = False
+    if nm == "matmul" and len(n.args) >= 2 and _is_last2_transpose(n.args[1]) is not None:
+        r = True
+    elif nm in ("where", "masked_fill", "add", "mul", "div", "tanh", "to", "type_as", "float", "contiguous", "clone"):
+        r = any(_contains_qk(a, memo) for a in n.args if isinstance(a, fx.Node))
+    else:
+        r = False
+    memo[n] = r
+    return r
+
+
+def _check_order(r: _Region, order_from_softmax: List[str]):
+    """Kernel order: scale, soft-cap, then biases and masks (which commute).  Walking up from the softmax the chain must
+    therefore read (bias|mask)* softcap? scale*."""
+    stage = 0  # 0: biases/masks, 1: softcap seen, 2: scale seen
+    for what in order_from_softmax:
+        if what in ("bias", "mask"):
+            if stage != 0:
+                raise _NoMatch("a bias or mask is applied before the scale or the soft-cap")
+        elif what == "softcap":
+            if stage >= 1:
+                raise _NoMatch("soft-cap applied before the scale")
+            stage = 1
+        elif what == "scale":
+            stage = 2
+
+
+def _match(softmax: fx.Node) -> _Region:
+    dim = _arg(softmax, 1, "dim")
+    x = softmax.args[0]
+    nd = _val(softmax).dim()
+    if not isinstance(dim, int) or dim % nd != nd - 1:
+        raise _NoMatch("softmax is not over the last axis")
+    r = _Region()
+    order: List[str] = []
+    _peel_scores(x, r, {}, order)
+    _check_order(r, order)
+    # downstream: [type_as / to]* -> matmul(p, v)
+    cur = softmax
+    tail = [softmax]
+    while True:
+        if len(cur.users) != 1:
+            raise _NoMatch("the softmax weights have more than one consumer")
+        (u,) = cur.users
+        nm = _name(u)
+        if nm in ("to", "type_as", "float", "contiguous") and u.args[0] is cur:
+            tail.append(u)
+            cur = u
+            continue
+        if nm == "dropout":
+            p = _arg(u, 1, "p", 0.5)
+            if p != 0.0:
+                raise _NoMatch("dropout with p > 0")
+            tail.append(u)
+            cur = u
+            continue
+        if nm == "matmul" and u.args[0] is cur and isinstance(u.args[1], fx.Node):
+            r.v, r.out = u.args[1], u
+            tail.append(u)
+            break
+        raise _NoMatch(f"softmax weights feed {nm}, not a matmul with the values")
+    r.nodes = list(reversed(tail)) + r.nodes
+    # interior values must not escape the region
+    inside = set(r.nodes)
+    for n in r.nodes:
+        if n is r.out:
+            continue
+        for u in n.users:
+            if u not in inside:
+                raise _NoMatch(f"intermediate {n.name} is used outside the attention region")
+    return r
+
+
+def _shapes(r: _Region):
+    q, k, v = _val(r.q), _val(r.k), _val(r.v)
+    if q.dim() < 3 or k.dim() < 3 or v.dim() < 3:
+        raise _NoMatch("operands need at least [batch, seq, dim]")
+    gqa = q.dim() == 5 and k.dim() == 5 and v.dim() == 5 and k.size(2) == 1 and v.size(2) == 1 and q.size(2) > 1 and \
+        q.size(1) == k.size(1)
+    L, S = q.size(-2), k.size(-2)
+    if v.size(-2) != S or q.size(-1) != k.size(-1):
+        raise _NoMatch("inconsistent operand shapes")
+    Hq = q.size(1) * q.size(2) if gqa else (q.size(-3) if q.dim() >= 4 else 1)
+    return gqa, L, S, Hq
+
+
+def _head_half(n: Any) -> Optional[Tuple[fx.Node, int]]:
+    """(x, 0) when n is the first half of x's heads (axis 1), (x, 1) for the second half: x[:, :h], x[:, h:] or
+    torch.chunk(x, 2, dim=1)[i]."""
+    if not (isinstance(n, fx.Node) and n.op == "call_function" and n.target is operator.getitem):
+        return None
+    src, idx = n.args
+    if _name(src) == "chunk" and isinstance(idx, int):
+        if _arg(src, 1, "chunks") == 2 and _arg(src, 2, "dim", 0) in (1, 1 - _val(src.args[0]).dim()):
+            return src.args[0], idx
+        return None
+    if not isinstance(idx, tuple) or len(idx) < 2 or not isinstance(src, fx.Node):
+        return None
+    full = slice(None, None, None)
+    if any(i != full for j, i in enumerate(idx) if j != 1) or not isinstance(idx[1], slice) or idx[1].step is not None:
+        return None
+    heads = _val(src).size(1)
+    if heads % 2:
+        return None
+    if idx[1].start in (None, 0) and idx[1].stop == heads // 2:
+        return src, 0
+    if idx[1].start == heads // 2 and idx[1].stop in (None, heads):
+        return src, 1
+    return None
+
+
+def _merge_differential(gm: fx.GraphModule) -> int:
+    """attn(q[:, :h], k[:, :h], v) - lam * attn(q[:, h:], k[:, h:], v) (diff_attn.py:14-29) -> one launch that keeps both
+    softmax states and reads v once."""
+    merged = 0
+    for sub in [n for n in gm.graph.nodes if _name(n) == "sub"]:
+        if len(sub.args) != 2 or sub.kwargs.get("alpha", 1) != 1:
+            continue
+        a, m = sub.args
+        if _name(m) != "mul" or not isinstance(a, fx.Node):
+            continue
+        lam, b = (m.args[0], m.args[1]) if _is_number(m.args[0]) else (m.args[1], m.args[0])
+        if not _is_number(lam) or not isinstance(b, fx.Node):
+            continue
+        if not all(x.op == "call_function" and x.target is fused_attention for x in (a, b)):
+            continue
+        if a.kwargs != b.kwargs or a.kwargs.get("gqa") or a.kwargs.get("diff_lambda") is not None:
+            continue
+        if a.args[2] is not b.args[2] or a.args[3] is not b.args[3]:
+            continue
+        if list(a.args[4]) or list(b.args[4]) or list(a.args[5]) or list(b.args[5]):
+            continue
+        qa, qb, ka, kb = _head_half(a.args[0]), _head_half(b.args[0]), _head_half(a.args[1]), _head_half(b.args[1])
+        if None in (qa, qb, ka, kb) or qa[0] is not qb[0] or ka[0] is not kb[0] or (qa[1], qb[1], ka[1], kb[1]) != (0, 1, 0, 1):
+            continue
+        if _val(qa[0]).dim() != 4 or len(a.users) != 1 or len(b.users) != 1 or len(m.users) != 1:
+            continue
+        with gm.graph.inserting_before(sub):
+            new = gm.graph.call_function(fused_attention, (qa[0], ka[0], a.args[2], a.args[3], [], []),
+                                         dict(a.kwargs, diff_lambda=float(lam)))
+        new.meta.update(sub.meta)
+        sub.replace_all_uses_with(new)
+        for n in (sub, m, b, a):
+            gm.graph.erase_node(n)
+        merged += 1
+    return merged
+
+
+def fuse_attention(gm: fx.GraphModule) -> int:
+    """Rewrites every attention region of `gm` (a Dynamo-captured graph with example values on its nodes) in place.
+    Returns the number of regions replaced."""
+    replaced = 0
+    for sm in [n for n in gm.graph.nodes if _name(n) == "softmax"]:
+        try:
+            r = _match(sm)
+            gqa, L, S, Hq = _shapes(r)
+            kwargs: Dict[str, Any] = dict(scale=float(r.scale), mask_kind=_ffi.MASK_NONE, window=0, prefix=0,
+                                          alibi_heads=0, softcap=float(r.softcap), gqa=gqa)
+            doc_ids = None
+            run_masks: List[fx.Node] = []
+            run_invert: List[bool] = []
+            const_biases: List[torch.Tensor] = []
+            run_biases: List[fx.Node] = []
+            for node, invert in r.masks:
+                phs = _placeholders_of(node)
+                got = None
+                if not phs:
+                    m = _try_evaluate(node, gm)
+                    if not isinstance(m, torch.Tensor) or m.dtype != torch.bool:
+                        run_masks.append(node)
+                        run_invert.append(invert)
+                        continue
+                    m = ~m if invert else m
+                    got = _classify_constant_mask(m, L, S)
+                    if got is not None and got[0] != _ffi.MASK_NONE:
+                        if kwargs["mask_kind"] != _ffi.MASK_NONE:
+                            got = None  # two positional masks: keep the second one dense
+                        else:
+                            kwargs.update(mask_kind=got[0], window=got[1], prefix=got[2])
+                    if got is None:
+                        const_biases.append(torch.zeros(m.shape, dtype=torch.bfloat16, device=m.device)
+                                            .masked_fill_(m, _NEG_INF))
+                    continue
+                if len(phs) == 1 and kwargs["mask_kind"] == _ffi.MASK_NONE:
+                    kind = _classify_document_mask(node, phs[0], invert, L, S, gm)
+                    if kind is not None:
+                        kwargs["mask_kind"] = kind
+                        doc_ids = phs[0]
+                        continue
+                run_masks.append(node)
+                run_invert.append(invert)
+            for node in r.biases:
+                b = _try_evaluate(node, gm) if not _placeholders_of(node) else None
+                if isinstance(b, torch.Tensor):
+                    if kwargs["alibi_heads"] == 0 and _is_alibi(b, Hq, L, S):
+                        kwargs["alibi_heads"] = Hq
+                    else:
+                        const_biases.append(b)
+                else:
+                    run_biases.append(node)
+        except _NoMatch:
+            continue
+        bias_nodes: List[fx.Node] = list(run_biases)
+        with gm.graph.inserting_before(r.out):
+            for i, t in enumerate(const_biases):
+                name = f"_flashlight_const_{replaced}_{i}"
+                gm.register_buffer(name, t, persistent=False)
+                bias_nodes.append(gm.graph.get_attr(name))
+            new = gm.graph.call_function(fused_attention, (r.q, r.k, r.v, doc_ids, bias_nodes, run_masks),
+                                         dict(kwargs, mask_invert=tuple(run_invert)))
+        new.meta.update(r.out.meta)
+        r.out.replace_all_uses_with(new)
+        for n in r.nodes:
+            if not n.users:
+                gm.graph.erase_node(n)
+        replaced += 1
+    if replaced:
+        _merge_differential(gm)
+        gm.graph.eliminate_dead_code()
+        gm.graph.lint()
+        gm.recompile()
+    return replaced
+
+
+def backend(gm: fx.GraphModule, example_inputs):
+    """`torch.compile(fn, backend=flashlight_amd.fusion.backend, dynamic=False)`, or `backend="flashlight_amd"` once
+    this module is imported: attention regions run on the fused kernel, the rest of the captured graph as eager
+    PyTorch."""
+    fuse_attention(gm)
+    return gm.forward
+
+
+torch._dynamo.register_backend(compiler_fn=backend, name="flashlight_amd")

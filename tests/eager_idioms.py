@@ -1,0 +1,142 @@
+"""Attention written out in eager PyTorch, the way callers of the reference write it (the idioms of
+attention_variants/*.py: explicit matmuls, a mask or bias built with tensor operations, softmax, second matmul; GQA by
+viewing the query as [N, Hkv, G, L, E]).  Inputs for the graph-rewrite tests: `flashlight_amd.fusion` has to recognise
+each of them, and on a GPU the rewritten function has to return what the eager function returns."""
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _gqa(query, key, value):
+    query = query.view(query.size(0), key.size(1), -1, query.size(-2), query.size(-1))
+    return query, key.unsqueeze(2), value.unsqueeze(2)
+
+
+def plain(query, key, value, enable_gqa=False):
+    s = 1 / math.sqrt(query.size(-1))
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+    w = torch.softmax(query @ key.transpose(-2, -1) * s, dim=-1)
+    return (w @ value).view(value.size(0), -1, value.size(-2), value.size(-1))
+
+
+def divided_by_sqrt_d(query, key, value):
+    return torch.matmul(F.softmax(torch.matmul(query, key.mT) / math.sqrt(query.size(-1)), dim=-1), value)
+
+
+def causal_triu(query, key, value, enable_gqa=False):
+    s = 1 / math.sqrt(query.size(-1))
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+    future = torch.triu(torch.ones(query.size(-2), key.size(-2), device=query.device, dtype=torch.bool), diagonal=1)
+    w = torch.where(future, float("-inf"), query @ key.transpose(-2, -1) * s)
+    return torch.softmax(w, dim=-1) @ value
+
+
+def causal_tril_keep(query, key, value):
+    keep = torch.ones(query.size(-2), key.size(-2), device=query.device).tril().bool()
+    w = torch.where(keep, torch.matmul(query, key.transpose(-1, -2)) * 0.2, -1e30)
+    return w.softmax(-1) @ value
+
+
+def sliding(query, key, value, window, enable_gqa=False):
+    s = 1.0 / math.sqrt(query.size(-1))
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+    n = query.size(-2)
+    qi = torch.arange(n, device=query.device).view(n, 1)
+    ki = torch.arange(n, device=query.device).view(1, n)
+    outside = ((qi < ki) | ((qi - ki) > window)).unsqueeze(0).unsqueeze(0)
+    w = (torch.matmul(query, key.transpose(-2, -1)) * s).masked_fill(outside, -1e10)
+    return torch.softmax(w, dim=-1) @ value
+
+
+def prefix_lm(query, key, value, prefix, enable_gqa=False):
+    s = 1.0 / math.sqrt(query.size(-1))
+    n = query.size(-2)
+    plen = torch.full((query.size(0),), prefix, dtype=torch.long, device=query.device)
+    qi = torch.arange(n, device=query.device).view(1, 1, n, 1)
+    ki = torch.arange(n, device=query.device).view(1, 1, 1, n)
+    hidden = ki > torch.maximum(plen.view(-1, 1, 1, 1) - 1, qi)
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+        hidden = hidden.unsqueeze(2).expand(hidden.size(0), key.size(1), -1, n, n)
+    w = (torch.matmul(query, key.transpose(-2, -1)) * s).masked_fill(hidden, -1e10)
+    return torch.softmax(w, dim=-1) @ value
+
+
+def documents(query, key, value, document_id, causal=False, enable_gqa=False):
+    s = 1.0 / math.sqrt(query.size(-1))
+    other = (document_id.unsqueeze(2) != document_id.unsqueeze(1)).unsqueeze(1)
+    if causal:
+        n = query.size(-2)
+        other = other | torch.ones(n, n, dtype=torch.bool, device=query.device).triu(1)
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+        other = other.unsqueeze(2).expand(other.size(0), key.size(1), -1, other.size(-2), other.size(-1))
+    w = torch.where(other, -1e10, torch.matmul(query, key.transpose(-2, -1)) * s)
+    return torch.softmax(w, dim=-1) @ value
+
+
+def alibi(query, key, value, enable_gqa=False):
+    s = 1 / math.sqrt(query.size(-1))
+    h = query.size(1)
+    if enable_gqa:
+        query, key, value = _gqa(query, key, value)
+    w = torch.matmul(query, key.transpose(-2, -1)) * s
+    slopes = torch.exp2(-((torch.arange(h, dtype=torch.int32, device=query.device) + 1) * 8.0 / h))
+    rel = torch.arange(w.size(-1), dtype=torch.int32, device=query.device)[None, :] - \
+        torch.arange(w.size(-2), dtype=torch.int32, device=query.device)[:, None]
+    bias = (slopes[:, None, None] * rel).to(w.dtype)
+    if enable_gqa:
+        bias = bias.view(w.size(1), w.size(2), w.size(3), w.size(4))
+    return torch.softmax(w + bias, dim=-1) @ value
+
+
+def softcap(query, key, value, cap, causal=False):
+    w = query @ key.transpose(-2, -1) * (1 / math.sqrt(query.size(-1)))
+    w = cap * torch.tanh(w / cap)
+    if causal:
+        w = w.masked_fill(torch.ones(w.size(-2), w.size(-1), dtype=torch.bool, device=w.device).triu(1), float("-inf"))
+    return torch.softmax(w, dim=-1) @ value
+
+
+def learned_bias(query, key, value, bias, key_padding):
+    """A run-time additive bias plus a boolean key-padding mask that no closed form covers."""
+    w = torch.matmul(query, key.transpose(-2, -1)) / math.sqrt(query.size(-1)) + bias
+    w = w.masked_fill(key_padding[:, None, None, :], float("-inf"))
+    return torch.matmul(torch.softmax(w, dim=-1), value)
+
+
+def checkerboard(query, key, value):
+    """A constant mask that is none of the positional forms: attend only keys of the query's parity."""
+    n = query.size(-2)
+    i = torch.arange(n, device=query.device)
+    hidden = (i.view(n, 1) + i.view(1, n)) % 2 == 1
+    w = (query @ key.transpose(-2, -1) * 0.125).masked_fill(hidden, float("-inf"))
+    return torch.softmax(w, dim=-1) @ value
+
+
+def differential(q, k, v, lam):
+    s = 1 / math.sqrt(q.size(-1))
+    h, hk = q.size(1) // 2, k.size(1) // 2
+    w0 = torch.matmul(q[:, :h], k[:, :hk].transpose(-1, -2)) * s
+    w1 = torch.matmul(q[:, h:], k[:, hk:].transpose(-1, -2)) * s
+    w0 = torch.softmax(w0, dim=-1).type_as(w0)
+    w1 = torch.softmax(w1, dim=-1).type_as(w1)
+    return torch.matmul(w0, v) - lam * torch.matmul(w1, v)
+
+
+def msa_row(q_in, k_in, v_in, biases):
+    q, k, v = (t.transpose(-2, -3) for t in (q_in, k_in, v_in))
+    a = torch.matmul(q, k.transpose(-1, -2)) * (1 / math.sqrt(q.size(-1)))
+    for b in biases:
+        a += b
+    return torch.matmul(F.softmax(a, dim=-1), v).transpose(-2, -3)
+
+
+def returns_weights(query, key, value):
+    """Not fusable: the caller wants the attention weights as well."""
+    w = torch.softmax(query @ key.transpose(-2, -1) * 0.125, dim=-1)
+    return w @ value, w

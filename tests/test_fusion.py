@@ -1,0 +1,222 @@
+"""`flashlight_amd.fusion`: eager attention captured by `torch.compile` is rewritten into one fused launch per region
+(the reference reaches the same end by patching TorchInductor: `from monkeypatch.fusion import ...`,
+tests/test_causal.py:14-17,33).  The CPU tests check what the rewrite recognises; the GPU tests check that the
+rewritten function returns what the eager one returns."""
+import functools
+
+import pytest
+import torch
+
+from flashlight_amd import _ffi, fusion
+from tests import eager_idioms as E
+from tests.conftest import assert_parity
+
+BF = torch.bfloat16
+
+
+def _rewrite(fn, *args):
+    """Captures `fn` with Dynamo, rewrites the graph and returns (graph module, fused call nodes) without running it."""
+    got = []
+
+    class _Stop(Exception):
+        pass
+
+    def be(gm, example_inputs):
+        fusion.fuse_attention(gm)
+        got.append(gm)
+
+        def run(*a):
+            raise _Stop
+        return run
+
+    torch._dynamo.reset()
+    with pytest.raises(_Stop):
+        torch.compile(fn, backend=be, dynamic=False, fullgraph=True)(*args)
+    assert len(got) == 1
+    gm = got[0]
+    return gm, [n for n in gm.graph.nodes if n.op == "call_function" and n.target is fusion.fused_attention]
+
+
+def _leftover(gm):
+    names = {fusion._name(n) for n in gm.graph.nodes}
+    return names & {"matmul", "softmax", "where", "masked_fill", "tanh"}
+
+
+def _qkv(N=2, Hq=4, Hkv=4, L=48, E=32, dev="cpu", seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g).to(BF).to(dev)  # noqa: E731
+    return mk(N, Hq, L, E), mk(N, Hkv, L, E), mk(N, Hkv, L, E)
+
+
+def _ids(N, L, dev="cpu"):
+    g = torch.Generator().manual_seed(3)
+    return torch.randint(0, 4, (N, L), generator=g).sort(dim=1).values.to(dev)
+
+
+# name -> (function of (q, k, v, *extra), extra-input builder, expected kwargs of the fused call, Hkv)
+CASES = {
+    "plain": (E.plain, None, dict(mask_kind=_ffi.MASK_NONE, gqa=False), 4),
+    "plain gqa": (functools.partial(E.plain, enable_gqa=True), None, dict(mask_kind=_ffi.MASK_NONE, gqa=True), 2),
+    "div by sqrt(d), .mT": (E.divided_by_sqrt_d, None, dict(mask_kind=_ffi.MASK_NONE), 4),
+    "causal triu/where": (E.causal_triu, None, dict(mask_kind=_ffi.MASK_CAUSAL), 4),
+    "causal gqa": (functools.partial(E.causal_triu, enable_gqa=True), None, dict(mask_kind=_ffi.MASK_CAUSAL, gqa=True), 2),
+    "causal tril/keep": (E.causal_tril_keep, None, dict(mask_kind=_ffi.MASK_CAUSAL, scale=0.2), 4),
+    "sliding": (functools.partial(E.sliding, window=5), None, dict(mask_kind=_ffi.MASK_SLIDING, window=5), 4),
+    "sliding gqa": (functools.partial(E.sliding, window=17, enable_gqa=True), None,
+                    dict(mask_kind=_ffi.MASK_SLIDING, window=17, gqa=True), 1),
+    "sliding wider than L": (functools.partial(E.sliding, window=1000), None, dict(mask_kind=_ffi.MASK_CAUSAL), 4),
+    "prefix": (functools.partial(E.prefix_lm, prefix=9), None, dict(mask_kind=_ffi.MASK_PREFIX_LM, prefix=9), 4),
+    "prefix gqa": (functools.partial(E.prefix_lm, prefix=20, enable_gqa=True), None,
+                   dict(mask_kind=_ffi.MASK_PREFIX_LM, prefix=20, gqa=True), 2),
+    "alibi": (E.alibi, None, dict(alibi_heads=4, mask_kind=_ffi.MASK_NONE), 4),
+    "alibi gqa": (functools.partial(E.alibi, enable_gqa=True), None, dict(alibi_heads=4, gqa=True), 2),
+    "softcap": (functools.partial(E.softcap, cap=30.0), None, dict(softcap=30.0, mask_kind=_ffi.MASK_NONE), 4),
+    "softcap causal": (functools.partial(E.softcap, cap=50.0, causal=True), None,
+                       dict(softcap=50.0, mask_kind=_ffi.MASK_CAUSAL), 4),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_rewrite_recognises(name):
+    fn, _, want, hkv = CASES[name]
+    q, k, v = _qkv(Hkv=hkv)
+    gm, calls = _rewrite(fn, q, k, v)
+    assert len(calls) == 1 and not _leftover(gm), gm.graph
+    kw = calls[0].kwargs
+    for key, val in want.items():
+        assert kw[key] == pytest.approx(val), (key, kw)
+    if "scale" not in want:
+        assert kw["scale"] == pytest.approx(32 ** -0.5)
+    # nothing dense survives: no bias operand, no run-time mask
+    assert list(calls[0].args[4]) == [] and list(calls[0].args[5]) == [] and calls[0].args[3] is None
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("gqa", [False, True])
+def test_rewrite_recognises_document_masks_by_probing(causal, gqa):
+    q, k, v = _qkv(Hkv=2 if gqa else 4)
+    ids = _ids(2, 48)
+    gm, calls = _rewrite(functools.partial(E.documents, causal=causal, enable_gqa=gqa), q, k, v, ids)
+    assert len(calls) == 1 and not _leftover(gm)
+    assert calls[0].kwargs["mask_kind"] == (_ffi.MASK_DOCUMENT_CAUSAL if causal else _ffi.MASK_DOCUMENT)
+    ids_node = calls[0].args[3]
+    assert ids_node.op == "placeholder" and list(calls[0].args[4]) == [] and list(calls[0].args[5]) == []
+
+
+def test_rewrite_keeps_what_it_cannot_name_as_dense_operands():
+    q, k, v = _qkv()
+    # constant mask without a closed form -> one constant additive operand
+    gm, calls = _rewrite(E.checkerboard, q, k, v)
+    assert len(calls) == 1 and not _leftover(gm)
+    (b,) = calls[0].args[4]
+    buf = getattr(gm, b.target)
+    assert b.op == "get_attr" and buf.dtype == BF and tuple(buf.shape) == (48, 48)
+    assert bool(torch.isinf(buf[0, 1])) and float(buf[0, 2]) == 0.0
+    # run-time bias and run-time boolean mask stay graph inputs
+    bias = torch.randn(2, 4, 48, 48)
+    pad = torch.zeros(2, 48, dtype=torch.bool)
+    gm, calls = _rewrite(E.learned_bias, q, k, v, bias, pad)
+    assert len(calls) == 1 and not _leftover(gm)
+    assert [n.op for n in calls[0].args[4]] == ["placeholder"] and len(calls[0].args[5]) == 1
+    assert calls[0].kwargs["mask_kind"] == _ffi.MASK_NONE
+
+
+def test_rewrite_differential_and_msa_row():
+    q, k, _ = _qkv(Hq=8, Hkv=8)
+    v = torch.randn(2, 4, 48, 64).to(BF)
+    gm, calls = _rewrite(functools.partial(E.differential, lam=0.3), q, k, v)
+    assert not _leftover(gm)
+    assert len(calls) == 1 and calls[0].kwargs["diff_lambda"] == pytest.approx(0.3)
+    assert calls[0].args[0].op == "placeholder" and calls[0].args[1].op == "placeholder"
+    Q, K, V = (torch.randn(1, 3, 40, 2, 32).to(BF) for _ in range(3))
+    mask, pair = torch.randn(1, 3, 1, 1, 40).to(BF), torch.randn(1, 1, 2, 40, 40).to(BF)
+    gm, calls = _rewrite(lambda Q, K, V, m, p: E.msa_row(Q, K, V, [m, p]), Q, K, V, mask, pair)
+    assert len(calls) == 1 and not _leftover(gm) and len(calls[0].args[4]) == 2
+
+
+def test_rewrite_leaves_other_graphs_alone():
+    q, k, v = _qkv()
+    gm, calls = _rewrite(E.returns_weights, q, k, v)
+    assert calls == [] and _leftover(gm) >= {"matmul", "softmax"}
+    gm, calls = _rewrite(lambda a, b: torch.softmax(a @ b, dim=-1), q, k.transpose(-2, -1))
+    assert calls == []
+    # softmax over the query axis is not attention
+    gm, calls = _rewrite(lambda q, k, v: torch.softmax(q @ k.transpose(-2, -1), dim=-2) @ v, q, k, v)
+    assert calls == []
+    # a bias added before the scale cannot be expressed
+    gm, calls = _rewrite(lambda q, k, v, b: torch.softmax((q @ k.transpose(-2, -1) + b) * 0.1, dim=-1) @ v, q, k, v,
+                         torch.randn(48, 48))
+    assert calls == []
+
+
+def test_rewritten_function_fails_loudly_without_a_gpu():
+    q, k, v = _qkv()
+    torch._dynamo.reset()
+    with pytest.raises(NotImplementedError, match="no CPU path"):
+        torch.compile(E.causal_triu, backend=fusion.backend, dynamic=False)(q, k, v)
+    torch._dynamo.reset()
+    with pytest.raises(NotImplementedError, match="no CPU path"):  # registered under a name as well
+        torch.compile(E.plain, backend="flashlight_amd", dynamic=False)(q, k, v)
+
+
+def test_mask_classifier_closed_forms():
+    L = 37
+    q, k = torch.arange(L).view(L, 1), torch.arange(L).view(1, L)
+    C = fusion._classify_constant_mask
+    assert C(torch.zeros(L, L, dtype=torch.bool), L, L) == (_ffi.MASK_NONE, 0, 0)
+    assert C((k > q), L, L) == (_ffi.MASK_CAUSAL, 0, 0)
+    assert C((k > q).expand(3, 2, L, L), L, L) == (_ffi.MASK_CAUSAL, 0, 0)
+    for w in (0, 1, 7, 35):
+        assert C((q < k) | (q - k > w), L, L) == (_ffi.MASK_SLIDING, w, 0)
+    assert C((q < k) | (q - k > 36), L, L) == (_ffi.MASK_CAUSAL, 0, 0)          # the window reaches every key
+    for p in (2, 9, 36):
+        assert C(k > torch.clamp(q, min=p - 1), L, L) == (_ffi.MASK_PREFIX_LM, 0, p)
+    assert C(k > torch.clamp(q, min=L - 1), L, L) == (_ffi.MASK_NONE, 0, 0)      # prefix covers everything
+    assert C((q + k) % 2 == 1, L, L) is None
+    assert C((k >= q), L, L) is None                                             # strictly-lower: row 0 attends nothing
+    per_batch = torch.stack([(k > q), (k > q + 1)])
+    assert C(per_batch, L, L) is None
+    # rectangular scores: causal is defined (upper-left aligned), the window forms are not
+    assert C(torch.arange(50).view(1, 50) > q, L, 50) == (_ffi.MASK_CAUSAL, 0, 0)
+
+
+# ---- on the GPU: rewritten == eager ------------------------------------------------------------------------------------------
+
+def _check_on_gpu(fn, args, what):
+    torch._dynamo.reset()
+    got = torch.compile(fn, backend=fusion.backend, dynamic=False, fullgraph=True)(*args)
+    want = fn(*[a.float() if isinstance(a, torch.Tensor) and a.is_floating_point() else
+                [x.float() for x in a] if isinstance(a, list) else a for a in args])
+    assert got.shape == want.shape and got.dtype == BF, what
+    assert_parity(got, want, what)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_rewritten_equals_eager_on_gpu(name):
+    fn, _, _, hkv = CASES[name]
+    q, k, v = _qkv(N=2, Hq=4, Hkv=hkv, L=200, E=64, dev="cuda", seed=11)
+    _check_on_gpu(fn, (q, k, v), name)
+
+
+@pytest.mark.gpu
+def test_rewritten_dense_document_differential_and_msa_on_gpu():
+    dev = "cuda"
+    q, k, v = _qkv(N=2, Hq=4, Hkv=4, L=136, E=64, dev=dev, seed=12)
+    _check_on_gpu(E.checkerboard, (q, k, v), "checkerboard")
+    g = torch.Generator().manual_seed(5)
+    bias = torch.randn(2, 4, 136, 136, generator=g).to(dev)
+    pad = torch.zeros(2, 136, dtype=torch.bool)
+    pad[0, 100:] = True
+    _check_on_gpu(E.learned_bias, (q, k, v, bias, pad.to(dev)), "bias + padding mask")
+    for causal in (False, True):
+        for gqa in (False, True):
+            qq, kk, vv = _qkv(N=2, Hq=4, Hkv=2 if gqa else 4, L=136, E=64, dev=dev, seed=13)
+            _check_on_gpu(functools.partial(E.documents, causal=causal, enable_gqa=gqa), (qq, kk, vv, _ids(2, 136, dev)),
+                          f"documents causal={causal} gqa={gqa}")
+    qd, kd, _ = _qkv(N=2, Hq=8, Hkv=8, L=136, E=64, dev=dev, seed=14)
+    vd = torch.randn(2, 4, 136, 128, generator=g).to(BF).to(dev)
+    _check_on_gpu(functools.partial(E.differential, lam=0.3), (qd, kd, vd), "differential")
+    Q, K, V = (torch.randn(1, 3, 104, 2, 32, generator=g).to(BF).to(dev) for _ in range(3))
+    mask, pair = torch.randn(1, 3, 1, 1, 104, generator=g).to(BF).to(dev), torch.randn(1, 1, 2, 104, 104, generator=g).to(BF).to(dev)
+    _check_on_gpu(lambda Q, K, V, m, p: E.msa_row(Q, K, V, [m, p]), (Q, K, V, mask, pair), "msa row")

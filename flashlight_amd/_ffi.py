@@ -42,7 +42,21 @@ class FlAttnParams(C.Structure):
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
         ("attended_dump", C.c_void_p),
         ("bias_dtype", C.c_int32 * 2),
-        ("reserved", C.c_int32 * 6),
+        ("lse", C.c_void_p),
+        ("reserved", C.c_int32 * 4),
+    ]
+
+
+class FlAttnBwdParams(C.Structure):
+    """Mirror of `fl_attn_bwd_params` (include/flashlight_amd.h)."""
+
+    _fields_ = [
+        ("fwd", FlAttnParams),
+        ("dout", C.c_void_p), ("dout_strides", C.c_int64 * 4),
+        ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("dq_strides", C.c_int64 * 4), ("dk_strides", C.c_int64 * 4), ("dv_strides", C.c_int64 * 4),
+        ("delta", C.c_void_p),
+        ("reserved", C.c_int32 * 8),
     ]
 
 
@@ -80,12 +94,20 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_plan.argtypes = [C.POINTER(FlAttnParams), C.POINTER(C.c_int64)]
     lib.fl_attn_fwd.restype = C.c_int
     lib.fl_attn_fwd.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
+    lib.fl_bwd_params_sizeof.restype = C.c_uint64
+    lib.fl_attn_bwd_validate.restype = C.c_int
+    lib.fl_attn_bwd_validate.argtypes = [C.POINTER(FlAttnBwdParams)]
+    lib.fl_attn_bwd.restype = C.c_int
+    lib.fl_attn_bwd.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
     lib.fl_probe_mfma_rate.restype = C.c_int
     lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
         raise RuntimeError(f"{p}: ABI version {lib.fl_version()} != expected {ABI_VERSION}")
     if lib.fl_params_sizeof() != C.sizeof(FlAttnParams):
         raise RuntimeError(f"{p}: fl_attn_params is {lib.fl_params_sizeof()} bytes, binding expects {C.sizeof(FlAttnParams)}")
+    if lib.fl_bwd_params_sizeof() != C.sizeof(FlAttnBwdParams):
+        raise RuntimeError(f"{p}: fl_attn_bwd_params is {lib.fl_bwd_params_sizeof()} bytes, binding expects "
+                           f"{C.sizeof(FlAttnBwdParams)}")
     if path is None:
         _lib = lib
     return lib
@@ -121,65 +143,11 @@ def _dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
-def attn_fwd(
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    *,
-    scale: Optional[float] = None,
-    mask_kind: int = MASK_NONE,
-    window: int = 0,
-    prefix: int = 0,
-    doc_ids: Optional[torch.Tensor] = None,
-    alibi_heads: int = 0,
-    softcap: float = 0.0,
-    biases: Sequence[tuple[torch.Tensor, int]] = (),
-    gate: Optional[torch.Tensor] = None,
-    diff: bool = False,
-    lambda_full: float = 0.0,
-    out: Optional[torch.Tensor] = None,
-    attended_dump: Optional[torch.Tensor] = None,
-    validate_only: bool = False,
-) -> torch.Tensor:
-    """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
-
-    `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, bf16 or fp32, broadcastable to
-    [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
-    """
-    lib = load_library()
-    for name, t in (("query", q), ("key", k), ("value", v)):
-        _require_gpu_bf16(name, t)
-        if t.dim() != 4:
-            raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
-    q, k, v = _dim_contiguous(q), _dim_contiguous(k), _dim_contiguous(v)
-    B, Hq_all, Lq, Dqk = q.shape
-    Bk, Hk_all, Lk, Dk = k.shape
-    Bv, Hv, Lv, Dv = v.shape
-    if not (B == Bk == Bv) or Dqk != Dk or Lk != Lv:
-        raise ValueError(f"inconsistent shapes: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
-    if diff:
-        if Hq_all % 2 or Hk_all % 2:
-            raise ValueError("differential attention needs an even number of query and key heads")
-        Hq, Hkv = Hq_all // 2, Hk_all // 2
-    else:
-        Hq, Hkv = Hq_all, Hk_all
-    if Hv != Hkv:
-        raise ValueError(f"value has {Hv} heads, expected {Hkv}")
-    if out is None:
-        out = torch.empty((B, Hq, Lq, Dv), dtype=torch.bfloat16, device=q.device)
-    elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != torch.bfloat16 or out.device != q.device:
-        raise ValueError("out has the wrong shape, dtype or device")
-    if diff and Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None:
-        # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,
-        # so wide values go in slabs of _MAX_DV_DIFF columns, one launch each, through strided views of v and out
-        # (the reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38).
-        for c in range(0, Dv, _MAX_DV_DIFF):
-            attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
-                     doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
-                     gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
-                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
-        return out
-
+def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases,
+                 gate, diff, lambda_full, attended_dump):
+    """Fills an `fl_attn_params` for validated 4-D tensors; returns it with the tensors that must outlive the launch."""
+    B, _, Lq, Dqk = q.shape
+    Lk, Dv = k.shape[2], v.shape[3]
     p = FlAttnParams()
     p.q, p.k, p.v, p.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     p.q_strides[:] = _strides4(q)
@@ -250,6 +218,76 @@ def attn_fwd(
         ws = torch.empty(need, dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), need
         keep.append(ws)
+    return p, keep
+
+
+def attn_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    scale: Optional[float] = None,
+    mask_kind: int = MASK_NONE,
+    window: int = 0,
+    prefix: int = 0,
+    doc_ids: Optional[torch.Tensor] = None,
+    alibi_heads: int = 0,
+    softcap: float = 0.0,
+    biases: Sequence[tuple[torch.Tensor, int]] = (),
+    gate: Optional[torch.Tensor] = None,
+    diff: bool = False,
+    lambda_full: float = 0.0,
+    out: Optional[torch.Tensor] = None,
+    attended_dump: Optional[torch.Tensor] = None,
+    validate_only: bool = False,
+    lse: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
+
+    `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, bf16 or fp32, broadcastable to
+    [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
+    `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
+    """
+    lib = load_library()
+    for name, t in (("query", q), ("key", k), ("value", v)):
+        _require_gpu_bf16(name, t)
+        if t.dim() != 4:
+            raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
+    q, k, v = _dim_contiguous(q), _dim_contiguous(k), _dim_contiguous(v)
+    B, Hq_all, Lq, Dqk = q.shape
+    Bk, Hk_all, Lk, Dk = k.shape
+    Bv, Hv, Lv, Dv = v.shape
+    if not (B == Bk == Bv) or Dqk != Dk or Lk != Lv:
+        raise ValueError(f"inconsistent shapes: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if diff:
+        if Hq_all % 2 or Hk_all % 2:
+            raise ValueError("differential attention needs an even number of query and key heads")
+        Hq, Hkv = Hq_all // 2, Hk_all // 2
+    else:
+        Hq, Hkv = Hq_all, Hk_all
+    if Hv != Hkv:
+        raise ValueError(f"value has {Hv} heads, expected {Hkv}")
+    if out is None:
+        out = torch.empty((B, Hq, Lq, Dv), dtype=torch.bfloat16, device=q.device)
+    elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != torch.bfloat16 or out.device != q.device:
+        raise ValueError("out has the wrong shape, dtype or device")
+    if diff and Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None:
+        # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,
+        # so wide values go in slabs of _MAX_DV_DIFF columns, one launch each, through strided views of v and out
+        # (the reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38).
+        for c in range(0, Dv, _MAX_DV_DIFF):
+            attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
+                     doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
+                     gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
+                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
+        return out
+
+    p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
+                           biases, gate, diff, lambda_full, attended_dump)
+    if lse is not None:
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
+            raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")
+        p.lse = lse.data_ptr()
     if validate_only:
         _check(lib.fl_attn_validate(C.byref(p)))
         return out
@@ -259,6 +297,46 @@ def attn_fwd(
     # tensors in `keep` were last used on the current stream; the caching allocator orders their reuse after it
     del keep
     return out
+
+
+def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, dout: torch.Tensor,
+             *, scale: Optional[float] = None, mask_kind: int = MASK_NONE, window: int = 0, prefix: int = 0,
+             doc_ids: Optional[torch.Tensor] = None, alibi_heads: int = 0, softcap: float = 0.0,
+             validate_only: bool = False):
+    """Gradients (dq, dk, dv) of `attn_fwd` called with the same arguments; `out` and `lse` are what that call
+    returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream."""
+    lib = load_library()
+    for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
+        _require_gpu_bf16(name, t)
+        if t.dim() != 4:
+            raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
+    q, k, v, out, dout = (_dim_contiguous(t) for t in (q, k, v, out, dout))
+    B, Hq, Lq, Dqk = q.shape
+    Hkv, Lk, Dv = k.shape[1], k.shape[2], v.shape[3]
+    if tuple(out.shape) != (B, Hq, Lq, Dv) or tuple(dout.shape) != (B, Hq, Lq, Dv):
+        raise ValueError("out and dout must be [B, Hq, Lq, Dv]")
+    if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
+        raise ValueError("lse must be the contiguous float32 [B, Hq, Lq] tensor the forward filled")
+    fwd, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
+                             (), None, False, 0.0, None)
+    fwd.lse = lse.data_ptr()
+    dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
+        torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
+    delta = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
+    b = FlAttnBwdParams()
+    b.fwd = fwd
+    b.dout, b.dq, b.dk, b.dv, b.delta = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr()
+    b.dout_strides[:] = _strides4(dout)
+    b.dq_strides[:] = _strides4(dq)
+    b.dk_strides[:] = _strides4(dk)
+    b.dv_strides[:] = _strides4(dv)
+    if validate_only:
+        _check(lib.fl_attn_bwd_validate(C.byref(b)))
+        return dq, dk, dv
+    with torch.cuda.device(q.device):
+        _check(lib.fl_attn_bwd(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    del keep, delta
+    return dq, dk, dv
 
 
 def plan(p: FlAttnParams) -> dict:

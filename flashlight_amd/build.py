@@ -110,8 +110,17 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
         if not o.exists():
             tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_NAME={name}", f"-DFL_INST_ARGS={args}", "-c",
                            str(CSRC / "instance_unit.hip"), "-o", str(o)], o))
-    # the instance table is host data only: compiling it for the device would reference the host launchers
-    for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("api.hip", []), ("probe.hip", [])):
+    # backward kernels: one unit per (head dim, feature bits) of FL_BWD_LIST in bwd_instances.h
+    bwd_list = re.search(r"#define FL_BWD_LIST\(X\)(.*)", (CSRC / "bwd_instances.h").read_text()).group(1)
+    for d, feat in re.findall(r"X\((\d+),\s*(\d+)\)", bwd_list):
+        o = objdir / f"bwd_{d}_{feat}.o"
+        objs.append(o)
+        if not o.exists():
+            tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_BWD_D={d}", f"-DFL_BWD_FEAT={feat}", "-c", str(CSRC / "bwd_unit.hip"),
+                           "-o", str(o)], o))
+    # the instance tables are host data only: compiling them for the device would reference the host launchers
+    for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("bwd_table.hip", ["--cuda-host-only"]),
+                       ("api.hip", []), ("probe.hip", [])):
         o = objdir / (Path(src).stem + ".o")
         objs.append(o)
         if not o.exists():

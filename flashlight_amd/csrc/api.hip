@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "flashlight_amd.h"
+#include "bwd_instances.h"
 #include "instances.h"
 
 namespace fl {
@@ -131,8 +132,12 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if ((rc = check_strides("q", p->q_strides, 8)) || (rc = check_strides("k", p->k_strides, 8)) ||
       (rc = check_strides("v", p->v_strides, 8)) || (rc = check_strides("o", p->o_strides, 4)))
     return rc;
-  for (int i = 0; i < 6; ++i)
+  for (int i = 0; i < 4; ++i)
     if (p->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
+  if (p->lse) {
+    if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
+    if (p->diff) return fail(FL_ERR_UNSUPPORTED, "lse is not produced for differential attention");
+  }
 
   switch (p->mask_kind) {
     case FL_MASK_NONE:
@@ -316,6 +321,7 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
     kp.k_branch_stride = (int64_t)p->Hkv * p->k_strides[1];
   }
   kp.dump = p->attended_dump;
+  kp.lse = p->lse;
   const int bm = in->rw * in->nw;
   kp.n_qtiles = (p->Lq + bm - 1) / bm;
   kp.n_ktiles = (p->Lk + in->bn - 1) / in->bn;
@@ -334,6 +340,121 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   }
   hipError_t e = in->launch(kp, grid, (int)lds_bytes_for(in, p), stream);
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));
+  return 0;
+}
+
+uint64_t fl_bwd_params_sizeof(void) { return sizeof(fl_attn_bwd_params); }
+
+static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out) {
+  if (!b) return fail(FL_ERR_NULL, "params is null");
+  const fl_attn_params* p = &b->fwd;
+  int rc = validate(p, nullptr);
+  if (rc) return rc;
+  if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
+    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands, gate, differential attention and the dump hook are not supported");
+  if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
+  if (!p->lse) return fail(FL_ERR_NULL, "backward: fwd.lse (the forward's row statistics) is null");
+  if ((rc = check_ptr("dout", b->dout, 16)) || (rc = check_ptr("dq", b->dq, 8)) || (rc = check_ptr("dk", b->dk, 8)) ||
+      (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 4)))
+    return rc;
+  if ((rc = check_strides("dout", b->dout_strides, 8)) || (rc = check_strides("dq", b->dq_strides, 4)) ||
+      (rc = check_strides("dk", b->dk_strides, 4)) || (rc = check_strides("dv", b->dv_strides, 4)) ||
+      (rc = check_strides("o", p->o_strides, 8)))
+    return rc;
+  if (reinterpret_cast<uintptr_t>(p->o) % 16) return fail(FL_ERR_ALIGN, "backward: o must be 16-byte aligned");
+  for (int i = 0; i < 8; ++i)
+    if (b->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
+  // per-lane byte offsets inside one staged tile (up to 128 rows) are 32-bit
+  const int64_t worst = std::max(std::max(p->q_strides[2], p->k_strides[2]), std::max(p->v_strides[2], b->dout_strides[2]));
+  if ((128 * worst + p->Dqk) * 2 >= ((int64_t)1 << 31))
+    return fail(FL_ERR_STRIDE, "backward: sequence stride too large (%lld elements)", (long long)worst);
+  if ((int64_t)p->B * p->Hq * ((p->Lq + 127) / 128) > 0x7fffffff || (int64_t)p->B * p->Hkv * ((p->Lk + 127) / 128) > 0x7fffffff)
+    return fail(FL_ERR_SHAPE, "backward: too many workgroups");
+  uint32_t want = 0;
+  if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
+  if (is_doc(p->mask_kind)) {
+    if (want) return fail(FL_ERR_UNSUPPORTED, "backward: document masks cannot be combined with ALiBi or a soft-cap");
+    want = fl::F_DOC;
+  }
+  const fl::BwdInstance* in = nullptr;
+  for (int i = 0; i < fl::kNumBwdInstances; ++i)
+    if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want) in = &fl::kBwdInstances[i];
+  if (!in) return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d (64 and 128 are compiled)", p->Dqk);
+  if (out) *out = in;
+  g_err[0] = 0;
+  return 0;
+}
+
+int fl_attn_bwd_validate(const fl_attn_bwd_params* b) { return validate_bwd(b, nullptr); }
+
+int fl_attn_bwd(const fl_attn_bwd_params* b, void* stream_) {
+  const fl::BwdInstance* in = nullptr;
+  int rc = validate_bwd(b, &in);
+  if (rc) return rc;
+  const fl_attn_params* p = &b->fwd;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  fl::BParams bp;
+  std::memset(&bp, 0, sizeof(bp));
+  bp.q = static_cast<const fl::bf16_t*>(p->q);
+  bp.k = static_cast<const fl::bf16_t*>(p->k);
+  bp.v = static_cast<const fl::bf16_t*>(p->v);
+  bp.o = static_cast<const fl::bf16_t*>(p->o);
+  bp.dout = static_cast<const fl::bf16_t*>(b->dout);
+  bp.lse = p->lse;
+  bp.delta = b->delta;
+  bp.dq = static_cast<fl::bf16_t*>(b->dq);
+  bp.dk = static_cast<fl::bf16_t*>(b->dk);
+  bp.dv = static_cast<fl::bf16_t*>(b->dv);
+  for (int i = 0; i < 3; ++i) {
+    bp.qs[i] = p->q_strides[i];
+    bp.ks[i] = p->k_strides[i];
+    bp.vs[i] = p->v_strides[i];
+    bp.os[i] = p->o_strides[i];
+    bp.dos[i] = b->dout_strides[i];
+    bp.dqs[i] = b->dq_strides[i];
+    bp.dks[i] = b->dk_strides[i];
+    bp.dvs[i] = b->dv_strides[i];
+  }
+  bp.B = p->B;
+  bp.Hq = p->Hq;
+  bp.Hkv = p->Hkv;
+  bp.Lq = p->Lq;
+  bp.Lk = p->Lk;
+  bp.group = p->Hq / p->Hkv;
+  bp.scale = p->scale;
+  bp.scale_log2 = p->scale * 1.4426950408889634f;
+  bp.mask_kind = p->mask_kind;
+  bp.window = p->window;
+  bp.prefix = p->prefix;
+  {
+    const int kFar = 1 << 29;
+    const bool causal_like = p->mask_kind == FL_MASK_CAUSAL || p->mask_kind == FL_MASK_SLIDING ||
+                             p->mask_kind == FL_MASK_PREFIX_LM || p->mask_kind == FL_MASK_DOCUMENT_CAUSAL;
+    bp.dmax = causal_like ? 0 : kFar;
+    bp.dmin = p->mask_kind == FL_MASK_SLIDING ? -(p->window < kFar ? p->window : kFar) : -kFar;
+    bp.pfx = p->mask_kind == FL_MASK_PREFIX_LM ? (p->prefix < 0 ? 0 : p->prefix) : 0;
+  }
+  bp.doc_ids = p->doc_ids;
+  bp.doc_stride = p->doc_stride;
+  bp.alibi_heads = p->alibi_heads;
+  bp.softcap = p->softcap;
+  if (is_doc(p->mask_kind)) {
+    const int blocks = (p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
+    const int total = p->B * blocks;
+    int64_t* table = static_cast<int64_t*>(p->workspace);
+    hipLaunchKernelGGL(fl::doc_table_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, p->doc_ids, p->doc_stride,
+                       p->Lk, blocks, total, table);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "doc_table_kernel launch failed: %s", hipGetErrorString(e));
+    bp.doc_table = table;
+    bp.doc_blocks = blocks;
+  }
+  hipError_t e = in->launch_delta(bp, stream);
+  if (e != hipSuccess) return fail((int)e, "backward: launch of the row-sum kernel failed: %s", hipGetErrorString(e));
+  e = in->launch_dq(bp, stream);
+  if (e != hipSuccess) return fail((int)e, "backward: launch of the dQ kernel failed: %s", hipGetErrorString(e));
+  e = in->launch_dkv(bp, stream);
+  if (e != hipSuccess) return fail((int)e, "backward: launch of the dK/dV kernel failed: %s", hipGetErrorString(e));
   return 0;
 }
 

@@ -1,0 +1,63 @@
+// Launchers of the backward kernels: one translation unit per (head dim, feature set), both roles in it.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "bwd_kernel.h"
+#include "instances.h"
+
+namespace fl {
+
+struct BwdInstance {
+  int d;
+  uint32_t feat;
+  hipError_t (*launch_dq)(const BParams&, hipStream_t);
+  hipError_t (*launch_dkv)(const BParams&, hipStream_t);
+  hipError_t (*launch_delta)(const BParams&, hipStream_t);
+};
+
+extern const BwdInstance kBwdInstances[];
+extern const int kNumBwdInstances;
+
+template <class T>
+hipError_t launch_bwd(const BParams& bp, hipStream_t stream) {
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&bwd_kernel<T>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+  if (attr != hipSuccess) return attr;
+  const int len = T::ROLE == ROLE_DQ ? bp.Lq : bp.Lk, heads = T::ROLE == ROLE_DQ ? bp.Hq : bp.Hkv;
+  const int64_t grid = (int64_t)bp.B * heads * ((len + T::OWN - 1) / T::OWN);
+  hipLaunchKernelGGL(bwd_kernel<T>, dim3((unsigned)grid), dim3(T::NT), T::LDS_BYTES, stream, bp);
+  return hipGetLastError();
+}
+
+template <int DV>
+hipError_t launch_delta(const BParams& bp, hipStream_t stream) {
+  const int64_t rows = (int64_t)bp.B * bp.Hq * bp.Lq;
+  const int rows_per_block = 256 / (DV / 8);
+  hipLaunchKernelGGL(bwd_delta_kernel<DV>, dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
+                     stream, bp);
+  return hipGetLastError();
+}
+
+}  // namespace fl
+
+// (D, FEAT) pairs with compiled backward kernels.  FEAT 3 = ALiBi and/or soft-cap (either may be off at run time),
+// 8 = document ids in the element predicate.
+#define FL_BWD_LIST(X) X(64, 0) X(64, 3) X(64, 8) X(128, 0) X(128, 3) X(128, 8)
+
+#define FL_BWD_DECL(D, FEAT)                                           \
+  namespace fl {                                                       \
+  hipError_t launch_bwd_dq_##D##_##FEAT(const BParams&, hipStream_t);  \
+  hipError_t launch_bwd_dkv_##D##_##FEAT(const BParams&, hipStream_t); \
+  hipError_t launch_bwd_delta_##D##_##FEAT(const BParams&, hipStream_t); \
+  }
+#define FL_BWD_DEF(D, FEAT)                                                                                  \
+  namespace fl {                                                                                             \
+  hipError_t launch_bwd_dq_##D##_##FEAT(const BParams& bp, hipStream_t s) {                                  \
+    return launch_bwd<BwdTraits<D, ROLE_DQ, FEAT>>(bp, s);                                                   \
+  }                                                                                                          \
+  hipError_t launch_bwd_dkv_##D##_##FEAT(const BParams& bp, hipStream_t s) {                                 \
+    return launch_bwd<BwdTraits<D, ROLE_DKV, FEAT>>(bp, s);                                                  \
+  }                                                                                                          \
+  hipError_t launch_bwd_delta_##D##_##FEAT(const BParams& bp, hipStream_t s) { return launch_delta<D>(bp, s); } \
+  }
+#define FL_BWD_ROW(D, FEAT) {D, FEAT, &fl::launch_bwd_dq_##D##_##FEAT, &fl::launch_bwd_dkv_##D##_##FEAT, &fl::launch_bwd_delta_##D##_##FEAT},

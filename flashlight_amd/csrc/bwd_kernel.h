@@ -1,0 +1,410 @@
+// Backward of the fused attention forward for gfx950: dQ, dK, dV from dO, the forward's inputs and its row statistics.
+//
+// The reference is forward-only (its FLOP helper models a backward, benchmarks/_utils.py:16-21, but no kernel exists);
+// the arithmetic is the textbook one for softmax attention with recomputation:
+//   P = exp2(S2 - LSE2),  dP = dO V^T,  dS = P o (dP - Delta) * d(score)/d(qk),  dQ = dS K,  dK = dS^T Q,  dV = P^T dO
+// with S2 the modified logits in log2 units, LSE2 the forward's log2-sum-exp2 per row and Delta = rowsum(dO o O).
+//
+// One kernel template, two roles, no atomics:
+//   ROLE_DQ   a workgroup owns 128 query rows of one head and streams the key tiles they attend;
+//   ROLE_DKV  a workgroup owns 128 keys of one key/value head and streams the query tiles (of every query head of the
+//             group) that attend them.
+// In both roles a lane owns one *owner* position (the column of every accumulator it holds) and its registers run over
+// the streamed positions, because every product is issued with the streamed tile as the A operand:
+//   X1 = T1 . O1^T   (ROLE_DQ: K.Q^T = S^T;   ROLE_DKV: Q.K^T = S)       v_mfma_f32_32x32x16_bf16
+//   X2 = T2 . O2^T   (ROLE_DQ: V.dO^T = dP^T; ROLE_DKV: dO.V^T = dP)
+//   acc1 += T1^T . dS  (ROLE_DQ: dQ^T;  ROLE_DKV: dK^T),  ROLE_DKV also acc2 += T2^T . P  (dV^T)
+// so the fp32 layout of X1/X2 is the bf16 B-operand layout of the accumulating products (as in the forward kernel) and
+// P, dS never leave registers.  T1/T2 are staged in LDS by global_load_lds transfers, two slots, one barrier per tile;
+// T^T operands come from the same tiles through the transposing LDS read.
+#pragma once
+#include "fwd_kernel.h"
+
+namespace fl {
+
+enum : int { ROLE_DQ = 0, ROLE_DKV = 1 };
+
+struct BParams {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  const bf16_t* o;
+  const bf16_t* dout;
+  const float* lse;    // [B, Hq, Lq], log2 units; +inf for a row that attends nothing
+  float* delta;        // [B, Hq, Lq] scratch: rowsum(dO o O)
+  bf16_t* dq;
+  bf16_t* dk;
+  bf16_t* dv;
+  int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];  // element strides: batch, head, seq
+  int32_t B, Hq, Hkv, Lq, Lk, group;
+  float scale, scale_log2;
+  int32_t mask_kind, window, prefix;
+  int32_t dmin, dmax, pfx;  // attend iff key < Lk && ((dmin <= key - q <= dmax) || key < pfx)
+  const int64_t* doc_ids;
+  int64_t doc_stride;
+  const int64_t* doc_table;  // [B][ceil(L / kDocBlock)][2] = (min, max), as in the forward
+  int32_t doc_blocks;
+  int32_t alibi_heads;
+  float softcap;
+};
+
+// Delta[b, h, q] = sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
+template <int DV>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
+  constexpr int LPR = DV / 8;  // lanes per row, 16 bytes each
+  const int64_t rows = (int64_t)p.B * p.Hq * p.Lq;
+  const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+  const int c = threadIdx.x % LPR;
+  float s = 0.f;
+  if (row < rows) {
+    const int q = (int)(row % p.Lq), h = (int)((row / p.Lq) % p.Hq), b = (int)(row / ((int64_t)p.Lq * p.Hq));
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(p.dout + b * p.dos[0] + h * p.dos[1] + q * p.dos[2] + 8 * c);
+    const bf16x8 o = *reinterpret_cast<const bf16x8*>(p.o + b * p.os[0] + h * p.os[1] + q * p.os[2] + 8 * c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)o[e];
+  }
+#pragma unroll
+  for (int d = 1; d < LPR; d *= 2) s += __shfl_xor(s, d);
+  if (row < rows && c == 0) p.delta[row] = s;
+}
+
+template <int D_, int ROLE_, uint32_t FEAT_>
+struct BwdTraits {
+  static constexpr int D = D_, ROLE = ROLE_;
+  static constexpr uint32_t FEAT = FEAT_;
+  static constexpr int NW = 4, NT = 256, OWN = 128;        // waves, threads, owner positions per workgroup
+  static constexpr int TB = (ROLE == ROLE_DQ && D_ <= 64) ? 2 : 1;  // 32-position blocks per streamed tile (register budget)
+  static constexpr int BT = 32 * TB;
+  static constexpr int KS = D / 16, DB = D / 32;
+  static constexpr int TBYTES = BT * D * 2;                // one streamed tile
+  static constexpr int T_PER_T = TBYTES / (NT * 16);       // 16-byte transfers per thread per tile
+  static_assert(TBYTES % (NT * 16) == 0, "streamed tile must divide evenly over the threads");
+  static constexpr int OBYTES = (ROLE == ROLE_DKV) ? OWN * D * 2 : 0;  // owner tile kept in LDS (ROLE_DKV: K and V)
+  static constexpr int O_PER_T = OBYTES / (NT * 16);
+  static constexpr int T1_OFF = 0, T2_OFF = 2 * TBYTES, O1_OFF = 4 * TBYTES, O2_OFF = O1_OFF + OBYTES;
+  static constexpr int LDS_BYTES = O2_OFF + OBYTES;
+  static constexpr int WAVES_PER_EU = (LDS_BYTES > 80 * 1024) ? 1 : 2;
+};
+
+template <class T>
+__global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WAVES_PER_EU, T::WAVES_PER_EU)))
+void bwd_kernel(const BParams p) {
+  constexpr int D = T::D, ROLE = T::ROLE, TB = T::TB, BT = T::BT, KS = T::KS, DB = T::DB, NT = T::NT;
+  constexpr uint32_t FEAT = T::FEAT;
+  constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC;
+  constexpr bool kDQ = ROLE == ROLE_DQ;
+  constexpr float kLog2e = 1.4426950408889634f;
+  using L = TileLayout<D>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int r = lane % 32, h = lane / 32;
+
+  // workgroup -> (batch, owner head, owner tile); owner tiles of one head are consecutive
+  const int n_own = kDQ ? (p.Lq + T::OWN - 1) / T::OWN : (p.Lk + T::OWN - 1) / T::OWN;
+  const int oh = kDQ ? p.Hq : p.Hkv;
+  const int ot = blockIdx.x % n_own, bh = blockIdx.x / n_own;
+  const int ohead = bh % oh, batch = bh / oh;
+  const int o0 = ot * T::OWN;               // first owner position of the workgroup
+  const int o1 = min(o0 + T::OWN, kDQ ? p.Lq : p.Lk);
+  const int opos = o0 + wave * 32 + r;      // this lane's owner position (a query row or a key)
+  const int olen = kDQ ? p.Lq : p.Lk;
+  const int slen = kDQ ? p.Lk : p.Lq;       // streamed sequence length
+  const int kvh = kDQ ? ohead / p.group : ohead;
+
+  // ---- streamed tile range [t_lo, t_hi] for the workgroup's owner range [o0, o1) under the positional mask ----------
+  int t_lo = 0, t_hi = (slen + BT - 1) / BT - 1;
+  {
+    const bool causal_like = p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_SLIDING || p.mask_kind == MASK_DOC_CAUSAL;
+    if (kDQ) {  // keys attended by queries [o0, o1)
+      if (causal_like) t_hi = min(t_hi, (o1 - 1) / BT);
+      if (p.mask_kind == MASK_PREFIX) t_hi = min(t_hi, (max(o1, p.prefix) - 1) / BT);
+      if (p.mask_kind == MASK_SLIDING) t_lo = max(0, o0 - p.window) / BT;
+    } else {    // queries that attend keys [o0, o1)
+      if (causal_like) t_lo = o0 / BT;
+      if (p.mask_kind == MASK_PREFIX && o0 >= p.prefix) t_lo = o0 / BT;
+      if (p.mask_kind == MASK_SLIDING) t_hi = min(t_hi, (int)min((int64_t)o1 - 1 + p.window, (int64_t)slen - 1) / BT);
+    }
+  }
+  const int n_tiles = t_hi >= t_lo ? t_hi - t_lo + 1 : 0;
+  const int n_heads = kDQ ? 1 : p.group;   // ROLE_DKV walks the query heads of its group
+  const int n_steps = n_tiles * n_heads;
+
+  // ---- per-lane constants ---------------------------------------------------------------------------------------------
+  float cap_k1 = 0.f, cap_c = 0.f;
+  bool cap_on = false;  // kernels compiled with the soft-cap also serve calls without one
+  if constexpr (kSoftcap) {
+    cap_on = p.softcap > 0.f;
+    cap_k1 = cap_on ? p.scale / p.softcap * 2.0f * kLog2e : 0.f;
+    cap_c = p.softcap * kLog2e;
+  }
+  int64_t odoc = 0;
+  if constexpr (kDoc) odoc = p.doc_ids[(int64_t)batch * p.doc_stride + min(opos, olen - 1)];
+  int64_t own_mn = 0, own_mx = 0;
+  if constexpr (kDoc) doc_range(p.doc_table + (int64_t)batch * p.doc_blocks * 2, o0, o1, own_mn, own_mx);
+
+  // ---- owner operands ---------------------------------------------------------------------------------------------------
+  // ROLE_DQ: Q and dO fragments of this lane's query row live in registers (B operands), with its LSE and Delta.
+  // ROLE_DKV: the workgroup's K and V rows are staged in LDS once and read as B operands where they are used.
+  bf16x8 o1f[kDQ ? KS : 1], o2f[kDQ ? KS : 1];
+  float lse_o = 0.f, delta_o = 0.f;
+  const bf16_t* kptr = p.k + (int64_t)batch * p.ks[0] + (int64_t)kvh * p.ks[1];
+  const bf16_t* vptr = p.v + (int64_t)batch * p.vs[0] + (int64_t)kvh * p.vs[1];
+  if constexpr (kDQ) {
+    const int qr = min(opos, p.Lq - 1);
+    const bf16_t* qp = p.q + (int64_t)batch * p.qs[0] + (int64_t)ohead * p.qs[1] + (int64_t)qr * p.qs[2];
+    const bf16_t* dp = p.dout + (int64_t)batch * p.dos[0] + (int64_t)ohead * p.dos[1] + (int64_t)qr * p.dos[2];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      o1f[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16 + 8 * h);
+      o2f[ks] = *reinterpret_cast<const bf16x8*>(dp + ks * 16 + 8 * h);
+    }
+    const int64_t row = ((int64_t)batch * p.Hq + ohead) * p.Lq + qr;
+    lse_o = p.lse[row];
+    delta_o = p.delta[row];
+  }
+
+  // ---- global -> LDS transfers of a [rows][D] tile into its swizzled image ---------------------------------------------------
+  // lane l of a 1 KiB transfer writes LDS bytes [16 l, 16 l + 16); it fetches the logical chunk that the swizzle maps
+  // there.  Rows past `valid` repeat the last valid row (their contributions are masked).
+  auto load_tile = [&](const bf16_t* row0, int64_t stride, int valid, unsigned lds_off, int n_per_t) FL_INLINE {
+    const uint64_t base = uniform_ptr(row0);
+    const unsigned lds0 = (unsigned)(uintptr_t)smem + lds_off + wave * 1024;
+    for (int it = 0; it < n_per_t; ++it) {
+      const int id = it * NT + tid, row = id / L::CPR, pc = id % L::CPR;
+      const unsigned off = (unsigned)(min(row, valid - 1) * (int)stride + L::swz_k(row, pc) * 8) * 2u;
+      dma16(base, off, lds0 + it * NT * 16);
+    }
+  };
+  // streamed step s -> (query head of the group, tile)
+  auto step_head = [&](int s) FL_INLINE { return kDQ ? ohead : kvh * p.group + s / n_tiles; };
+  auto step_tile = [&](int s) FL_INLINE { return t_lo + (kDQ ? s : s % n_tiles); };
+  auto load_step = [&](int s, int slot) FL_INLINE {
+    const int t0 = step_tile(s) * BT, valid = min(BT, slen - t0);
+    if constexpr (kDQ) {
+      load_tile(kptr + (int64_t)t0 * p.ks[2], p.ks[2], valid, T::T1_OFF + slot * T::TBYTES, T::T_PER_T);
+      load_tile(vptr + (int64_t)t0 * p.vs[2], p.vs[2], valid, T::T2_OFF + slot * T::TBYTES, T::T_PER_T);
+    } else {
+      const int hd = step_head(s);
+      load_tile(p.q + (int64_t)batch * p.qs[0] + (int64_t)hd * p.qs[1] + (int64_t)t0 * p.qs[2], p.qs[2], valid,
+                T::T1_OFF + slot * T::TBYTES, T::T_PER_T);
+      load_tile(p.dout + (int64_t)batch * p.dos[0] + (int64_t)hd * p.dos[1] + (int64_t)t0 * p.dos[2], p.dos[2], valid,
+                T::T2_OFF + slot * T::TBYTES, T::T_PER_T);
+    }
+  };
+
+  // ---- LDS operand reads --------------------------------------------------------------------------------------------------
+  // row-wise: 8 consecutive elements [row][16 ks + 8 h, +8) (A operand of X1/X2 from a streamed tile, or B operand from
+  // an owner tile)
+  auto frag_row = [&](unsigned tile_off, int row, int ks) FL_INLINE -> bf16x8 {
+    return *reinterpret_cast<const bf16x8*>(smem + tile_off + row * (D * 2) + L::swz_k(row, 2 * ks + h) * 16);
+  };
+  // transposing: A operand of the accumulating products for 16-position chunk c and column block db; slot j of lane
+  // (r, h) is streamed position 16 c + 8 (j / 4) + 4 h + j % 4, the order in which the weights are packed
+  auto frag_tr = [&](unsigned tile_off, int c, int db) FL_INLINE -> bf16x8 {
+    bf16x8 f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i16 = lane % 16, g = (lane / 16) % 2;
+      const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
+      const int col = db * 32 + g * 16 + 4 * (i16 % 4);
+      const unsigned char* ap = smem + tile_off + row * (D * 2) + L::swz_k(row, col / 8) * 16 + (col % 8) * 2;
+      typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+      const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
+      const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f[4 * j + e] = b4[e];
+    }
+    return f;
+  };
+
+  f32x16 acc1[DB], acc2[kDQ ? 1 : DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc1[db][i] = 0.f;
+  if constexpr (!kDQ) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc2[db][i] = 0.f;
+  }
+
+  if (n_steps > 0) {
+    if constexpr (!kDQ) {
+      const int valid = o1 - o0;
+      load_tile(kptr + (int64_t)o0 * p.ks[2], p.ks[2], valid, T::O1_OFF, T::O_PER_T);
+      load_tile(vptr + (int64_t)o0 * p.vs[2], p.vs[2], valid, T::O2_OFF, T::O_PER_T);
+    }
+    load_step(0, 0);
+    dma_wait<0>();
+  }
+
+  for (int s = 0; s < n_steps; ++s) {
+    const int slot = s & 1;
+    __syncthreads();  // publishes slot `slot` (every wave waited for its own transfers) and frees the other slot
+    if (s + 1 < n_steps) load_step(s + 1, slot ^ 1);
+    const int t0 = step_tile(s) * BT;
+    const int shead = step_head(s);  // the query head of this step
+
+    // workgroup-level skip: nothing of this tile is attended by the workgroup's owner range (document ranges apart;
+    // positional emptiness inside [t_lo, t_hi] only occurs for a prefix-LM mask)
+    bool skip = false;
+    {
+      const int s1 = min(t0 + BT, slen);
+      const int qa = kDQ ? o0 : t0, qb_ = kDQ ? o1 : s1, ka = kDQ ? t0 : o0, kb_ = kDQ ? s1 : o1;
+      skip = classify_positional(p.mask_kind, qa, qb_, ka, kb_, p.window, p.prefix) == TILE_EMPTY;
+      if constexpr (kDoc) {
+        int64_t mn, mx;
+        doc_range(p.doc_table + (int64_t)batch * p.doc_blocks * 2, t0, s1, mn, mx);
+        skip = skip || mx < own_mn || mn > own_mx;
+      }
+    }
+    if (!skip) {
+      const unsigned t1 = T::T1_OFF + slot * T::TBYTES, t2 = T::T2_OFF + slot * T::TBYTES;
+      // ---- X1 = T1 . O1^T, X2 = T2 . O2^T ----------------------------------------------------------------------------------
+      f32x16 x1[TB], x2[TB];
+#pragma unroll
+      for (int sb = 0; sb < TB; ++sb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          x1[sb][i] = 0.f;
+          x2[sb][i] = 0.f;
+        }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        bf16x8 b1, b2;
+        if constexpr (kDQ) {
+          b1 = o1f[ks];
+          b2 = o2f[ks];
+        } else {
+          b1 = frag_row(T::O1_OFF, wave * 32 + r, ks);
+          b2 = frag_row(T::O2_OFF, wave * 32 + r, ks);
+        }
+#pragma unroll
+        for (int sb = 0; sb < TB; ++sb) {
+          x1[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t1, sb * 32 + r, ks), b1, x1[sb], 0, 0, 0);
+          x2[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t2, sb * 32 + r, ks), b2, x2[sb], 0, 0, 0);
+        }
+      }
+      // ---- P and dS in registers; register i of block sb is streamed position t0 + 32 sb + 8 (i / 4) + 4 h + i % 4 -------
+      float slope_l2 = 0.f;
+      if constexpr (kAlibi)
+        slope_l2 = p.alibi_heads > 0 ? exp2f(-8.0f * (float)(shead + 1) / (float)p.alibi_heads) * kLog2e : 0.f;
+      bf16x8 pf[2 * TB], dsf[2 * TB];
+#pragma unroll
+      for (int sb = 0; sb < TB; ++sb) {
+        const int sbase = t0 + 32 * sb + 4 * h;  // streamed position of register 0
+        // element predicate as an interval of the register offset `off` (8 (i / 4) + i % 4): lo <= off <= hi
+        int lo, hi;
+        if constexpr (kDQ) {
+          // streamed = key, owner = query: key < Lk && (dmin <= key - q <= dmax || key < pfx)
+          const int rel = sbase - opos;
+          hi = min(p.Lk - sbase - 1, max(p.dmax - rel, p.pfx - sbase - 1));
+          lo = p.dmin - rel;
+        } else {
+          // streamed = query, owner = key: q < Lq && (dmin <= key - q <= dmax || key < pfx), key = opos
+          const int rel = opos - sbase;  // key - q at off = 0; key - q = rel - off
+          hi = min(p.Lq - sbase - 1, opos < p.pfx ? (1 << 29) : rel - p.dmin);
+          lo = opos < p.pfx ? -(1 << 29) : rel - p.dmax;
+          if (opos >= p.Lk) hi = -(1 << 29);
+        }
+        // per-register row statistics of the streamed queries (ROLE_DKV)
+        float lse_s[kDQ ? 1 : 16], delta_s[kDQ ? 1 : 16];
+        int64_t sdoc[kDoc ? 16 : 1];
+        if constexpr (!kDQ) {
+          const int64_t row0 = ((int64_t)batch * p.Hq + shead) * p.Lq;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            // 4 consecutive rows; clamped reads past the end are masked below
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int qq = min(sbase + 8 * g + e, p.Lq - 1);
+              lse_s[4 * g + e] = p.lse[row0 + qq];
+              delta_s[4 * g + e] = p.delta[row0 + qq];
+            }
+          }
+        }
+        if constexpr (kDoc) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            sdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(sbase + 8 * (i / 4) + (i % 4), slen - 1)];
+        }
+        float pv[16], dv_[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int off = 8 * (i / 4) + (i % 4);
+          const float x = x1[sb][i];
+          float s2, dfac = 1.0f;  // logit in log2 units; d(score) / d(qk * scale)
+          if constexpr (kSoftcap) {
+            const float e = fast_exp2(x * cap_k1);
+            const float rc = fast_rcp(e + 1.0f);
+            const float th = __builtin_fmaf(rc, -2.0f, 1.0f);  // tanh(x * scale / cap)
+            s2 = cap_on ? th * cap_c : x * p.scale_log2;
+            dfac = cap_on ? __builtin_fmaf(-th, th, 1.0f) : 1.0f;
+          } else {
+            s2 = x * p.scale_log2;
+          }
+          if constexpr (kAlibi) {
+            const float rel_f = kDQ ? (float)(sbase + off - opos) : (float)(opos - sbase - off);
+            s2 = __builtin_fmaf(slope_l2, rel_f, s2);
+          }
+          bool ok = (off <= hi) & (off >= lo);
+          if constexpr (kDoc) ok = ok & (sdoc[i] == odoc);
+          const float lse = kDQ ? lse_o : lse_s[i];
+          const float dl = kDQ ? delta_o : delta_s[i];
+          const float pw = ok ? fast_exp2(s2 - lse) : 0.f;
+          pv[i] = pw;
+          dv_[i] = pw * (x2[sb][i] - dl) * dfac;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            pf[2 * sb + j][e] = (bf16_t)pv[8 * j + e];
+            dsf[2 * sb + j][e] = (bf16_t)dv_[8 * j + e];
+          }
+      }
+      // ---- acc1 += T1^T . dS,  acc2 += T2^T . P -------------------------------------------------------------------------------
+#pragma unroll
+      for (int c = 0; c < 2 * TB; ++c)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t1, c, db), dsf[c], acc1[db], 0, 0, 0);
+          if constexpr (!kDQ)
+            acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t2, c, db), pf[c], acc2[db], 0, 0, 0);
+        }
+    }
+    dma_wait<0>();
+  }
+
+  // ---- epilogue: register i of block db is column 32 db + 8 (i / 4) + 4 h + i % 4 of this lane's owner row ---------------
+  if (opos < olen) {
+    bf16_t* out1 = kDQ ? p.dq + (int64_t)batch * p.dqs[0] + (int64_t)ohead * p.dqs[1] + (int64_t)opos * p.dqs[2]
+                       : p.dk + (int64_t)batch * p.dks[0] + (int64_t)ohead * p.dks[1] + (int64_t)opos * p.dks[2];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 o4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)(acc1[db][4 * g + e] * p.scale);
+        *reinterpret_cast<bf16x4*>(out1 + 32 * db + 8 * g + 4 * h) = o4;
+      }
+    if constexpr (!kDQ) {
+      bf16_t* out2 = p.dv + (int64_t)batch * p.dvs[0] + (int64_t)ohead * p.dvs[1] + (int64_t)opos * p.dvs[2];
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          bf16x4 o4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)acc2[db][4 * g + e];
+          *reinterpret_cast<bf16x4*>(out2 + 32 * db + 8 * g + 4 * h) = o4;
+        }
+    }
+  }
+}
+
+}  // namespace fl

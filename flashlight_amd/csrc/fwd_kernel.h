@@ -78,6 +78,7 @@ struct KParams {
   float lambda;
   int64_t q_branch_stride, k_branch_stride;  // element offset of the second softmax branch (diff)
   uint8_t* dump;
+  float* lse;        // optional [B, Hq, Lq]: log2 of the row's sum of 2^(logit in log2 units); +inf if nothing attended
   int32_t n_qtiles;  // ceil(Lq / BM)
   int32_t n_ktiles;  // ceil(Lk / BN)
 };
@@ -1073,6 +1074,13 @@ void fwd_kernel(const KParams p) {
     for (int qb = 0; qb < QB; ++qb) {
       const float l = xhalf_sum(l_run[qb]);
       const float inv = l > 0.f ? 1.0f / l : 0.f;  // a row that attends nothing yields zeros
+      if constexpr (!kDiff) {
+        // row statistic for a backward pass: weights were exp2(s * c2 - m_run * c2), so the row's log2-sum-exp2 is
+        if (p.lse != nullptr && h == 0 && qrow[qb] < p.Lq) {
+          const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
+          p.lse[((int64_t)batch * p.Hq + head) * p.Lq + qrow[qb]] = l > 0.f ? mc + __builtin_log2f(l) : INFINITY;
+        }
+      }
       if constexpr (kDiff) {
         if (br == 0) {
 #pragma unroll

@@ -14,7 +14,7 @@ import torch
 
 from . import _ffi
 
-__all__ = ["attn_fwd", "dispatch"]
+__all__ = ["attn_fwd", "attn_fwd_lse", "attn_bwd", "dispatch"]
 
 
 def _out_shape(q: torch.Tensor, v: torch.Tensor, diff: bool):
@@ -52,9 +52,72 @@ def _attn_fwd_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_hea
     return _alloc_out(q, v, diff, seq_major_out)
 
 
+@torch.library.custom_op("flashlight_amd::attn_fwd_lse", mutates_args=())
+def attn_fwd_lse(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, mask_kind: int, window: int, prefix: int,
+                 doc_ids: Optional[torch.Tensor], alibi_heads: int, softcap: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """The forward for calls that will be differentiated: also returns the row statistics (float32 [B, Hq, Lq], log2 of
+    each row's sum of 2^logit) from which `attn_bwd` recomputes the weights.  The reference has no backward; this
+    operator carries the autograd rule registered below."""
+    out = _alloc_out(q, v, False, False)
+    lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
+    _ffi.attn_fwd(q, k, v, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window, prefix=prefix,
+                  doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, out=out, lse=lse)
+    return out, lse
+
+
+@attn_fwd_lse.register_fake
+def _attn_fwd_lse_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("query, key and value must be 4-D [batch, heads, seq, dim]")
+    return _alloc_out(q, v, False, False), torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
+
+
+@torch.library.custom_op("flashlight_amd::attn_bwd", mutates_args=())
+def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, dout: torch.Tensor,
+             scale: float, mask_kind: int, window: int, prefix: int, doc_ids: Optional[torch.Tensor], alibi_heads: int,
+             softcap: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dq, dk, dv) of `attn_fwd_lse` for the output gradient `dout`."""
+    return _ffi.attn_bwd(q, k, v, out, lse, dout, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window,
+                         prefix=prefix, doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap)
+
+
+@attn_bwd.register_fake
+def _attn_bwd_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap):
+    c = torch.contiguous_format
+    return torch.empty_like(q, memory_format=c), torch.empty_like(k, memory_format=c), torch.empty_like(v, memory_format=c)
+
+
+def _setup_context(ctx, inputs, output):
+    q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap = inputs
+    out, lse = output
+    ctx.save_for_backward(q, k, v, out, lse)
+    ctx.doc_ids = doc_ids
+    ctx.args = (scale, mask_kind, window, prefix, alibi_heads, softcap)
+
+
+def _backward(ctx, dout, dlse):
+    q, k, v, out, lse = ctx.saved_tensors
+    scale, mask_kind, window, prefix, alibi_heads, softcap = ctx.args
+    dq, dk, dv = attn_bwd(q, k, v, out, lse, dout.to(torch.bfloat16), scale, mask_kind, window, prefix, ctx.doc_ids,
+                          alibi_heads, softcap)
+    return dq, dk, dv, None, None, None, None, None, None, None
+
+
+attn_fwd_lse.register_autograd(_backward, setup_context=_setup_context)
+
+
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False) -> torch.Tensor:
-    """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise."""
+    """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise; the
+    differentiable operator when a gradient with respect to q, k or v will be asked for."""
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        if biases or gate is not None or diff or seq_major_out:
+            raise NotImplementedError(
+                "no backward is implemented for bias operands, the sigmoid gate or differential attention: call under "
+                "torch.no_grad() (or detach the inputs) if only the forward is wanted")
+        out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
+                              int(prefix), doc_ids, int(alibi_heads), float(softcap))
+        return out
     if torch.compiler.is_compiling():
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),

@@ -109,7 +109,11 @@ typedef struct fl_attn_params {
 
   int32_t bias_dtype[2]; /* enum fl_dtype of bias[0], bias[1]: FL_BF16 or FL_F32 */
 
-  int32_t reserved[6]; /* must be 0 */
+  /* Optional output for a later fl_attn_bwd: fp32 [B, Hq, Lq], contiguous; per query row the base-2 logarithm of
+   * the sum over attended keys of 2^(score * log2(e)) (+inf for a row that attends nothing).  Not with diff. */
+  float* lse;
+
+  int32_t reserved[4]; /* must be 0 */
 } fl_attn_params;
 
 /* ABI version of the loaded library (FL_ABI_VERSION it was built with). */
@@ -134,6 +138,37 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream);
 /* Describes the kernel instance fl_attn_fwd would pick for *p: tile sizes and launch shape.
  * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
 int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
+
+/* Backward of fl_attn_fwd.  No counterpart in the reference, which is forward-only (its FLOP helper models a
+ * backward pass, benchmarks/_utils.py:16-21, but no kernel or autograd rule exists): the textbook gradients of
+ * softmax attention, recomputing the weights from the forward's row statistics.
+ * `fwd` describes the forward call whose gradients are wanted: same q, k, v, sizes, scale, mask and score
+ * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
+ * kind, grouped-query heads, ALiBi, the tanh soft-cap; Dqk == Dv in {64, 128}.  Not supported (FL_ERR_UNSUPPORTED):
+ * bias operands, gate, differential attention, the attended_dump hook.
+ * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
+ * receive the gradients (bf16, strides in elements, last stride 1, others multiples of 8).
+ * delta: caller-provided scratch of B * Hq * Lq floats.  fwd.workspace as for the forward (document masks). */
+typedef struct fl_attn_bwd_params {
+  fl_attn_params fwd;
+  const void* dout;
+  int64_t dout_strides[4];
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t dq_strides[4], dk_strides[4], dv_strides[4];
+  float* delta;
+  int32_t reserved[8]; /* must be 0 */
+} fl_attn_bwd_params;
+
+/* sizeof(fl_attn_bwd_params) in the loaded library. */
+uint64_t fl_bwd_params_sizeof(void);
+
+/* Host-only argument check of a backward call. */
+int fl_attn_bwd_validate(const fl_attn_bwd_params* p);
+
+/* Launches the three backward kernels (row sums of dO o O, then dQ, then dK and dV) on `stream`. */
+int fl_attn_bwd(const fl_attn_bwd_params* p, void* stream);
 
 /* Measurement aid with no counterpart in the reference: launches a kernel that does nothing but issue
  * v_mfma_f32_32x32x16_bf16 (the instruction both products of the forward are built from) on operand fragments read

@@ -1,0 +1,209 @@
+"""Backward pass (dq, dk, dv).  The reference is forward-only, so there is nothing of its own to compare with: the
+checker is autograd through the CPU oracle's eager functions, which `test_oracle_gradients_against_finite_differences`
+pins against central differences in float64 (a wrong formula in the oracle, or in autograd's use of it, fails there).
+GPU tests compare the HIP kernels' gradients, through the C ABI, with those."""
+import ctypes as C
+
+import pytest
+import torch
+
+import flashlight_amd.attention_variants as A
+import oracle as O
+from flashlight_amd import _ffi
+from tests.conftest import assert_parity
+from tests.test_abi import good_params
+
+DEV = "cuda"
+
+
+# ---- the checker itself ----------------------------------------------------------------------------------------------------
+
+def _tiny(dtype=torch.float64, N=1, Hq=2, Hkv=1, L=5, E=4, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=dtype).requires_grad_(True)  # noqa: E731
+    return mk(N, Hq, L, E), mk(N, Hkv, L, E), mk(N, Hkv, L, E)
+
+
+@pytest.mark.parametrize("name,fn", [
+    ("vanilla", lambda q, k, v: O.attention_vanilla(q, k, v, enable_gqa=True)),
+    ("causal", lambda q, k, v: O.attention_causal(q, k, v, enable_gqa=True)),
+    ("sliding", lambda q, k, v: O.attention_sliding_window(q, k, v, window_size=2, enable_gqa=True)),
+    ("prefix", lambda q, k, v: O.attention_prefix_lm(q, k, v, prefix_lengths=3, enable_gqa=True)),
+    ("document", lambda q, k, v: O.attention_document_mask(q, k, v, torch.tensor([[0, 0, 1, 1, 1]]), enable_gqa=True,
+                                                           is_causal=True)),
+    ("alibi+softcap", lambda q, k, v: O.attention_alibi(q, k, v, score_mod=2, enable_gqa=True, softcap=1.5,
+                                                        is_causal=True, honor_causal=True)),
+    ("softcap", lambda q, k, v: O.attention_softcapped(q, k, v, score_mod=0.7, enable_gqa=True)),
+])
+def test_oracle_gradients_against_finite_differences(name, fn):
+    q, k, v = _tiny()
+    assert torch.autograd.gradcheck(lambda a, b, c: fn(a, b, c), (q, k, v), eps=1e-6, atol=1e-5, rtol=1e-4), name
+
+
+def test_backward_abi_validation():
+    lib = _ffi.load_library()
+    assert lib.fl_bwd_params_sizeof() == C.sizeof(_ffi.FlAttnBwdParams)
+
+    def params(**kw):
+        b = _ffi.FlAttnBwdParams()
+        b.fwd = good_params(**kw)
+        L, D, Hq, Hkv = b.fwd.Lq, b.fwd.Dqk, b.fwd.Hq, b.fwd.Hkv
+        b.fwd.lse = 0x90000
+        b.dout, b.dq, b.dk, b.dv, b.delta = 0xA0000, 0xB0000, 0xC0000, 0xD0000, 0xE0000
+        b.dout_strides[:] = (Hq * L * D, L * D, D, 1)
+        b.dq_strides[:] = (Hq * L * D, L * D, D, 1)
+        b.dk_strides[:] = (Hkv * L * D, L * D, D, 1)
+        b.dv_strides[:] = (Hkv * L * D, L * D, D, 1)
+        return b
+
+    rc = lambda b: lib.fl_attn_bwd_validate(C.byref(b))  # noqa: E731
+    for D in (64, 128):
+        assert rc(params(D=D)) == 0, _ffi.last_error()
+    assert lib.fl_attn_bwd_validate(None) == -1
+    cases = [
+        (lambda b: setattr(b.fwd, "lse", 0), -1, "lse"),
+        (lambda b: setattr(b, "delta", 0), -1, "delta"),
+        (lambda b: setattr(b, "dout", 0xA0008), -7, "dout"),
+        (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),
+        (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1)), -4, "not supported"),
+        (lambda b: (setattr(b.fwd, "gate", 0x70000), b.fwd.gate_strides.__setitem__(slice(0, 4), list(b.fwd.o_strides))),
+         -4, "not supported"),
+        (lambda b: b.reserved.__setitem__(3, 1), -5, "reserved"),
+        (lambda b: setattr(b.fwd, "scale", -1.0), -5, "scale"),
+    ]
+    for mutate, code, word in cases:
+        b = params()
+        mutate(b)
+        assert rc(b) == code and word in _ffi.last_error(), (_ffi.last_error(), word)
+        assert lib.fl_attn_bwd(C.byref(b), None) == code  # the same check runs before any launch
+    b = params(D=32)
+    assert rc(b) == -4 and "head dim" in _ffi.last_error()
+    b = params(D=64, Dv=128)
+    b.fwd.diff = 0
+    assert rc(b) == -4
+
+
+def test_front_end_refuses_to_differentiate_what_has_no_backward():
+    # checked before anything touches a GPU
+    q = torch.randn(1, 3, 16, 2, 32).bfloat16().requires_grad_(True)
+    with pytest.raises(NotImplementedError, match="no backward"):
+        A.attention_reference(q, q, q, [torch.zeros(1, 1, 2, 16, 16).bfloat16()])
+    qd = torch.randn(1, 4, 16, 64).bfloat16().requires_grad_(True)
+    with pytest.raises(NotImplementedError, match="no backward"):
+        A.diffattn(qd, qd, torch.randn(1, 2, 16, 128).bfloat16())
+
+
+# ---- the kernels ---------------------------------------------------------------------------------------------------------------
+
+def _inputs(B, Hq, Hkv, L, D, seed, S=None):
+    g = torch.Generator().manual_seed(seed)
+    S = S or L
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)  # noqa: E731
+    return mk(B, Hq, L, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, L, D)
+
+
+def _grads(fn, q, k, v, dout, dtype):
+    q, k, v = (t.detach().to(dtype).requires_grad_(True) for t in (q, k, v))
+    out = fn(q, k, v)
+    out.backward(dout.to(out.dtype).reshape(out.shape))
+    return out.detach(), q.grad, k.grad, v.grad
+
+
+def _check(name, hip_fn, oracle_fn, q, k, v, dout):
+    out, dq, dk, dv = _grads(hip_fn, q, k, v, dout, torch.bfloat16)
+    ref, rq, rk, rv = _grads(oracle_fn, q, k, v, dout, torch.float32)
+    torch.cuda.synchronize()
+    assert_parity(out.reshape(ref.shape), ref, f"{name}: forward")
+    for what, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        assert got.dtype == torch.bfloat16 and got.shape == want.shape
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{name}: {what}")
+
+
+VARIANTS = {
+    "vanilla": (lambda q, k, v: A.attention_pytorch(q, k, v, enable_gqa=True),
+                lambda q, k, v: O.attention_vanilla(q, k, v, enable_gqa=True)),
+    "causal": (lambda q, k, v: A.attention_pytorch_causal(q, k, v, enable_gqa=True),
+               lambda q, k, v: O.attention_causal(q, k, v, enable_gqa=True)),
+    "sliding": (lambda q, k, v: A.attention_pytorch_sliding_window(q, k, v, window_size=37, enable_gqa=True),
+                lambda q, k, v: O.attention_sliding_window(q, k, v, window_size=37, enable_gqa=True)),
+    "prefix": (lambda q, k, v: A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=70, enable_gqa=True),
+               lambda q, k, v: O.attention_prefix_lm(q, k, v, prefix_lengths=70, enable_gqa=True)),
+    "alibi": (lambda q, k, v: A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(q.size(1)),
+                                                        enable_gqa=True),
+              lambda q, k, v: O.attention_alibi(q, k, v, score_mod=q.size(1), enable_gqa=True)),
+    "softcap": (lambda q, k, v: A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(2.0), enable_gqa=True,
+                                                       is_causal=True),
+                lambda q, k, v: O.attention_softcapped(q, k, v, score_mod=2.0, enable_gqa=True, is_causal=True,
+                                                       honor_causal=True)),
+    "alibi+softcap+causal": (
+        lambda q, k, v: A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(q.size(1)),
+                                                  enable_gqa=True, is_causal=True, softcap=5.0),
+        lambda q, k, v: O.attention_alibi(q, k, v, score_mod=q.size(1), enable_gqa=True, is_causal=True,
+                                          honor_causal=True, softcap=5.0)),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name", sorted(VARIANTS))
+def test_gradients_match_the_oracle(name, D):
+    hip_fn, oracle_fn = VARIANTS[name]
+    # 300 rows: two full owner tiles and a ragged one; 4 query heads on 2 key/value heads
+    q, k, v, dout = _inputs(2, 4, 2, 300, D, seed=sum(map(ord, name)) + D)
+    _check(f"{name} D={D}", hip_fn, oracle_fn, q, k, v, dout)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_gradients_document_mask(D, causal):
+    q, k, v, dout = _inputs(2, 4, 2, 333, D, seed=77 + D)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 5, (2, 333), generator=g).sort(dim=1).values.to(DEV)
+    _check(f"document causal={causal} D={D}",
+           lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal),
+           lambda q, k, v: O.attention_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal), q, k, v, dout)
+    # ids in no order: every tile pair has to be looked at
+    ids = torch.randint(0, 3, (2, 333), generator=g).to(DEV)
+    _check(f"document unsorted D={D}",
+           lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal),
+           lambda q, k, v: O.attention_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal), q, k, v, dout)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L,S", [(1, 1), (31, 31), (64, 200), (200, 64), (129, 257), (1000, 1000)])
+def test_gradients_ragged_and_cross_lengths(L, S):
+    for D in (64, 128):
+        q, k, v, dout = _inputs(1, 2, 2, L, D, seed=L + S + D, S=S)
+        _check(f"vanilla {L}x{S} D={D}", lambda q, k, v: A.attention_pytorch(q, k, v),
+               lambda q, k, v: O.attention_vanilla(q, k, v), q, k, v, dout)
+        _check(f"causal {L}x{S} D={D}", lambda q, k, v: A.attention_pytorch_causal(q, k, v),
+               lambda q, k, v: O.attention_causal(q, k, v), q, k, v, dout)
+
+
+@pytest.mark.gpu
+def test_gradient_properties_at_benchmark_size():
+    # B=1 H=4 S=4096 D=128 causal: too large for the CPU oracle in a test, so check what the mathematics fixes:
+    # (1) dv is linear in dout; (2) sum_k dk . k == sum_q dq . q (both equal sum_{q,k} dS[q,k] S[q,k] / scale, since the
+    # logits are bilinear in q and k); (3) a row's dq is orthogonal to nothing in particular, but dout = 0 gives zeros
+    g = torch.Generator().manual_seed(9)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)  # noqa: E731
+    q, k, v, d1, d2 = mk(1, 4, 4096, 128), mk(1, 4, 4096, 128), mk(1, 4, 4096, 128), mk(1, 4, 4096, 128), mk(1, 4, 4096, 128)
+
+    def grads(dout):
+        qq, kk, vv = (t.detach().requires_grad_(True) for t in (q, k, v))
+        A.attention_pytorch_causal(qq, kk, vv).backward(dout)
+        return qq.grad.float(), kk.grad.float(), vv.grad.float()
+
+    q1, k1, v1 = grads(d1)
+    q2, k2, v2 = grads(d2)
+    q3, k3, v3 = grads((d1.float() + d2.float()).to(torch.bfloat16))
+    # dout is rounded to bf16 once more in the third call; gradients are O(1)
+    assert (v3 - (v1 + v2)).abs().max().item() < 6e-2 and (v3 - (v1 + v2)).abs().mean().item() < 4e-3
+    lhs, rhs = (q1 * q.float()).sum().item(), (k1 * k.float()).sum().item()
+    assert abs(lhs - rhs) <= 2e-2 * max(abs(lhs), abs(rhs), 1.0), (lhs, rhs)
+    z = grads(torch.zeros_like(d1))
+    assert all(float(t.abs().max()) == 0.0 for t in z)
+    # row 0 attends only key 0, with weight 1 whatever q is: its dq is zero and dv[0] collects dout[0] in full
+    assert float(q1[0, :, 0].abs().max()) < 1e-6

@@ -148,11 +148,13 @@ def write_results_csv(rows: List[tuple], path: str) -> None:
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer", "ipa"), default="variants",
+    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer", "ipa", "backward"), default="variants",
                     help="variants: run_flex_variants.py; diffattn: run_diff_attn.py (model dim 2048, head dims 64 and "
                          "128, published FLOP estimate 8 B S^2 H D); evoformer: run_evoformer.py (N_seq = S = 256, 4 "
                          "heads, mask bias + pair bias, FLOPs 4 B 256 S^2 H D); ipa: invariant point attention of "
-                         "tests/test_ipa.py at 12 heads x (16 scalar + 4 query/key points + 8 value points)")
+                         "tests/test_ipa.py at 12 heads x (16 scalar + 4 query/key points + 8 value points); backward: the "
+                         "gradient kernels alone (dq, dk, dv from saved output and row statistics), FLOPs = 2.5 x the "
+                         "forward's as in benchmarks/_utils.py:16-21")
     ap.add_argument("--filter", type=str, nargs="+", default=[], help="keywords of variants to benchmark")
     ap.add_argument("--batch_size", type=int, nargs="+", default=DEFAULTS["batch_sizes"])
     ap.add_argument("--seqlen", type=int, nargs="+", default=DEFAULTS["seq_lengths"])
@@ -163,9 +165,9 @@ def parse_args(argv=None):
     ap.add_argument("--output", type=str, default="benchmark", help="output file name, `.csv` is appended")
     a = ap.parse_args(argv)
     if a.dim is None:
-        a.dim = DEFAULTS["model_dim"] if a.suite == "variants" else 2048
+        a.dim = DEFAULTS["model_dim"] if a.suite in ("variants", "backward") else 2048
     if a.headdim is None:
-        a.headdim = DEFAULTS["head_dims"] if a.suite == "variants" else [16] if a.suite == "ipa" else [64, 128]
+        a.headdim = DEFAULTS["head_dims"] if a.suite in ("variants", "backward") else [16] if a.suite == "ipa" else [64, 128]
     return a
 
 
@@ -178,7 +180,7 @@ def main(argv=None) -> List[tuple]:
     torch.manual_seed(0)
     rows: List[tuple] = []
     if args.suite != "variants":
-        rows = _run_other_suite(args)
+        rows = _run_backward_suite(args) if args.suite == "backward" else _run_other_suite(args)
         write_results_csv(rows, f"{args.output}.csv")
         return rows
     variants = registry()
@@ -197,6 +199,46 @@ def main(argv=None) -> List[tuple]:
                     rows.append((name, ms, tflops, *config))
                     print(f"{name:28s} {ms:9.4f} ms {tflops:8.1f} TFLOP/s")
     write_results_csv(rows, f"{args.output}.csv")
+    return rows
+
+
+def _run_backward_suite(args) -> List[tuple]:
+    """Times fl_attn_bwd alone for the variants that have a backward, on the sweep's shapes.  The reference has no
+    backward to compare with; its FLOP helper's "bwd" mode (2.5 x forward, benchmarks/_utils.py:16-21) and the same
+    128-block accounting as the forward sweep give the TFLOP/s column."""
+    import torch
+
+    from flashlight_amd import _ffi
+    from flashlight_amd.attention_variants.document_mask import create_document_id
+
+    rows: List[tuple] = []
+    for group_size in args.group_size:
+        for headdim in args.headdim:
+            for batch, seqlen in zip(args.batch_size, args.seqlen):
+                nheads = args.dim // headdim
+                config = (batch, seqlen, nheads, headdim, group_size, args.dropout_p)
+                print(f"### Config: {config} ###")
+                q, k, v = make_qkv(batch, seqlen, nheads, headdim, group_size)
+                dout = torch.randn_like(q)
+                cases = {  # the forward sweep's names and parameters (registry() above)
+                    "full": {},
+                    "full_with_alibi": dict(alibi_heads=nheads),
+                    "full_with_softcap": dict(softcap=30.0),
+                    "full_with_causal": dict(mask_kind=_ffi.MASK_CAUSAL),
+                    "full_with_sliding_window": dict(mask_kind=_ffi.MASK_SLIDING, window=256),
+                    "full_with_prefix_lm": dict(mask_kind=_ffi.MASK_PREFIX_LM, prefix=256),
+                    "full_with_document_mask": dict(mask_kind=_ffi.MASK_DOCUMENT,
+                                                    doc_ids=create_document_id(batch, seqlen, num_docs=12)),
+                }
+                for name, kw in cases.items():
+                    if args.filter and all(key not in name for key in args.filter):
+                        continue
+                    lse = torch.empty(batch, nheads, seqlen, dtype=torch.float32, device="cuda")
+                    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+                    ms = time_forward(lambda: _ffi.attn_bwd(q, k, v, out, lse, dout, **kw))
+                    tflops = 2.5 * variant_flops(name, batch, seqlen, nheads, headdim) / ms / 1e9
+                    rows.append((name + "_bwd", ms, tflops, *config))
+                    print(f"{name + '_bwd':28s} {ms:9.4f} ms {tflops:8.1f} TFLOP/s")
     return rows
 
 

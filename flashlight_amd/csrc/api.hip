@@ -353,9 +353,9 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
     return fail(FL_ERR_UNSUPPORTED, "backward: bias operands, gate, differential attention and the dump hook are not supported");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
-  if (!p->lse) return fail(FL_ERR_NULL, "backward: fwd.lse (the forward's row statistics) is null");
   if ((rc = check_ptr("dout", b->dout, 16)) || (rc = check_ptr("dq", b->dq, 8)) || (rc = check_ptr("dk", b->dk, 8)) ||
-      (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 4)))
+      (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 16)) ||
+      (rc = check_ptr("fwd.lse", p->lse, 16)))
     return rc;
   if ((rc = check_strides("dout", b->dout_strides, 8)) || (rc = check_strides("dq", b->dq_strides, 4)) ||
       (rc = check_strides("dk", b->dk_strides, 4)) || (rc = check_strides("dv", b->dv_strides, 4)) ||

@@ -101,10 +101,22 @@ void bwd_kernel(const BParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
   const int r = lane % 32, h = lane / 32;
 
-  // workgroup -> (batch, owner head, owner tile); owner tiles of one head are consecutive
+  // workgroup -> (batch, owner head, owner tile).  Without a mask every owner tile costs the same and the tiles of one
+  // head are consecutive (they share the streamed operands in L2).  Under causal-like masks the work of a tile grows
+  // with the query position (ROLE_DQ) or shrinks with the key position (ROLE_DKV): the longest tiles of every head go
+  // first, so that the grid drains on short ones.
   const int n_own = kDQ ? (p.Lq + T::OWN - 1) / T::OWN : (p.Lk + T::OWN - 1) / T::OWN;
   const int oh = kDQ ? p.Hq : p.Hkv;
-  const int ot = blockIdx.x % n_own, bh = blockIdx.x / n_own;
+  int ot, bh;
+  if (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || p.mask_kind == MASK_DOC_CAUSAL) {
+    const int nbh = p.B * oh;
+    const int rank = blockIdx.x / nbh;  // 0 = longest
+    bh = blockIdx.x % nbh;
+    ot = kDQ ? n_own - 1 - rank : rank;
+  } else {
+    ot = blockIdx.x % n_own;
+    bh = blockIdx.x / n_own;
+  }
   const int ohead = bh % oh, batch = bh / oh;
   const int o0 = ot * T::OWN;               // first owner position of the workgroup
   const int o1 = min(o0 + T::OWN, kDQ ? p.Lq : p.Lk);
@@ -317,12 +329,24 @@ void bwd_kernel(const BParams p) {
           const int64_t row0 = ((int64_t)batch * p.Hq + shead) * p.Lq;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            // 4 consecutive rows; clamped reads past the end are masked below
+            // registers 4 g .. 4 g + 3 are 4 consecutive rows: one 16-byte load each when the rows are aligned and
+            // inside the sequence, else element by element (clamped reads past the end are masked below)
+            const int q4 = sbase + 8 * g;
+            if (p.Lq % 4 == 0 && q4 + 3 < p.Lq) {
+              const f32x4 l4 = *reinterpret_cast<const f32x4*>(p.lse + row0 + q4);
+              const f32x4 d4 = *reinterpret_cast<const f32x4*>(p.delta + row0 + q4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int qq = min(sbase + 8 * g + e, p.Lq - 1);
-              lse_s[4 * g + e] = p.lse[row0 + qq];
-              delta_s[4 * g + e] = p.delta[row0 + qq];
+              for (int e = 0; e < 4; ++e) {
+                lse_s[4 * g + e] = l4[e];
+                delta_s[4 * g + e] = d4[e];
+              }
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int qq = min(q4 + e, p.Lq - 1);
+                lse_s[4 * g + e] = p.lse[row0 + qq];
+                delta_s[4 * g + e] = p.delta[row0 + qq];
+              }
             }
           }
         }

@@ -148,7 +148,8 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * bias operands, gate, differential attention, the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
  * receive the gradients (bf16, strides in elements, last stride 1, others multiples of 8).
- * delta: caller-provided scratch of B * Hq * Lq floats.  fwd.workspace as for the forward (document masks). */
+ * delta: caller-provided scratch of B * Hq * Lq floats; delta and fwd.lse must be 16-byte aligned.
+ * fwd.workspace as for the forward (document masks). */
 typedef struct fl_attn_bwd_params {
   fl_attn_params fwd;
   const void* dout;

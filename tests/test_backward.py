@@ -62,6 +62,7 @@ def test_backward_abi_validation():
     assert lib.fl_attn_bwd_validate(None) == -1
     cases = [
         (lambda b: setattr(b.fwd, "lse", 0), -1, "lse"),
+        (lambda b: setattr(b.fwd, "lse", 0x90004), -7, "lse"),
         (lambda b: setattr(b, "delta", 0), -1, "delta"),
         (lambda b: setattr(b, "dout", 0xA0008), -7, "dout"),
         (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),

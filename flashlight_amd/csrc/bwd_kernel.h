@@ -72,18 +72,28 @@ template <int D_, int ROLE_, uint32_t FEAT_>
 struct BwdTraits {
   static constexpr int D = D_, ROLE = ROLE_;
   static constexpr uint32_t FEAT = FEAT_;
-  static constexpr int NW = 4, NT = 256, OWN = 128;        // waves, threads, owner positions per workgroup
-  static constexpr int TB = (ROLE == ROLE_DQ && D_ <= 64) ? 2 : 1;  // 32-position blocks per streamed tile (register budget)
-  static constexpr int BT = 32 * TB;
+  static constexpr int OWN = 128;                          // owner positions per workgroup: 4 waves x 32
+  // ROLE_DKV at D = 128 holds 128 accumulator registers per lane; to still run two waves per SIMD its workgroup has
+  // 8 waves, two per owner block, which take the two halves of every streamed tile and add up their partial sums
+  // through LDS at the end (one workgroup per CU, 128 KB of LDS).
+  static constexpr int QH = (ROLE == ROLE_DKV && D_ > 64) ? 2 : 1;   // waves per owner block
+  static constexpr int NW = 4 * QH, NT = 64 * NW;
+  static constexpr int TB = (ROLE == ROLE_DQ && D_ <= 64) ? 2 : 1;  // 32-position blocks per wave and step (register budget)
+  static constexpr int BT = 32 * TB * QH;                  // streamed positions per step
   static constexpr int KS = D / 16, DB = D / 32;
   static constexpr int TBYTES = BT * D * 2;                // one streamed tile
   static constexpr int T_PER_T = TBYTES / (NT * 16);       // 16-byte transfers per thread per tile
   static_assert(TBYTES % (NT * 16) == 0, "streamed tile must divide evenly over the threads");
   static constexpr int OBYTES = (ROLE == ROLE_DKV) ? OWN * D * 2 : 0;  // owner tile kept in LDS (ROLE_DKV: K and V)
   static constexpr int O_PER_T = OBYTES / (NT * 16);
-  static constexpr int T1_OFF = 0, T2_OFF = 2 * TBYTES, O1_OFF = 4 * TBYTES, O2_OFF = O1_OFF + OBYTES;
-  static constexpr int LDS_BYTES = O2_OFF + OBYTES;
-  static constexpr int WAVES_PER_EU = (LDS_BYTES > 80 * 1024) ? 1 : 2;
+  static_assert(OBYTES % (NT * 16) == 0, "owner tile must divide evenly over the threads");
+  // ROLE_DKV also stages the streamed rows' statistics (LSE and Delta, fp32) with every tile: 1 KiB each per slot
+  static constexpr int SBYTES = (ROLE == ROLE_DKV) ? 1024 : 0;
+  static constexpr int T1_OFF = 0, T2_OFF = 2 * TBYTES, O1_OFF = 4 * TBYTES, O2_OFF = O1_OFF + OBYTES,
+                       S1_OFF = O2_OFF + OBYTES, S2_OFF = S1_OFF + 2 * SBYTES;
+  static constexpr int LDS_BYTES = S2_OFF + 2 * SBYTES;
+  static_assert(QH == 1 || LDS_BYTES >= 4 * 64 * 64 * 4, "the partial sums of one accumulator set must fit in LDS");
+  static constexpr int WAVES_PER_EU = 2;
 };
 
 template <class T>
@@ -100,27 +110,36 @@ void bwd_kernel(const BParams p) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
   const int r = lane % 32, h = lane / 32;
+  const int ow = wave % 4;       // owner block of this wave
+  const int qh = wave / 4;       // which part of every streamed tile this wave takes (0 unless QH == 2)
 
-  // workgroup -> (batch, owner head, owner tile).  Without a mask every owner tile costs the same and the tiles of one
-  // head are consecutive (they share the streamed operands in L2).  Under causal-like masks the work of a tile grows
-  // with the query position (ROLE_DQ) or shrinks with the key position (ROLE_DKV): the longest tiles of every head go
-  // first, so that the grid drains on short ones.
+  // workgroup -> (batch, owner head, owner tile).  All owner tiles of one head stream the same tensors, so they should
+  // run at the same time on one XCD (its L2 then serves all but the first read): consecutive workgroup ids land on
+  // different XCDs, hence ids are regrouped to give every XCD a contiguous run of (batch, head) pairs, head by head.
+  // Under causal-like masks the work of a tile grows with the query position (ROLE_DQ) or shrinks with the key position
+  // (ROLE_DKV): heads are taken four at a time and their tiles dealt longest first, so the grid drains on short ones.
   const int n_own = kDQ ? (p.Lq + T::OWN - 1) / T::OWN : (p.Lk + T::OWN - 1) / T::OWN;
   const int oh = kDQ ? p.Hq : p.Hkv;
   int ot, bh;
-  if (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || p.mask_kind == MASK_DOC_CAUSAL) {
+  {
     const int nbh = p.B * oh;
-    const int rank = blockIdx.x / nbh;  // 0 = longest
-    bh = blockIdx.x % nbh;
+    int i = blockIdx.x, run = nbh, base = 0;
+    if (nbh % 8 == 0) {
+      run = nbh / 8;
+      base = (i % 8) * run;
+      i /= 8;
+    }
+    const int G = (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || p.mask_kind == MASK_DOC_CAUSAL) ? 4 : 1;
+    const int g = i / (G * n_own), rem = i % (G * n_own);
+    const int gg = min(G, run - G * g);
+    const int rank = rem / gg;  // 0 = longest under a causal-like mask
+    bh = base + G * g + rem % gg;
     ot = kDQ ? n_own - 1 - rank : rank;
-  } else {
-    ot = blockIdx.x % n_own;
-    bh = blockIdx.x / n_own;
   }
   const int ohead = bh % oh, batch = bh / oh;
   const int o0 = ot * T::OWN;               // first owner position of the workgroup
   const int o1 = min(o0 + T::OWN, kDQ ? p.Lq : p.Lk);
-  const int opos = o0 + wave * 32 + r;      // this lane's owner position (a query row or a key)
+  const int opos = o0 + ow * 32 + r;        // this lane's owner position (a query row or a key)
   const int olen = kDQ ? p.Lq : p.Lk;
   const int slen = kDQ ? p.Lk : p.Lq;       // streamed sequence length
   const int kvh = kDQ ? ohead / p.group : ohead;
@@ -185,10 +204,13 @@ void bwd_kernel(const BParams p) {
     const unsigned lds0 = (unsigned)(uintptr_t)smem + lds_off + wave * 1024;
     for (int it = 0; it < n_per_t; ++it) {
       const int id = it * NT + tid, row = id / L::CPR, pc = id % L::CPR;
-      const unsigned off = (unsigned)(min(row, valid - 1) * (int)stride + L::swz_k(row, pc) * 8) * 2u;
+      const unsigned off = (unsigned)(min(row, valid - 1) * (int)stride + L::swz_kv(row, pc) * 8) * 2u;
       dma16(base, off, lds0 + it * NT * 16);
     }
   };
+  // ROLE_DKV: the statistics of the streamed rows ride the tile transfers when every row block starts on a 16-byte
+  // boundary (then a tile's valid rows are a multiple of 4 too); otherwise they are read from global memory in place
+  const bool stats_staged = !kDQ && p.Lq % 4 == 0;
   // streamed step s -> (query head of the group, tile)
   auto step_head = [&](int s) FL_INLINE { return kDQ ? ohead : kvh * p.group + s / n_tiles; };
   auto step_tile = [&](int s) FL_INLINE { return t_lo + (kDQ ? s : s % n_tiles); };
@@ -203,6 +225,15 @@ void bwd_kernel(const BParams p) {
                 T::T1_OFF + slot * T::TBYTES, T::T_PER_T);
       load_tile(p.dout + (int64_t)batch * p.dos[0] + (int64_t)hd * p.dos[1] + (int64_t)t0 * p.dos[2], p.dos[2], valid,
                 T::T2_OFF + slot * T::TBYTES, T::T_PER_T);
+      if (stats_staged && wave == 0) {
+        // one wave brings both arrays (every wave waits for all of its own transfers before the barrier, so the
+        // counts need not match).  Lane l fetches rows 4 l .. 4 l + 3; lanes past the end of the sequence repeat its
+        // last four rows.
+        const int64_t row0 = ((int64_t)batch * p.Hq + hd) * p.Lq + t0;
+        const unsigned off = (unsigned)min(lane, valid / 4 - 1) * 16u;
+        dma16(uniform_ptr(p.lse + row0), off, (unsigned)(uintptr_t)smem + T::S1_OFF + slot * T::SBYTES);
+        dma16(uniform_ptr(p.delta + row0), off, (unsigned)(uintptr_t)smem + T::S2_OFF + slot * T::SBYTES);
+      }
     }
   };
 
@@ -210,7 +241,7 @@ void bwd_kernel(const BParams p) {
   // row-wise: 8 consecutive elements [row][16 ks + 8 h, +8) (A operand of X1/X2 from a streamed tile, or B operand from
   // an owner tile)
   auto frag_row = [&](unsigned tile_off, int row, int ks) FL_INLINE -> bf16x8 {
-    return *reinterpret_cast<const bf16x8*>(smem + tile_off + row * (D * 2) + L::swz_k(row, 2 * ks + h) * 16);
+    return *reinterpret_cast<const bf16x8*>(smem + tile_off + row * (D * 2) + L::swz_kv(row, 2 * ks + h) * 16);
   };
   // transposing: A operand of the accumulating products for 16-position chunk c and column block db; slot j of lane
   // (r, h) is streamed position 16 c + 8 (j / 4) + 4 h + j % 4, the order in which the weights are packed
@@ -221,7 +252,7 @@ void bwd_kernel(const BParams p) {
       const int i16 = lane % 16, g = (lane / 16) % 2;
       const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
       const int col = db * 32 + g * 16 + 4 * (i16 % 4);
-      const unsigned char* ap = smem + tile_off + row * (D * 2) + L::swz_k(row, col / 8) * 16 + (col % 8) * 2;
+      const unsigned char* ap = smem + tile_off + row * (D * 2) + L::swz_kv(row, col / 8) * 16 + (col % 8) * 2;
       typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
       const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
       const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
@@ -262,149 +293,186 @@ void bwd_kernel(const BParams p) {
 
     // workgroup-level skip: nothing of this tile is attended by the workgroup's owner range (document ranges apart;
     // positional emptiness inside [t_lo, t_hi] only occurs for a prefix-LM mask)
-    bool skip = false;
+    bool skip = false, full = false;
+    bool doc_uniform = false;  // every position of the tile and of the owner range carries one and the same document id
     {
       const int s1 = min(t0 + BT, slen);
       const int qa = kDQ ? o0 : t0, qb_ = kDQ ? o1 : s1, ka = kDQ ? t0 : o0, kb_ = kDQ ? s1 : o1;
-      skip = classify_positional(p.mask_kind, qa, qb_, ka, kb_, p.window, p.prefix) == TILE_EMPTY;
+      const int cls = classify_positional(p.mask_kind, qa, qb_, ka, kb_, p.window, p.prefix);
+      skip = cls == TILE_EMPTY;
+      // every pair of the step attended: the positional mask holds everywhere and both ranges lie inside the sequences
+      full = cls == TILE_FULL && t0 + BT <= slen && o0 + T::OWN <= olen;
       if constexpr (kDoc) {
         int64_t mn, mx;
         doc_range(p.doc_table + (int64_t)batch * p.doc_blocks * 2, t0, s1, mn, mx);
         skip = skip || mx < own_mn || mn > own_mx;
+        doc_uniform = mn == mx && own_mn == own_mx && mn == own_mn;
+        full = full && doc_uniform;
       }
     }
     if (!skip) {
       const unsigned t1 = T::T1_OFF + slot * T::TBYTES, t2 = T::T2_OFF + slot * T::TBYTES;
-      // ---- X1 = T1 . O1^T, X2 = T2 . O2^T ----------------------------------------------------------------------------------
-      f32x16 x1[TB], x2[TB];
-#pragma unroll
-      for (int sb = 0; sb < TB; ++sb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          x1[sb][i] = 0.f;
-          x2[sb][i] = 0.f;
-        }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        bf16x8 b1, b2;
-        if constexpr (kDQ) {
-          b1 = o1f[ks];
-          b2 = o2f[ks];
-        } else {
-          b1 = frag_row(T::O1_OFF, wave * 32 + r, ks);
-          b2 = frag_row(T::O2_OFF, wave * 32 + r, ks);
-        }
-#pragma unroll
-        for (int sb = 0; sb < TB; ++sb) {
-          x1[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t1, sb * 32 + r, ks), b1, x1[sb], 0, 0, 0);
-          x2[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t2, sb * 32 + r, ks), b2, x2[sb], 0, 0, 0);
-        }
-      }
-      // ---- P and dS in registers; register i of block sb is streamed position t0 + 32 sb + 8 (i / 4) + 4 h + i % 4 -------
+      // ---- X1 = T1 . O1^T, then the weights; X2 = T2 . O2^T, then dS (one after the other: the two fp32 tiles are
+      // never live together, which is what lets 128 accumulator registers fit) ----------------------------------------------
+      // register i of block sb is streamed position t0 + 32 (qh TB + sb) + 8 (i / 4) + 4 h + i % 4
       float slope_l2 = 0.f;
       if constexpr (kAlibi)
         slope_l2 = p.alibi_heads > 0 ? exp2f(-8.0f * (float)(shead + 1) / (float)p.alibi_heads) * kLog2e : 0.f;
-      bf16x8 pf[2 * TB], dsf[2 * TB];
+      const int64_t srow0 = ((int64_t)batch * p.Hq + shead) * p.Lq;  // ROLE_DKV: row statistics of the streamed head
+      // 4 consecutive streamed rows of a per-row fp32 array: one 16-byte load when aligned and inside the sequence
+      auto rows4 = [&](const float* base, unsigned staged_off, int q4) FL_INLINE -> f32x4 {
+        if (stats_staged)  // rows past the end hold copies of valid rows; they are masked
+          return *reinterpret_cast<const f32x4*>(smem + staged_off + slot * T::SBYTES + (q4 - t0) * 4);
+        f32x4 out;
 #pragma unroll
-      for (int sb = 0; sb < TB; ++sb) {
-        const int sbase = t0 + 32 * sb + 4 * h;  // streamed position of register 0
-        // element predicate as an interval of the register offset `off` (8 (i / 4) + i % 4): lo <= off <= hi
-        int lo, hi;
-        if constexpr (kDQ) {
-          // streamed = key, owner = query: key < Lk && (dmin <= key - q <= dmax || key < pfx)
-          const int rel = sbase - opos;
-          hi = min(p.Lk - sbase - 1, max(p.dmax - rel, p.pfx - sbase - 1));
-          lo = p.dmin - rel;
-        } else {
-          // streamed = query, owner = key: q < Lq && (dmin <= key - q <= dmax || key < pfx), key = opos
-          const int rel = opos - sbase;  // key - q at off = 0; key - q = rel - off
-          hi = min(p.Lq - sbase - 1, opos < p.pfx ? (1 << 29) : rel - p.dmin);
-          lo = opos < p.pfx ? -(1 << 29) : rel - p.dmax;
-          if (opos >= p.Lk) hi = -(1 << 29);
+        for (int e = 0; e < 4; ++e) out[e] = base[srow0 + min(q4 + e, p.Lq - 1)];  // clamped rows are masked
+        return out;
+      };
+      bf16x8 pf[2 * TB], dsf[2 * TB];
+      float pd[TB][16];  // weight times d(score) / d(qk * scale)
+      {
+        f32x16 x1[TB];
+#pragma unroll
+        for (int sb = 0; sb < TB; ++sb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) x1[sb][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          bf16x8 b1;
+          if constexpr (kDQ) b1 = o1f[ks]; else b1 = frag_row(T::O1_OFF, ow * 32 + r, ks);
+#pragma unroll
+          for (int sb = 0; sb < TB; ++sb)
+            x1[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t1, (qh * TB + sb) * 32 + r, ks), b1, x1[sb], 0, 0, 0);
         }
-        // per-register row statistics of the streamed queries (ROLE_DKV)
-        float lse_s[kDQ ? 1 : 16], delta_s[kDQ ? 1 : 16];
-        int64_t sdoc[kDoc ? 16 : 1];
-        if constexpr (!kDQ) {
-          const int64_t row0 = ((int64_t)batch * p.Hq + shead) * p.Lq;
+#pragma unroll
+        for (int sb = 0; sb < TB; ++sb) {
+          const int sbase = t0 + 32 * (qh * TB + sb) + 4 * h;  // streamed position of register 0
+          // element predicate as an interval of the register offset `off` (8 (i / 4) + i % 4): lo <= off <= hi
+          int lo, hi;
+          if constexpr (kDQ) {
+            // streamed = key, owner = query: key < Lk && (dmin <= key - q <= dmax || key < pfx)
+            const int rel = sbase - opos;
+            hi = min(p.Lk - sbase - 1, max(p.dmax - rel, p.pfx - sbase - 1));
+            lo = p.dmin - rel;
+          } else {
+            // streamed = query, owner = key: q < Lq && (dmin <= key - q <= dmax || key < pfx), key = opos
+            const int rel = opos - sbase;  // key - q at off = 0; key - q = rel - off
+            hi = min(p.Lq - sbase - 1, opos < p.pfx ? (1 << 29) : rel - p.dmin);
+            lo = opos < p.pfx ? -(1 << 29) : rel - p.dmax;
+            if (opos >= p.Lk) hi = -(1 << 29);
+          }
+          float pv[16];
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            // registers 4 g .. 4 g + 3 are 4 consecutive rows: one 16-byte load each when the rows are aligned and
-            // inside the sequence, else element by element (clamped reads past the end are masked below)
-            const int q4 = sbase + 8 * g;
-            if (p.Lq % 4 == 0 && q4 + 3 < p.Lq) {
-              const f32x4 l4 = *reinterpret_cast<const f32x4*>(p.lse + row0 + q4);
-              const f32x4 d4 = *reinterpret_cast<const f32x4*>(p.delta + row0 + q4);
+            f32x4 lse4;
+            if constexpr (!kDQ) lse4 = rows4(p.lse, T::S1_OFF, sbase + 8 * g);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                lse_s[4 * g + e] = l4[e];
-                delta_s[4 * g + e] = d4[e];
+            for (int e = 0; e < 4; ++e) {
+              const int i = 4 * g + e, off = 8 * g + e;
+              const float x = x1[sb][i];
+              float s2, dfac = 1.0f;  // logit in log2 units; d(score) / d(qk * scale)
+              if constexpr (kSoftcap) {
+                const float ex = fast_exp2(x * cap_k1);
+                const float rc = fast_rcp(ex + 1.0f);
+                const float th = __builtin_fmaf(rc, -2.0f, 1.0f);  // tanh(x * scale / cap)
+                s2 = cap_on ? th * cap_c : x * p.scale_log2;
+                dfac = cap_on ? __builtin_fmaf(-th, th, 1.0f) : 1.0f;
+              } else {
+                s2 = x * p.scale_log2;
               }
-            } else {
+              if constexpr (kAlibi) {
+                const float rel_f = kDQ ? (float)(sbase + off - opos) : (float)(opos - sbase - off);
+                s2 = __builtin_fmaf(slope_l2, rel_f, s2);
+              }
+              float pw = fast_exp2(s2 - (kDQ ? lse_o : lse4[e]));
+              if (!full) {  // workgroup-uniform
+                bool ok = (off <= hi) & (off >= lo);
+                if constexpr (kDoc) {
+                  if (!doc_uniform) ok = ok & (p.doc_ids[(int64_t)batch * p.doc_stride + min(sbase + off, slen - 1)] == odoc);
+                }
+                pw = ok ? pw : 0.f;
+              }
+              pv[i] = pw;
+              pd[sb][i] = kSoftcap ? pw * dfac : pw;
+            }
+          }
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int qq = min(q4 + e, p.Lq - 1);
-                lse_s[4 * g + e] = p.lse[row0 + qq];
-                delta_s[4 * g + e] = p.delta[row0 + qq];
-              }
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[2 * sb + j][e] = (bf16_t)pv[8 * j + e];
+        }
+      }
+      {
+        f32x16 x2[TB];
+#pragma unroll
+        for (int sb = 0; sb < TB; ++sb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) x2[sb][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          bf16x8 b2;
+          if constexpr (kDQ) b2 = o2f[ks]; else b2 = frag_row(T::O2_OFF, ow * 32 + r, ks);
+#pragma unroll
+          for (int sb = 0; sb < TB; ++sb)
+            x2[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t2, (qh * TB + sb) * 32 + r, ks), b2, x2[sb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int sb = 0; sb < TB; ++sb) {
+          const int sbase = t0 + 32 * (qh * TB + sb) + 4 * h;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 dl4;
+            if constexpr (!kDQ) dl4 = rows4(p.delta, T::S2_OFF, sbase + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = 4 * g + e;
+              const float ds = pd[sb][i] * (x2[sb][i] - (kDQ ? delta_o : dl4[e]));
+              dsf[2 * sb + i / 8][i % 8] = (bf16_t)ds;
             }
           }
         }
-        if constexpr (kDoc) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            sdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(sbase + 8 * (i / 4) + (i % 4), slen - 1)];
-        }
-        float pv[16], dv_[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int off = 8 * (i / 4) + (i % 4);
-          const float x = x1[sb][i];
-          float s2, dfac = 1.0f;  // logit in log2 units; d(score) / d(qk * scale)
-          if constexpr (kSoftcap) {
-            const float e = fast_exp2(x * cap_k1);
-            const float rc = fast_rcp(e + 1.0f);
-            const float th = __builtin_fmaf(rc, -2.0f, 1.0f);  // tanh(x * scale / cap)
-            s2 = cap_on ? th * cap_c : x * p.scale_log2;
-            dfac = cap_on ? __builtin_fmaf(-th, th, 1.0f) : 1.0f;
-          } else {
-            s2 = x * p.scale_log2;
-          }
-          if constexpr (kAlibi) {
-            const float rel_f = kDQ ? (float)(sbase + off - opos) : (float)(opos - sbase - off);
-            s2 = __builtin_fmaf(slope_l2, rel_f, s2);
-          }
-          bool ok = (off <= hi) & (off >= lo);
-          if constexpr (kDoc) ok = ok & (sdoc[i] == odoc);
-          const float lse = kDQ ? lse_o : lse_s[i];
-          const float dl = kDQ ? delta_o : delta_s[i];
-          const float pw = ok ? fast_exp2(s2 - lse) : 0.f;
-          pv[i] = pw;
-          dv_[i] = pw * (x2[sb][i] - dl) * dfac;
-        }
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            pf[2 * sb + j][e] = (bf16_t)pv[8 * j + e];
-            dsf[2 * sb + j][e] = (bf16_t)dv_[8 * j + e];
-          }
       }
       // ---- acc1 += T1^T . dS,  acc2 += T2^T . P -------------------------------------------------------------------------------
 #pragma unroll
       for (int c = 0; c < 2 * TB; ++c)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t1, c, db), dsf[c], acc1[db], 0, 0, 0);
+          acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t1, 2 * TB * qh + c, db), dsf[c], acc1[db], 0, 0, 0);
           if constexpr (!kDQ)
-            acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t2, c, db), pf[c], acc2[db], 0, 0, 0);
+            acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t2, 2 * TB * qh + c, db), pf[c], acc2[db], 0, 0, 0);
         }
     }
     dma_wait<0>();
   }
 
+  // ---- the waves of one owner block add up their partial sums: the second wave parks its accumulators in LDS (element
+  // (register, lane) of owner block ow at float ((ow * 64 + register) * 64 + lane): consecutive lanes, no conflicts) ----
+  if constexpr (T::QH == 2) {
+    float* park = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int set = 0; set < 2; ++set) {
+      __syncthreads();  // the tiles (set 0) or the previous set's sums (set 1) have been read
+      if (qh == 1) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) park[((ow * 64 + db * 16 + i) * 64) + lane] = set == 0 ? acc1[db][i] : acc2[db][i];
+      }
+      __syncthreads();
+      if (qh == 0) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const float x = park[((ow * 64 + db * 16 + i) * 64) + lane];
+            if (set == 0) acc1[db][i] += x; else acc2[db][i] += x;
+          }
+      }
+    }
+  }
+
   // ---- epilogue: register i of block db is column 32 db + 8 (i / 4) + 4 h + i % 4 of this lane's owner row ---------------
-  if (opos < olen) {
+  if (opos < olen && qh == 0) {
     bf16_t* out1 = kDQ ? p.dq + (int64_t)batch * p.dqs[0] + (int64_t)ohead * p.dqs[1] + (int64_t)opos * p.dqs[2]
                        : p.dk + (int64_t)batch * p.dks[0] + (int64_t)ohead * p.dks[1] + (int64_t)opos * p.dks[2];
 #pragma unroll

@@ -193,6 +193,14 @@ struct TileLayout {
     constexpr int M = (CPR >= 16 ? 16 : CPR) - 1;
     return chunk ^ ((row / RPW) & M);
   }
+  // Tiles that are read both ways (the backward's streamed operands): the row's window index rotated left by two
+  // bits.  Still a permutation of the chunk index over 16 consecutive rows (row-wise reads), and 4 consecutive rows
+  // land in 4 different 64-byte groups (transposing reads).
+  __device__ static __forceinline__ int swz_kv(int row, int chunk) {
+    constexpr int NB = CPR >= 16 ? 4 : (CPR >= 8 ? 3 : 2);
+    const int m = (row / RPW) & ((1 << NB) - 1);
+    return chunk ^ (((m << 2) | (m >> (NB - 2))) & ((1 << NB) - 1));
+  }
   // V operand reads (transposing): 4 consecutive rows x 64 contiguous bytes.
   __device__ static __forceinline__ int swz_v(int row, int chunk) {
     constexpr int G = (CPR >= 16 ? 16 : CPR) / 4;  // 64-byte groups per window row

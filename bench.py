@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-other-configs] [--calibrate-copy]
 
-A step is one pass of the hot path over the benchmark batch of BASELINE config 1 (B=4, H=16, S=4096, D=128, bf16,
+A step is one pass of the hot path over the headline benchmark batch (configuration 1: B=4, H=16, S=4096, D=128, bf16,
 seeded N(0,1) inputs already resident in HBM): one vanilla, one causal and one sliding-window (window 256) forward,
 three kernel launches.  `value` is the unmasked (algorithmic) FLOPs of the step divided by its wall time.  Prints one
 JSON line; per-variant numbers, the roofline of the dominant kernel, the other configurations (measured outside the

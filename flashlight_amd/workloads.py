@@ -57,7 +57,7 @@ def document_ids(lengths: List[int], batch: int, device) -> torch.Tensor:
 @dataclass
 class Workload:
     name: str            # e.g. "cfg1/causal"
-    config: int          # index into BASELINE.json configs
+    config: int          # number of the benchmark configuration (1-4)
     seed: int
     shapes: Dict[str, tuple]
     pairs_per_head: int  # attended (q, k) pairs per query head (per (n, h) for Evoformer)
@@ -86,7 +86,7 @@ def _qkv(seed, B, Hq, Hkv, S, D, Dv=None):
 
 
 def build_workloads(scale_down: int = 1) -> List[Workload]:
-    """All variants of BASELINE configs 1-4.  scale_down > 1 shrinks sequence lengths (and windows/prefixes with
+    """All variants of benchmark configurations 1-4.  scale_down > 1 shrinks sequence lengths (and windows/prefixes with
     them) for quick parity runs; 1 gives the full sizes."""
     from .attention_variants import (attention_pytorch, attention_pytorch_alibi, attention_pytorch_causal,
                                      attention_pytorch_document_mask, attention_pytorch_prefix_lm,

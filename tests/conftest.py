@@ -11,7 +11,7 @@ if str(ROOT) not in sys.path:
 
 GOLDEN = ROOT / "tests" / "golden" / "attention_golden.npz"
 
-# Tolerance of BASELINE.json's north_star for a bf16 kernel against the fp32 reference.
+# Parity bar for a bf16 kernel against the fp32 reference.
 MAX_ABS_TOL = 2e-2
 MEAN_ABS_TOL = 2e-3
 

@@ -85,7 +85,7 @@ def test_benchmark_configs_reduced(name):
 
 @pytest.mark.parametrize("name", WORKLOAD_NAMES)
 def test_benchmark_configs_full_size(name):
-    """Full BASELINE sizes.  The oracle (same eager fp32 code) is evaluated on the GPU tensors, in blocks of
+    """Full benchmark sizes.  The oracle (same eager fp32 code) is evaluated on the GPU tensors, in blocks of
     query rows, because the dense score matrices do not fit a CPU run of a few seconds."""
     w = W.workload_by_name(name)
     t = w.make(DEV)

@@ -60,6 +60,21 @@ class FlAttnBwdParams(C.Structure):
     ]
 
 
+class FlIpaPackParams(C.Structure):
+    """Mirror of `fl_ipa_pack_params` (include/flashlight_amd.h)."""
+
+    _fields_ = [
+        ("q_scalar", C.c_void_p), ("k_scalar", C.c_void_p), ("v_scalar", C.c_void_p),
+        ("q_points", C.c_void_p), ("k_points", C.c_void_p), ("v_points", C.c_void_p),
+        ("q_cat", C.c_void_p), ("k_cat", C.c_void_p), ("v_cat", C.c_void_p),
+        ("key_term", C.c_void_p),
+        ("rows", C.c_int64),
+        ("c_qk", C.c_int32), ("c_v", C.c_int32), ("n_qk_coords", C.c_int32), ("n_v_coords", C.c_int32),
+        ("dqk", C.c_int32), ("dv", C.c_int32),
+        ("q_scale", C.c_float), ("point_weight", C.c_float),
+    ]
+
+
 class FlashlightError(RuntimeError):
     """fl_attn_fwd / fl_attn_validate returned non-zero; `.code` holds the return value."""
 
@@ -99,6 +114,8 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_bwd_validate.argtypes = [C.POINTER(FlAttnBwdParams)]
     lib.fl_attn_bwd.restype = C.c_int
     lib.fl_attn_bwd.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
+    lib.fl_ipa_pack.restype = C.c_int
+    lib.fl_ipa_pack.argtypes = [C.POINTER(FlIpaPackParams), C.c_void_p]
     lib.fl_probe_mfma_rate.restype = C.c_int
     lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
@@ -337,6 +354,38 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
         _check(lib.fl_attn_bwd(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     del keep, delta
     return dq, dk, dv
+
+
+def ipa_pack(q_scalar, k_scalar, v_scalar, q_points, k_points, v_points, dqk: int, dv: int, q_scale: float,
+             point_weight: float):
+    """[rows, *] bf16 tensors -> (q_cat [rows, dqk], k_cat [rows, dqk], v_cat [rows, dv], key_term [rows] fp32), one
+    launch on the current stream (see `fl_ipa_pack` in include/flashlight_amd.h)."""
+    lib = load_library()
+    ts = [q_scalar, k_scalar, v_scalar, q_points, k_points, v_points]
+    for i, t in enumerate(ts):
+        _require_gpu_bf16("invariant point attention operand", t)
+        if t.dim() != 2 or t.size(0) != q_scalar.size(0):
+            raise ValueError("operands must be 2-D with one row per (batch, head, residue)")
+        ts[i] = t.contiguous()
+    rows, dev = q_scalar.size(0), q_scalar.device
+    if k_scalar.size(1) != q_scalar.size(1) or k_points.size(1) != q_points.size(1):
+        raise ValueError("query and key operands differ in width")
+    q_cat = torch.empty((rows, dqk), dtype=torch.bfloat16, device=dev)
+    k_cat = torch.empty((rows, dqk), dtype=torch.bfloat16, device=dev)
+    v_cat = torch.empty((rows, dv), dtype=torch.bfloat16, device=dev)
+    key_term = torch.empty((rows,), dtype=torch.float32, device=dev)
+    p = FlIpaPackParams()
+    (p.q_scalar, p.k_scalar, p.v_scalar, p.q_points, p.k_points, p.v_points) = (t.data_ptr() for t in ts)
+    p.q_cat, p.k_cat, p.v_cat, p.key_term = q_cat.data_ptr(), k_cat.data_ptr(), v_cat.data_ptr(), key_term.data_ptr()
+    p.rows = rows
+    p.c_qk, p.c_v, p.n_qk_coords, p.n_v_coords = ts[0].size(1), ts[2].size(1), ts[3].size(1), ts[5].size(1)
+    p.dqk, p.dv, p.q_scale, p.point_weight = int(dqk), int(dv), float(q_scale), float(point_weight)
+    with torch.cuda.device(dev):
+        rc = lib.fl_ipa_pack(C.byref(p), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc != 0:
+        raise FlashlightError(rc, "fl_ipa_pack rejected its arguments or could not launch")
+    del ts
+    return q_cat, k_cat, v_cat, key_term
 
 
 def plan(p: FlAttnParams) -> dict:

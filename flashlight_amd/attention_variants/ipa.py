@@ -19,7 +19,7 @@ from typing import Optional, Tuple
 import torch
 import torch.nn.functional as F
 
-from .. import ops
+from .. import _ffi, ops
 
 # (Dqk, Dv) pairs with a kernel instance that takes bias operands, cheapest first
 _BIAS_SHAPES = ((32, 32), (32, 64), (64, 64), (64, 128), (128, 128))
@@ -72,12 +72,23 @@ def invariant_point_attention(q_scalar: torch.Tensor, k_scalar: torch.Tensor, v_
     def flat(t, tail):  # [*, H, n, ...tail] -> [B, H, n, prod(tail)]
         return t.reshape(B, H, t.shape[len(lead) + 1], tail)
 
-    qs = (flat(q_scalar, C).float() * (1.0 / (math.sqrt(c_hidden) * scale))).to(torch.bfloat16)
-    q_cat = F.pad(torch.cat([qs, flat(q_points, nq)], dim=-1), (0, dqk - C - nq))
-    k_cat = F.pad(torch.cat([flat(k_scalar, C), flat(k_points, nq)], dim=-1), (0, dqk - C - nq))
-    v_cat = F.pad(torch.cat([flat(v_scalar, v_scalar.shape[-1]), flat(v_points, nv)], dim=-1),
-                  (0, dv - v_scalar.shape[-1] - nv))
-    key_term = (w * flat(k_points, nq).float().square().sum(-1)).unsqueeze(-2)  # [B, H, 1, S] fp32
+    cv = v_scalar.shape[-1]
+    q_scale = 1.0 / (math.sqrt(c_hidden) * scale)
+    if torch.compiler.is_compiling() or S != N:
+        # traced (or cross-attention, which the packing kernel's single row count does not cover): plain tensor code
+        qs = (flat(q_scalar, C).float() * q_scale).to(torch.bfloat16)
+        q_cat = F.pad(torch.cat([qs, flat(q_points, nq)], dim=-1), (0, dqk - C - nq))
+        k_cat = F.pad(torch.cat([flat(k_scalar, C), flat(k_points, nq)], dim=-1), (0, dqk - C - nq))
+        v_cat = F.pad(torch.cat([flat(v_scalar, cv), flat(v_points, nv)], dim=-1), (0, dv - cv - nv))
+        key_term = (w * flat(k_points, nq).float().square().sum(-1)).unsqueeze(-2)  # [B, H, 1, S] fp32
+    else:
+        # one launch builds all four operands
+        rows = B * H * N
+        q_cat, k_cat, v_cat, key_term = _ffi.ipa_pack(
+            q_scalar.reshape(rows, C), k_scalar.reshape(rows, C), v_scalar.reshape(rows, cv), q_points.reshape(rows, nq),
+            k_points.reshape(rows, nq), v_points.reshape(rows, nv), dqk, dv, q_scale, w)
+        q_cat, k_cat, v_cat = q_cat.view(B, H, N, dqk), k_cat.view(B, H, N, dqk), v_cat.view(B, H, N, dv)
+        key_term = key_term.view(B, H, 1, N)
     biases = []
     if pair_bias is not None:
         pb = pair_bias
@@ -99,7 +110,6 @@ def invariant_point_attention(q_scalar: torch.Tensor, k_scalar: torch.Tensor, v_
     biases.append((key_term, 1))
 
     out = ops.dispatch(q_cat, k_cat, v_cat, scale=scale, biases=biases)  # [B, H, N, dv]
-    cv = v_scalar.shape[-1]
     out_scalar = out[..., :cv].reshape(*lead, H, N, cv)
     out_points = out[..., cv:cv + nv].reshape(*lead, H, N, Pv, X).transpose(-3, -4)
     return out_scalar, out_points

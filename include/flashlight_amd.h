@@ -171,6 +171,26 @@ int fl_attn_bwd_validate(const fl_attn_bwd_params* p);
 /* Launches the three backward kernels (row sums of dO o O, then dQ, then dK and dV) on `stream`. */
 int fl_attn_bwd(const fl_attn_bwd_params* p, void* stream);
 
+/* Operand packing for invariant point attention (tests/test_ipa.py:57-125, a test-only function of the reference):
+ * builds the concatenated operands with which the function becomes one fl_attn_fwd call.  All tensors are bf16,
+ * contiguous, `rows` = batch * heads * residues rows each:
+ *   q_cat[row] = [q_scalar[row] * q_scale | q_points[row] | 0...]   (dqk columns)
+ *   k_cat[row] = [k_scalar[row]           | k_points[row] | 0...]
+ *   v_cat[row] = [v_scalar[row]           | v_points[row] | 0...]   (dv columns)
+ *   key_term[row] = point_weight * sum(k_points[row]^2)              (fp32)
+ * The squared-distance term of test_ipa.py:102-108 then equals -2 * point_weight * (q_points . k_points) + key_term[k]
+ * plus a term that is constant along a softmax row. */
+typedef struct fl_ipa_pack_params {
+  const void *q_scalar, *k_scalar, *v_scalar; /* [rows, c_qk], [rows, c_qk], [rows, c_v] */
+  const void *q_points, *k_points, *v_points; /* [rows, n_qk_coords], [rows, n_qk_coords], [rows, n_v_coords] */
+  void *q_cat, *k_cat, *v_cat;                /* [rows, dqk], [rows, dqk], [rows, dv] */
+  float* key_term;                            /* [rows] */
+  int64_t rows;
+  int32_t c_qk, c_v, n_qk_coords, n_v_coords, dqk, dv;
+  float q_scale, point_weight;
+} fl_ipa_pack_params;
+int fl_ipa_pack(const fl_ipa_pack_params* p, void* stream);
+
 /* Measurement aid with no counterpart in the reference: launches a kernel that does nothing but issue
  * v_mfma_f32_32x32x16_bf16 (the instruction both products of the forward are built from) on operand fragments read
  * once from `operands`, so that the matrix-pipe rate this part sustains on given data can be put next to the

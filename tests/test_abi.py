@@ -150,6 +150,19 @@ def test_front_end_refuses_cpu_and_fp32_tensors(lib):
         attention_pytorch_alibi(q, q, q)
 
 
+def test_ipa_pack_rejects_bad_arguments_without_a_gpu(lib):
+    assert "fl_ipa_pack" in declared_functions() and "fl_attn_bwd" in declared_functions()
+    assert lib.fl_ipa_pack(None, None) == -1
+    p = _ffi.FlIpaPackParams()
+    assert lib.fl_ipa_pack(C.byref(p), None) == -1                       # null tensors
+    for name in ("q_scalar", "k_scalar", "v_scalar", "q_points", "k_points", "v_points", "q_cat", "k_cat", "v_cat", "key_term"):
+        setattr(p, name, 0x10000)
+    p.rows, p.c_qk, p.c_v, p.n_qk_coords, p.n_v_coords, p.dqk, p.dv = 10, 16, 16, 12, 24, 24, 64
+    assert lib.fl_ipa_pack(C.byref(p), None) == -2                       # 16 + 12 channels do not fit 24 columns
+    p.dqk, p.rows = 32, 0
+    assert lib.fl_ipa_pack(C.byref(p), None) == -2                       # no rows
+
+
 def test_probe_rejects_bad_arguments_without_a_gpu(lib):
     # the measurement aid checks its arguments on the host before it launches anything
     assert lib.fl_probe_mfma_rate(None, 1, 1, 1, None, None) == -5

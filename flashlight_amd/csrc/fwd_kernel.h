@@ -453,7 +453,10 @@ void fwd_kernel(const KParams p) {
     if constexpr (kDoc) {
       return tlist[min(i, n_list - 1)];
     } else {
-      const int t = t_lo + min(i, n_list - 1);
+      // ALiBi adds a term that grows with the key position: visiting the tiles from the last one down makes every
+      // later tile's scores fall away from the running reference instead of climbing above it, so the reference set by
+      // the first tile visited holds and the accumulators are never rescaled
+      const int t = (FEAT & F_ALIBI) ? t_lo + n_list - 1 - min(i, n_list - 1) : t_lo + min(i, n_list - 1);
       const int cw = (t < e_lo || t > e_hi) ? TILE_EMPTY : ((t >= f_lo && t <= f_hi) ? TILE_FULL : TILE_PARTIAL);
       return ((uint32_t)cw << (16 + 2 * wave)) | (uint32_t)t;
     }
@@ -910,10 +913,10 @@ void fwd_kernel(const KParams p) {
     // is not <= kBig (a weight overflowed, or NaN), or whose sum and running sum are both < kTiny (the tile may have
     // underflowed with nothing to be negligible against), sends the wave through the exact path: row maxima, new
     // reference, weights again.  Any reference gives the same O / l; fp32 sums keep their relative precision.
-    // ALiBi moves the scores by a large, steady amount from tile to tile, which would send most tiles through the
-    // exact path after the fact: kernels with ALiBi take the exact path up front instead.
+    // ALiBi moves the scores by a large, steady amount from tile to tile; its kernels visit the tiles in descending key
+    // order (see list_entry), so that the amount is downwards and the first reference holds.
     constexpr float kBig = 0x1p24f, kTiny = 0x1p-24f;
-    constexpr bool kFastRef = !kAlibi;
+    constexpr bool kFastRef = true;
     auto weights_checked = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB], bool check, auto in_loop,
                                bf16x8 (&vfirst)[DVB], int vslot) FL_INLINE {
       float rs[QB];

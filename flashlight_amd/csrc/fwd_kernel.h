@@ -784,9 +784,20 @@ void fwd_kernel(const KParams p) {
         const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
         int64_t kdoc[16];
         if constexpr (kDoc) {
+          // a 32-key block lies inside one document far more often than not, and the (min, max) table says so with two
+          // scalar loads: only blocks that hold a boundary read their keys' ids one by one
+          static_assert(kDocBlock == 32, "one table entry per 32-key block of a tile");
+          // (a block that starts past the last key reads the last entry: all of its keys are masked anyway)
+          const int64_t* tb = p.doc_table + ((int64_t)batch * p.doc_blocks + min((k0 + 32 * kb) / kDocBlock, p.doc_blocks - 1)) * 2;
+          const int64_t bmn = tb[0], bmx = tb[1];
+          if (bmn == bmx) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i)
-            kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
+            for (int i = 0; i < 16; ++i) kdoc[i] = bmn;
+          } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
+          }
         }
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {

@@ -19,6 +19,7 @@ LIB_PATH = Path(os.environ.get("FL_LIB") or Path(__file__).resolve().parent / LI
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING, MASK_PREFIX_LM, MASK_DOCUMENT, MASK_DOCUMENT_CAUSAL = range(6)
 FL_BF16 = 0
 FL_F32 = 1
+FL_F16 = 2
 ABI_VERSION = 1
 
 
@@ -143,14 +144,26 @@ def _strides4(t: torch.Tensor) -> Sequence[int]:
     return tuple(int(s) for s in t.stride())
 
 
-def _require_gpu_bf16(name: str, t: torch.Tensor) -> None:
+_HALF_TYPES = {torch.bfloat16: FL_BF16, torch.float16: FL_F16}
+
+
+def _require_gpu_half(name: str, t: torch.Tensor, like: Optional[torch.Tensor] = None) -> None:
+    """`t` must be a bf16 or fp16 GPU tensor (of `like`'s element type when that is given)."""
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
     if not t.is_cuda:
         raise NotImplementedError(
             f"{name} is on {t.device}: flashlight_amd only runs its HIP kernels on a GPU tensor (no CPU path)")
+    if t.dtype not in _HALF_TYPES:
+        raise NotImplementedError(f"{name} has dtype {t.dtype}: the HIP kernels take bfloat16 or float16")
+    if like is not None and t.dtype != like.dtype:
+        raise NotImplementedError(f"{name} has dtype {t.dtype} but the query has {like.dtype}: mixed element types")
+
+
+def _require_gpu_bf16(name: str, t: torch.Tensor) -> None:
+    _require_gpu_half(name, t)
     if t.dtype != torch.bfloat16:
-        raise NotImplementedError(f"{name} has dtype {t.dtype}: the HIP kernels take bfloat16")
+        raise NotImplementedError(f"{name} has dtype {t.dtype}: this entry point takes bfloat16")
 
 
 def _dim_contiguous(t: torch.Tensor) -> torch.Tensor:
@@ -192,7 +205,8 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
         if b.dtype == torch.float32 and b.is_cuda:
             p.bias_dtype[i] = FL_F32
         else:
-            _require_gpu_bf16(f"bias[{i}]", b)
+            _require_gpu_half(f"bias[{i}]", b, q)
+            p.bias_dtype[i] = _HALF_TYPES[q.dtype]
         if b.dim() != 4:
             raise ValueError(f"bias[{i}] must be 4-D, got {tuple(b.shape)}")
         want = (B // div, Hq, Lq, Lk)
@@ -214,7 +228,7 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
         p.bias_batch_div[i] = int(div)
         keep.append(b)
     if gate is not None:
-        _require_gpu_bf16("gate", gate)
+        _require_gpu_half("gate", gate, q)
         if tuple(gate.shape) != (B, Hq, Lq, Dv):
             raise ValueError(f"gate must have the output's shape {(B, Hq, Lq, Dv)}, got {tuple(gate.shape)}")
         if gate.stride(-1) != 1 or any(s % 4 for s in gate.stride()[:-1]) or gate.data_ptr() % 8:
@@ -224,7 +238,7 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
         keep.append(gate)
     p.diff = 1 if diff else 0
     p.lambda_ = float(lambda_full)
-    p.dtype = FL_BF16
+    p.dtype = _HALF_TYPES[q.dtype]
     if attended_dump is not None:
         if attended_dump.dtype != torch.uint8 or tuple(attended_dump.shape) != (B, Hq, Lq, Lk) or \
                 not attended_dump.is_contiguous() or attended_dump.device != q.device:
@@ -262,12 +276,13 @@ def attn_fwd(
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
     `biases` holds up to two (tensor, batch_div) pairs; each tensor is 4-D, bf16 or fp32, broadcastable to
-    [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  Returns `out` [B, Hq, Lq, Dv] (bf16), written on the current stream.
+    [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  q, k, v (and gate, 16-bit biases) are all bf16 or all fp16.  Returns `out` [B, Hq, Lq, Dv]
+    in that type, written on the current stream.
     `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
-        _require_gpu_bf16(name, t)
+        _require_gpu_half(name, t, q if isinstance(q, torch.Tensor) and q.dtype in _HALF_TYPES else None)
         if t.dim() != 4:
             raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
     q, k, v = _dim_contiguous(q), _dim_contiguous(k), _dim_contiguous(v)
@@ -285,8 +300,8 @@ def attn_fwd(
     if Hv != Hkv:
         raise ValueError(f"value has {Hv} heads, expected {Hkv}")
     if out is None:
-        out = torch.empty((B, Hq, Lq, Dv), dtype=torch.bfloat16, device=q.device)
-    elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != torch.bfloat16 or out.device != q.device:
+        out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
+    elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != q.dtype or out.device != q.device:
         raise ValueError("out has the wrong shape, dtype or device")
     if diff and Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None:
         # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,

@@ -3,7 +3,7 @@
 Same module names, function names, positional parameters and result layouts as the reference's eager definitions
 (attention_variants/*.py); where callers of the reference write `torch.compile(fn)(q, k, v, ...)`, callers of this
 package call `fn(q, k, v, ...)` and get one fused HIP kernel launch on the current stream.
-Inputs must be bfloat16 tensors on a GPU; anything else raises (there is no eager fallback).
+Inputs must be bfloat16 (or float16) tensors on a GPU; anything else raises (there is no eager fallback).
 """
 from .vanilla import attention_pytorch, attention_pytorch_nogqa  # noqa: F401
 from .causal import attention_pytorch_causal  # noqa: F401

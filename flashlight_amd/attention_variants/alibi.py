@@ -85,7 +85,7 @@ def dense_bias_operand(bias, query: torch.Tensor, key: torch.Tensor, enable_gqa:
     for got, want in zip(bias.shape, (n, hq, l, s)):
         if got not in (1, want):
             raise ValueError(f"bias of shape {tuple(bias.shape)} does not broadcast to the scores {(n, hq, l, s)}")
-    if bias.dtype not in (torch.bfloat16, torch.float32):
+    if bias.dtype != torch.float32 and bias.dtype != query.dtype:
         bias = bias.to(torch.float32)
     if bias.device != query.device:
         bias = bias.to(query.device)

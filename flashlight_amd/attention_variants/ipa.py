@@ -74,9 +74,9 @@ def invariant_point_attention(q_scalar: torch.Tensor, k_scalar: torch.Tensor, v_
 
     cv = v_scalar.shape[-1]
     q_scale = 1.0 / (math.sqrt(c_hidden) * scale)
-    if torch.compiler.is_compiling() or S != N:
-        # traced (or cross-attention, which the packing kernel's single row count does not cover): plain tensor code
-        qs = (flat(q_scalar, C).float() * q_scale).to(torch.bfloat16)
+    if torch.compiler.is_compiling() or S != N or q_scalar.dtype != torch.bfloat16:
+        # traced, fp16, or cross-attention (which the packing kernel's single row count does not cover): tensor code
+        qs = (flat(q_scalar, C).float() * q_scale).to(q_scalar.dtype)
         q_cat = F.pad(torch.cat([qs, flat(q_points, nq)], dim=-1), (0, dqk - C - nq))
         k_cat = F.pad(torch.cat([flat(k_scalar, C), flat(k_points, nq)], dim=-1), (0, dqk - C - nq))
         v_cat = F.pad(torch.cat([flat(v_scalar, cv), flat(v_points, nv)], dim=-1), (0, dv - cv - nv))
@@ -104,7 +104,7 @@ def invariant_point_attention(q_scalar: torch.Tensor, k_scalar: torch.Tensor, v_
             div = B
         if pb.size(-1) != S:
             pb = pb.expand(*pb.shape[:-1], S).contiguous()
-        if pb.dtype not in (torch.bfloat16, torch.float32):
+        if pb.dtype != torch.float32 and pb.dtype != q_scalar.dtype:
             pb = pb.float()
         biases.append((pb, div))
     biases.append((key_term, 1))

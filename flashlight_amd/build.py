@@ -105,11 +105,12 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
     tasks: list[tuple[list[str], Path]] = []
     objs: list[Path] = []
     for name, args in instance_rows():
-        o = objdir / f"inst_{name}.o"
-        objs.append(o)
-        if not o.exists():
-            tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_NAME={name}", f"-DFL_INST_ARGS={args}", "-c",
-                           str(CSRC / "instance_unit.hip"), "-o", str(o)], o))
+        for f16 in (0, 1):  # every instance once for bf16 and once for fp16 elements
+            o = objdir / f"inst_{name}{'_f16' if f16 else ''}.o"
+            objs.append(o)
+            if not o.exists():
+                tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_NAME={name}", f"-DFL_INST_ARGS={args}", f"-DFL_INST_F16={f16}",
+                               "-c", str(CSRC / "instance_unit.hip"), "-o", str(o)], o))
     # backward kernels: one unit per (head dim, feature bits) of FL_BWD_LIST in bwd_instances.h
     bwd_list = re.search(r"#define FL_BWD_LIST\(X\)(.*)", (CSRC / "bwd_instances.h").read_text()).group(1)
     for d, feat in re.findall(r"X\((\d+),\s*(\d+)\)", bwd_list):

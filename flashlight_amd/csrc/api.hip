@@ -71,7 +71,7 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   const bool short_loop = p->mask_kind == FL_MASK_SLIDING && visited <= 640;
   for (int i = 0; i < fl::kNumInstances; ++i) {
     const fl::Instance& in = fl::kInstances[i];
-    if (in.dqk != p->Dqk || in.dv != p->Dv) continue;
+    if (in.dqk != p->Dqk || in.dv != p->Dv || in.dtype != p->dtype) continue;
     if ((in.feat & want) != want) continue;
     const uint32_t extra = in.feat & ~want;
     if (extra & ~kOptionalFeatures) continue;
@@ -121,7 +121,8 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if ((rc = check_ptr("q", p->q, 16)) || (rc = check_ptr("k", p->k, 16)) || (rc = check_ptr("v", p->v, 16)) ||
       (rc = check_ptr("o", p->o, 8)))
     return rc;
-  if (p->dtype != FL_BF16) return fail(FL_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
+  if (p->dtype != FL_BF16 && p->dtype != FL_F16)
+    return fail(FL_ERR_UNSUPPORTED, "dtype %d is not supported (FL_BF16 or FL_F16)", p->dtype);
   if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lq <= 0 || p->Lk <= 0 || p->Dqk <= 0 || p->Dv <= 0)
     return fail(FL_ERR_SHAPE, "sizes must be positive: B=%d Hq=%d Hkv=%d Lq=%d Lk=%d Dqk=%d Dv=%d", p->B, p->Hq, p->Hkv,
                 p->Lq, p->Lk, p->Dqk, p->Dv);
@@ -162,8 +163,8 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if (!(p->softcap >= 0.f) || !std::isfinite(p->softcap)) return fail(FL_ERR_ARG, "softcap must be finite and >= 0");
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb]) continue;
-    if (p->bias_dtype[nb] != FL_BF16 && p->bias_dtype[nb] != FL_F32)
-      return fail(FL_ERR_UNSUPPORTED, "bias_dtype[%d]=%d is not supported (bf16 or fp32)", nb, p->bias_dtype[nb]);
+    if (p->bias_dtype[nb] != p->dtype && p->bias_dtype[nb] != FL_F32)
+      return fail(FL_ERR_UNSUPPORTED, "bias_dtype[%d]=%d is not supported (fp32, or the element type of q)", nb, p->bias_dtype[nb]);
     const int esz = p->bias_dtype[nb] == FL_F32 ? 4 : 2;
     if (reinterpret_cast<uintptr_t>(p->bias[nb]) % esz)
       return fail(FL_ERR_ALIGN, "bias[%d] must be %d-byte aligned", nb, esz);
@@ -353,6 +354,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
     return fail(FL_ERR_UNSUPPORTED, "backward: bias operands, gate, differential attention and the dump hook are not supported");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
+  if (p->dtype != FL_BF16) return fail(FL_ERR_UNSUPPORTED, "backward: bf16 only");
   if ((rc = check_ptr("dout", b->dout, 16)) || (rc = check_ptr("dq", b->dq, 8)) || (rc = check_ptr("dk", b->dk, 8)) ||
       (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 16)) ||
       (rc = check_ptr("fwd.lse", p->lse, 16)))

@@ -257,8 +257,20 @@ __device__ __forceinline__ void sched_second_product() {
 #endif
 }
 
-template <int DQK_, int DV_, int RW_, int BN_, int NW_, uint32_t FEAT_, int NS_ = 4>
+// Element types of q, k, v, biases (unless fp32), gate and the output: bf16 or fp16.  The two differ in the MFMA and dot
+// instructions and in the conversions from and to fp32; everything else treats the elements as 16 opaque bits.
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ float dot2acc(bf16x2 a, bf16x2 b, float c) { return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false); }
+__device__ __forceinline__ float dot2acc(f16x2 a, f16x2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
+
+template <int DQK_, int DV_, int RW_, int BN_, int NW_, uint32_t FEAT_, int NS_ = 4, class Elem_ = bf16_t>
 struct FwdTraits {
+  using Elem = Elem_;
   static constexpr int DQK = DQK_, DV = DV_, RW = RW_, BN = BN_, NW = NW_;
   static constexpr int NS = NS_;  // K/V tiles resident in LDS (ring); transfers run NS - 1 tiles ahead of their use
   static_assert(NS >= 2 && NS <= 8 && NS % 2 == 0, "ring depth (even: the two score buffers alternate with the slots)");
@@ -314,6 +326,10 @@ void fwd_kernel(const KParams p) {
   constexpr bool kDiff = FEAT & F_DIFF, kGate = FEAT & F_GATE, kDump = FEAT & F_DUMP;
   constexpr bool kMod = kAlibi || kSoftcap || kBias;  // scores are transformed before the softmax
   constexpr float kLog2e = 1.4426950408889634f;
+  using E = typename T::Elem;  // pointers in KParams are typed bf16_t whatever E is: 16 opaque bits
+  typedef E ex8 __attribute__((ext_vector_type(8)));
+  typedef E ex4 __attribute__((ext_vector_type(4)));
+  typedef E ex2 __attribute__((ext_vector_type(2)));
   using LK = TileLayout<DQK>;
   using LV = TileLayout<DV>;
 
@@ -492,7 +508,7 @@ void fwd_kernel(const KParams p) {
   // Gate logits of this lane's output elements, fetched before the key loop when they fit the register budget so that
   // their latency is not paid in the epilogue.
   constexpr bool kGateEarly = kGate && DV <= 32;
-  bf16x4 gpre[kGateEarly ? DVB : 1][kGateEarly ? QB : 1][4];
+  ex4 gpre[kGateEarly ? DVB : 1][kGateEarly ? QB : 1][4];
   if constexpr (kGateEarly) {
     if (p.gate) {
       const bf16_t* gp = p.gate + (int64_t)batch * p.gs[0] + (int64_t)head * p.gs[1];
@@ -502,7 +518,7 @@ void fwd_kernel(const KParams p) {
         for (int dvb = 0; dvb < DVB; ++dvb)
 #pragma unroll
           for (int g = 0; g < 4; ++g)
-            gpre[dvb][qb][g] = *reinterpret_cast<const bf16x4*>(gp + (int64_t)min(qrow[qb], p.Lq - 1) * p.gs[2] +
+            gpre[dvb][qb][g] = *reinterpret_cast<const ex4*>(gp + (int64_t)min(qrow[qb], p.Lq - 1) * p.gs[2] +
                                                                 32 * dvb + 8 * g + 4 * h);
     }
   }
@@ -518,12 +534,12 @@ void fwd_kernel(const KParams p) {
     const bf16_t* vptr = p.v + (int64_t)batch * p.vs[0] + (int64_t)kvh * p.vs[1];
 
     // Q fragments: B operand of S^T = K.Q^T; lane (r, h) holds Q[q = r][16*ks + 8h .. +8].
-    bf16x8 qf[QB][KS];
+    ex8 qf[QB][KS];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
-        qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qptr + (int64_t)min(qrow[qb], p.Lq - 1) * p.qs[2] + ks * 16 + 8 * h);
+        qf[qb][ks] = *reinterpret_cast<const ex8*>(qptr + (int64_t)min(qrow[qb], p.Lq - 1) * p.qs[2] + ks * 16 + 8 * h);
 
 #pragma unroll
     for (int dvb = 0; dvb < DVB; ++dvb)
@@ -662,10 +678,10 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
           const int row = kb * 32 + r;
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kb_ + row * (DQK * 2) + LK::swz_k(row, 2 * ks + h) * 16);
+          const ex8 kf = *reinterpret_cast<const ex8*>(kb_ + row * (DQK * 2) + LK::swz_k(row, 2 * ks + h) * 16);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb)
-            s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], s[kb][qb], 0, 0, 0);
+            s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
         }
     };
 
@@ -689,7 +705,7 @@ void fwd_kernel(const KParams p) {
                 const unsigned char* bl = smem + T::R_OFF + bslot * T::RBYTES + wave * 1024 + 8 * h;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                  const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bl + (4 * kb + g) * 16);
+                  const ex4 b4 = *reinterpret_cast<const ex4*>(bl + (4 * kb + g) * 16);
 #pragma unroll
                   for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
                 }
@@ -700,7 +716,7 @@ void fwd_kernel(const KParams p) {
                 const unsigned char* bl = smem + T::B_OFF + bslot * T::BBYTES + wave * (RW * BN * 2) + row * (BN * 2) + 8 * h;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                  const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bl + LB::swz(row, 4 * kb + g) * 16);
+                  const ex4 b4 = *reinterpret_cast<const ex4*>(bl + LB::swz(row, 4 * kb + g) * 16);
 #pragma unroll
                   for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
                 }
@@ -734,13 +750,13 @@ void fwd_kernel(const KParams p) {
                   for (int g = 0; g < 4; ++g) {
                     const int key = kbase + 8 * g;
                     if (p.bias_vec[nb] && key + 3 < p.Lk) {
-                      bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bp + key);
+                      ex4 b4 = *reinterpret_cast<const ex4*>(bp + key);
 #pragma unroll
                       for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
                     } else {
 #pragma unroll
                       for (int e = 0; e < 4; ++e)
-                        if (key + e < p.Lk) bv[4 * g + e] += (float)bp[(int64_t)(key + e) * p.bs[nb][3]];
+                        if (key + e < p.Lk) bv[4 * g + e] += (float)reinterpret_cast<const E*>(bp)[(int64_t)(key + e) * p.bs[nb][3]];
                     }
                   }
                 }
@@ -835,9 +851,9 @@ void fwd_kernel(const KParams p) {
 
     // ---- A operand of O^T += V^T . P^T for 16-key chunk c and value block dvb, through the transposing LDS read.
     // Slot j of lane (r, h) is key 16c + 8*(j/4) + 4h + j%4, the key order of the packed weights.
-    auto v_frag = [&](int buf, int c, int dvb) FL_INLINE -> bf16x8 {
+    auto v_frag = [&](int buf, int c, int dvb) FL_INLINE -> ex8 {
       const unsigned char* vb_ = smem + T::V_OFF + buf * T::VBYTES;
-      bf16x8 vf;
+      ex8 vf;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         // within each 16-lane group, lane i supplies row (key) i/4, 4 columns at 4*(i%4), and receives column i
@@ -848,7 +864,7 @@ void fwd_kernel(const KParams p) {
         const unsigned char* ap = vb_ + row * (DV * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
         typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
         const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
-        const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
+        const ex4 b4 = __builtin_bit_cast(ex4, t4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
       }
@@ -891,9 +907,8 @@ void fwd_kernel(const KParams p) {
     };
 
     // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
-    auto softmax_p = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB], float (&rsum)[QB]) FL_INLINE {
-      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-      const bf16x2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], float (&rsum)[QB]) FL_INLINE {
+      const ex2 ones = {(E)1.0f, (E)1.0f};
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
@@ -906,13 +921,13 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pf[qb][2 * kb + j][e] = (bf16_t)pv[8 * j + e];
+            for (int e = 0; e < 8; ++e) pf[qb][2 * kb + j][e] = (E)pv[8 * j + e];
             // the row sum adds up the rounded weights, the very numbers the second product uses (v_dot2 with ones:
             // two weights per instruction)
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
-              const bf16x2 pr = {pf[qb][2 * kb + j][e], pf[qb][2 * kb + j][e + 1]};
-              rs = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, rs, false);
+              const ex2 pr = {pf[qb][2 * kb + j][e], pf[qb][2 * kb + j][e + 1]};
+              rs = dot2acc(pr, ones, rs);
             }
           }
         }
@@ -928,8 +943,8 @@ void fwd_kernel(const KParams p) {
     // order (see list_entry), so that the amount is downwards and the first reference holds.
     constexpr float kBig = 0x1p24f, kTiny = 0x1p-24f;
     constexpr bool kFastRef = true;
-    auto weights_checked = [&](const f32x16 (&s)[KB][QB], bf16x8 (&pf)[QB][2 * KB], bool check, auto in_loop,
-                               bf16x8 (&vfirst)[DVB], int vslot) FL_INLINE {
+    auto weights_checked = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], bool check, auto in_loop,
+                               ex8 (&vfirst)[DVB], int vslot) FL_INLINE {
       float rs[QB];
       softmax_p(s, pf, rs);
       if constexpr (decltype(in_loop)::value) {
@@ -965,17 +980,17 @@ void fwd_kernel(const KParams p) {
     // ---- O^T += V^T . P^T: A = V fragment through the transposing LDS read, B = P ---------------------------------------
     // A operand slot j of lane (r, h) for 16-key chunk c is key 16c + 8*(j/4) + 4h + j%4, the key order of pf.
     // `first` holds the fragments of key chunk 0 when the caller has fetched them ahead (HAVE_FIRST)
-    auto pv_mma = [&](const bf16x8 (&pf)[QB][2 * KB], int buf, const bf16x8 (&first)[DVB], auto have_first) FL_INLINE {
+    auto pv_mma = [&](const ex8 (&pf)[QB][2 * KB], int buf, const ex8 (&first)[DVB], auto have_first) FL_INLINE {
 #pragma unroll
       for (int c = 0; c < 2 * KB; ++c)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
-          bf16x8 vf;
+          ex8 vf;
           if (decltype(have_first)::value && c == 0) vf = first[dvb];
           else vf = v_frag(buf, c, dvb);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb)
-            oacc[dvb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[qb][c], oacc[dvb][qb], 0, 0, 0);
+            oacc[dvb][qb] = mfma32(vf, pf[qb][c], oacc[dvb][qb]);
         }
     };
 
@@ -1035,13 +1050,13 @@ void fwd_kernel(const KParams p) {
         }
         if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
         settle(sc, ent[0]);
-        bf16x8 pf[QB][2 * KB];
+        ex8 pf[QB][2 * KB];
         // Raised issue priority while this wave has matrix work: of the two waves sharing a SIMD, the one that is in
         // its MFMA phase wins the issue port, which drives the pair into opposite phases (one on the matrix pipe while
         // the other does vector work) instead of both stalling on each other.
         __builtin_amdgcn_s_setprio(3);
         qk(sn, (slot + 1) % NS);
-        bf16x8 vfirst[DVB];
+        ex8 vfirst[DVB];
         weights_checked(sc, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::true_type{}, vfirst, slot);
         pv_mma(pf, slot, vfirst, std::true_type{});
         score_mods(sn, entry_tile(ent[1]), (slot + 1) % NS);
@@ -1077,8 +1092,8 @@ void fwd_kernel(const KParams p) {
       static_while<0, NS>([&](auto idx) FL_INLINE  {
         constexpr int slot = decltype(idx)::value;
         if (last_slot != slot) return true;
-        bf16x8 pf[QB][2 * KB];
-        bf16x8 vfirst[DVB];
+        ex8 pf[QB][2 * KB];
+        ex8 vfirst[DVB];
         if constexpr (slot % 2 == 0) {
           settle(s_a, ent[0]);
           weights_checked(s_a, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot);
@@ -1135,21 +1150,21 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int dv = 32 * dvb + 8 * g + 4 * h;
-        bf16x4 o4;
+        ex4 o4;
         if (kGate && gptr) {
-          bf16x4 g4;
+          ex4 g4;
           if constexpr (kGateEarly) g4 = gpre[dvb][qb][g];
-          else g4 = *reinterpret_cast<const bf16x4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
+          else g4 = *reinterpret_cast<const ex4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
-            o4[e] = (bf16_t)(oacc[dvb][qb][4 * g + e] * sg);
+            o4[e] = (E)(oacc[dvb][qb][4 * g + e] * sg);
           }
         } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)oacc[dvb][qb][4 * g + e];
+          for (int e = 0; e < 4; ++e) o4[e] = (E)oacc[dvb][qb][4 * g + e];
         }
-        *reinterpret_cast<bf16x4*>(optr + (int64_t)qrow[qb] * p.os[2] + dv) = o4;
+        *reinterpret_cast<ex4*>(optr + (int64_t)qrow[qb] * p.os[2] + dv) = o4;
       }
   }
 }

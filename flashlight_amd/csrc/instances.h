@@ -8,6 +8,7 @@ namespace fl {
 
 struct Instance {
   const char* name;
+  int dtype;  // element type of q, k, v, o: FL_BF16 (0) or FL_F16 (2)
   int dqk, dv;
   int rw, bn, nw, ns;  // rows per wave, keys per tile, waves per workgroup, K/V tiles resident in LDS
   uint32_t feat;
@@ -32,14 +33,20 @@ hipError_t launch_fwd(const KParams& kp, int grid, int lds_bytes, hipStream_t st
 
 }  // namespace fl
 
-// Declares (FL_INSTANCE_DECL) or defines (FL_INSTANCE_DEF) the launcher of one instance.
+// Declares (FL_INSTANCE_DECL) or defines (FL_INSTANCE_DEF) the launcher of one instance for one element type
+// (SFX = _bf16 / _f16, ELEM = fl::bf16_t / fl::f16_t), and its row of the table (DT = FL_BF16 / FL_F16).
+#define FL_INSTANCE_DECL_(NAME, SFX) \
+  namespace fl { hipError_t launch_##NAME##SFX(const KParams&, int, int, hipStream_t); }
 #define FL_INSTANCE_DECL(NAME, DQK, DV, RW, BN, NW, NS, FEAT) \
-  namespace fl { hipError_t launch_##NAME(const KParams&, int, int, hipStream_t); }
-#define FL_INSTANCE_DEF(NAME, DQK, DV, RW, BN, NW, NS, FEAT)                               \
-  namespace fl {                                                                           \
-  hipError_t launch_##NAME(const KParams& kp, int grid, int lds, hipStream_t s) {          \
-    return launch_fwd<FwdTraits<DQK, DV, RW, BN, NW, (FEAT), NS>>(kp, grid, lds, s);       \
-  }                                                                                        \
+  FL_INSTANCE_DECL_(NAME, _bf16) FL_INSTANCE_DECL_(NAME, _f16)
+#define FL_INSTANCE_DEF_(NAME, SFX, ELEM, DQK, DV, RW, BN, NW, NS, FEAT)                          \
+  namespace fl {                                                                                  \
+  hipError_t launch_##NAME##SFX(const KParams& kp, int grid, int lds, hipStream_t s) {            \
+    return launch_fwd<FwdTraits<DQK, DV, RW, BN, NW, (FEAT), NS, ELEM>>(kp, grid, lds, s);        \
+  }                                                                                               \
   }
-#define FL_INSTANCE_ROW(NAME, DQK, DV, RW, BN, NW, NS, FEAT) \
-  {#NAME, DQK, DV, RW, BN, NW, NS, (FEAT), fl::FwdTraits<DQK, DV, RW, BN, NW, (FEAT), NS>::LDS_FIXED_BYTES, &fl::launch_##NAME},
+#define FL_INSTANCE_DEF(NAME, SFX, ELEM, ...) FL_INSTANCE_DEF_(NAME, SFX, ELEM, __VA_ARGS__)
+#define FL_INSTANCE_ROW_(NAME, SFX, DT, DQK, DV, RW, BN, NW, NS, FEAT) \
+  {#NAME, DT, DQK, DV, RW, BN, NW, NS, (FEAT), fl::FwdTraits<DQK, DV, RW, BN, NW, (FEAT), NS>::LDS_FIXED_BYTES, &fl::launch_##NAME##SFX},
+#define FL_INSTANCE_ROW(NAME, ...) \
+  FL_INSTANCE_ROW_(NAME, _bf16, 0, __VA_ARGS__) FL_INSTANCE_ROW_(NAME, _f16, 2, __VA_ARGS__)

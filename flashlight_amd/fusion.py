@@ -244,7 +244,8 @@ def _is_alibi(b: torch.Tensor, H: int, L: int, S: int) -> bool:
 
 # ---- the run-time side: what the replacement node calls -----------------------------------------------------------------------
 
-def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...], L: int, S: int):
+def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...], L: int, S: int,
+                 qdtype: torch.dtype = torch.bfloat16):
     """Maps a tensor broadcastable to the scores [*lead, *heads, L, S] onto the kernel's ([Nb, H|1, L|1, S], batch divisor)
     form (batch index = flat_batch // divisor), copying only when the broadcast pattern has no such form."""
     nl, nh = len(lead), len(heads)
@@ -257,7 +258,7 @@ def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...],
             raise ValueError(f"bias of shape {tuple(b.shape)} does not broadcast to the scores {(*lead, *heads, L, S)}")
     if b.dtype == torch.bool:
         raise TypeError("boolean biases are masks; use masked_fill / where")
-    if b.dtype not in (torch.bfloat16, torch.float32):
+    if b.dtype != torch.float32 and b.dtype != qdtype:
         b = b.to(torch.float32)
     if b.size(-1) != S:
         b = b.expand(*b.shape[:-1], S)
@@ -305,12 +306,12 @@ def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: 
             return t if tuple(t.shape[:-3]) == lead else t.expand(*lead, *t.shape[-3:])
 
         q4, k4, v4 = (t.reshape(-1, *t.shape[-3:]) for t in (q, like_q(k), like_q(v)))
-    kb = [_kernel_bias(b, lead, heads, L, S) for b in biases]
+    kb = [_kernel_bias(b, lead, heads, L, S, q.dtype) for b in biases]
     for i, m in enumerate(masks):
         if i < len(mask_invert) and mask_invert[i]:
             m = ~m
-        add = torch.zeros(m.shape, dtype=torch.bfloat16, device=m.device).masked_fill_(m, _NEG_INF)
-        kb.append(_kernel_bias(add, lead, heads, L, S))
+        add = torch.zeros(m.shape, dtype=q.dtype, device=m.device).masked_fill_(m, _NEG_INF)
+        kb.append(_kernel_bias(add, lead, heads, L, S, q.dtype))
     while len(kb) > 2:  # the kernel takes two operands: fold the rest into the last one
         (b1, d1), (b2, d2) = kb[-2], kb[-1]
         if d1 != d2:  # different batch groupings: give both one row per flat batch index
@@ -607,7 +608,7 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                         else:
                             kwargs.update(mask_kind=got[0], window=got[1], prefix=got[2])
                     if got is None:
-                        const_biases.append(torch.zeros(m.shape, dtype=torch.bfloat16, device=m.device)
+                        const_biases.append(torch.zeros(m.shape, dtype=_val(r.q).dtype, device=m.device)
                                             .masked_fill_(m, _NEG_INF))
                     continue
                 if len(phs) == 1 and kwargs["mask_kind"] == _ffi.MASK_NONE:

@@ -24,8 +24,8 @@ def _out_shape(q: torch.Tensor, v: torch.Tensor, diff: bool):
 def _alloc_out(q: torch.Tensor, v: torch.Tensor, diff: bool, seq_major_out: bool) -> torch.Tensor:
     B, H, L, Dv = _out_shape(q, v, diff)
     if seq_major_out:  # memory order [B, L, H, Dv] (the Evoformer layout), returned as its [B, H, L, Dv] view
-        return torch.empty((B, L, H, Dv), dtype=torch.bfloat16, device=q.device).transpose(1, 2)
-    return torch.empty((B, H, L, Dv), dtype=torch.bfloat16, device=q.device)
+        return torch.empty((B, L, H, Dv), dtype=q.dtype, device=q.device).transpose(1, 2)
+    return torch.empty((B, H, L, Dv), dtype=q.dtype, device=q.device)
 
 
 @torch.library.custom_op("flashlight_amd::attn_fwd", mutates_args=())
@@ -111,6 +111,9 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise; the
     differentiable operator when a gradient with respect to q, k or v will be asked for."""
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        if q.dtype != torch.bfloat16:
+            raise NotImplementedError("the backward kernels take bfloat16 only: call under torch.no_grad() for a forward "
+                                      f"in {q.dtype}")
         if biases or gate is not None or diff or seq_major_out:
             raise NotImplementedError(
                 "no backward is implemented for bias operands, the sigmoid gate or differential attention: call under "

@@ -43,7 +43,7 @@ enum fl_mask_kind {
                                  benchmarks/run_flex_variants.py:86) */
 };
 
-enum fl_dtype { FL_BF16 = 0, FL_F32 = 1 };
+enum fl_dtype { FL_BF16 = 0, FL_F32 = 1, FL_F16 = 2 };
 
 /* error codes (negative) */
 #define FL_ERR_NULL (-1)
@@ -82,8 +82,8 @@ typedef struct fl_attn_params {
 
   /* Optional additive biases (evoformer.py:26-27; the dense fp32 tensor `score_mod(L, S)` of alibi.py:26),
    * logical shape [B, Hq, Lq, Lk] with strides in elements over (batch / bias_batch_div, head, q, k); a
-   * stride of 0 broadcasts; the k stride must be 1 (or 0 when Lk == 1).  bias_dtype (below) selects bf16
-   * (default) or fp32 elements per operand. */
+   * stride of 0 broadcasts; the k stride must be 1 (or 0 when Lk == 1).  bias_dtype (below) says per operand
+   * whether its elements are fp32 or of the same 16-bit type as q. */
   const void* bias[2];
   int64_t bias_strides[2][4];
   int32_t bias_batch_div[2];
@@ -97,7 +97,8 @@ typedef struct fl_attn_params {
   int32_t diff;
   float lambda;
 
-  int32_t dtype; /* enum fl_dtype */
+  int32_t dtype; /* element type of q, k, v, o and gate: FL_BF16 or FL_F16 (the reference's typing admits both,
+                  * monkeypatch/fusion/_reduction.py:55-57); the backward takes FL_BF16 only */
 
   /* Scratch for the document-mask tile table; size from fl_workspace_bytes(); may be NULL otherwise. */
   void* workspace;
@@ -107,7 +108,7 @@ typedef struct fl_attn_params {
    * for every (q, k) pair it attends (after tile skipping and the element predicate). */
   uint8_t* attended_dump;
 
-  int32_t bias_dtype[2]; /* enum fl_dtype of bias[0], bias[1]: FL_BF16 or FL_F32 */
+  int32_t bias_dtype[2]; /* element type of bias[0], bias[1]: FL_F32, or the same as `dtype` */
 
   /* Optional output for a later fl_attn_bwd: fp32 [B, Hq, Lq], contiguous; per query row the base-2 logarithm of
    * the sum over attended keys of 2^(score * log2(e)) (+inf for a row that attends nothing).  Not with diff. */

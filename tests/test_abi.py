@@ -58,6 +58,16 @@ def rc(lib, p):
 def test_valid_params_pass(lib):
     for D in (32, 64, 128):
         assert rc(lib, good_params(D=D)) == 0, _ffi.last_error()
+        p = good_params(D=D)
+        p.dtype = _ffi.FL_F16
+        assert rc(lib, p) == 0, _ffi.last_error()
+    p = good_params()  # a 16-bit bias must have the element type of q
+    p.dtype = _ffi.FL_F16
+    p.bias[0], p.bias_batch_div[0] = 0x60000, 1
+    p.bias_strides[0][:] = (0, 0, 304, 1)
+    assert rc(lib, p) == -4 and "bias_dtype" in _ffi.last_error()
+    p.bias_dtype[0] = _ffi.FL_F16
+    assert rc(lib, p) == 0, _ffi.last_error()
     p = good_params()
     p.mask_kind, p.window = _ffi.MASK_SLIDING, 17
     assert rc(lib, p) == 0

@@ -406,3 +406,72 @@ def test_invariant_point_attention_far_from_the_origin_and_broadcast_bias():
     assert o_s.shape == r_s.shape == (1, 2, 2, 40, 16) and o_p.shape == r_p.shape == (1, 2, 40, 2, 8, 3)
     assert_parity(o_s, r_s, "scalar, 5-D")
     assert_parity(o_p, r_p, "points, 5-D")
+
+
+# ---- fp16 elements (the reference's typing admits them: monkeypatch/fusion/_reduction.py:55-57) ------------------------------
+
+def _half(*ts):
+    return tuple(t.to(torch.float16) for t in ts)
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_fp16_variants(D):
+    q, k, v = _half(*qkv(2, 4, 2, 333, D, seed=40 + D))
+    ref32 = f32(q, k, v)
+    cases = {
+        "vanilla": (A.attention_pytorch(q, k, v, enable_gqa=True), O.attention_vanilla(*ref32, enable_gqa=True)),
+        "causal": (A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(*ref32, enable_gqa=True)),
+        "sliding": (A.attention_pytorch_sliding_window(q, k, v, window_size=50, enable_gqa=True),
+                    O.attention_sliding_window(*ref32, window_size=50, enable_gqa=True)),
+        "prefix": (A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=77, enable_gqa=True),
+                   O.attention_prefix_lm(*ref32, prefix_lengths=77, enable_gqa=True)),
+    }
+    if D != 32:  # the score-modification and document kernels are compiled for head dims 64 and 128
+        ids = torch.arange(333).div(100, rounding_mode="floor")[None].expand(2, -1).to(DEV)
+        cases.update({
+            "alibi+softcap+causal": (
+                A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(4), enable_gqa=True,
+                                          is_causal=True, softcap=20.0),
+                O.attention_alibi(*ref32, score_mod=4, enable_gqa=True, is_causal=True, honor_causal=True, softcap=20.0)),
+            "document": (A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True, is_causal=True),
+                         O.attention_document_mask(*ref32, ids, enable_gqa=True, is_causal=True)),
+        })
+    for name, (out, ref) in cases.items():
+        assert out.dtype == torch.float16
+        assert_parity(out, ref, f"fp16 D={D} {name}")
+
+
+def test_fp16_differential_evoformer_and_mixed_types():
+    qd, kd, _ = _half(*qkv(2, 8, 8, 200, 64, seed=50))
+    vd = _half(qkv(2, 4, 4, 200, 128, seed=51)[2])[0]
+    assert_parity(A.diffattn(qd, kd, vd, lambda_full=0.7, is_causal=True),
+                  O.diff_attention(*f32(qd, kd, vd), lambda_full=0.7, is_causal=True), "fp16 diff")
+    g = torch.Generator().manual_seed(52)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.float16).to(DEV)  # noqa: E731
+    Q, K, V, G = mk(1, 3, 104, 2, 32), mk(1, 3, 104, 2, 32), mk(1, 3, 104, 2, 32), mk(1, 3, 104, 2, 32)
+    pair, mask = mk(1, 1, 2, 104, 104), mk(1, 3, 1, 1, 104)
+    out = A.attention_reference(Q, K, V, [mask, pair.float()], gate=G)  # one fp16 operand, one fp32 operand
+    assert out.dtype == torch.float16
+    assert_parity(out, O.attention_evoformer(*f32(Q, K, V), [mask.float(), pair.float()], gate=G.float()), "fp16 evoformer")
+    # element types do not mix, and the backward is bf16 only
+    qb, kb, vb = qkv(1, 2, 2, 64, 64, seed=53)
+    with pytest.raises(NotImplementedError, match="mixed element types"):
+        A.attention_pytorch(qb, kb.to(torch.float16), vb)
+    with pytest.raises(NotImplementedError, match="mixed element types"):
+        A.attention_reference(Q, K, V, [pair.bfloat16()])
+    with pytest.raises(NotImplementedError, match="bfloat16 only"):
+        A.attention_pytorch_causal(qb.to(torch.float16).requires_grad_(True), kb.to(torch.float16), vb.to(torch.float16))
+
+
+def test_fp16_large_weights_take_the_exact_path():
+    # logits that climb by hundreds per tile: weights formed against a stale reference overflow fp16 (65504), the row
+    # sums see it, and the exact path recomputes them
+    g = torch.Generator().manual_seed(54)
+    S, D = 512, 64
+    q = torch.randn(1, 1, S, D, generator=g)
+    k = torch.randn(1, 1, S, D, generator=g)
+    k[0, 0] += torch.linspace(0, 3, S).unsqueeze(1) * q[0, 0].mean(0, keepdim=True).sign()
+    v = torch.randn(1, 1, S, D, generator=g)
+    q, k, v = (t.to(torch.float16).to(DEV) for t in (q * 4, k * 4, v))
+    out = A.attention_pytorch(q, k, v, scale=1.0)
+    assert_parity(out, O.attention_vanilla(*f32(q, k, v), scale=1.0), "fp16 large logits")

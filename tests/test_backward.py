@@ -208,3 +208,19 @@ def test_gradient_properties_at_benchmark_size():
     assert all(float(t.abs().max()) == 0.0 for t in z)
     # row 0 attends only key 0, with weight 1 whatever q is: its dq is zero and dv[0] collects dout[0] in full
     assert float(q1[0, :, 0].abs().max()) < 1e-6
+
+
+@pytest.mark.gpu
+def test_gradients_under_torch_compile_equal_eager():
+    # the differentiable operator carries its autograd rule into compiled graphs (forward and backward graphs hold
+    # flashlight_amd::attn_fwd_lse and flashlight_amd::attn_bwd)
+    q, k, v, dout = _inputs(2, 4, 2, 200, 64, seed=91)
+    fn = lambda q, k, v: A.attention_pytorch_sliding_window(q, k, v, window_size=31, enable_gqa=True)  # noqa: E731
+    eager = _grads(fn, q, k, v, dout, torch.bfloat16)
+    torch._dynamo.reset()
+    compiled = _grads(torch.compile(fn, backend="aot_eager", fullgraph=True), q, k, v, dout, torch.bfloat16)
+    for a, b in zip(eager, compiled):
+        assert torch.equal(a, b)
+    torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd_lse.default,
+                          (q.detach().requires_grad_(True), k, v, -1.0, 1, 0, 0, None, 0, 0.0),
+                          test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))

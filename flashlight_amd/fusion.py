@@ -96,19 +96,6 @@ def _is_last2_transpose(n: Any) -> Optional[fx.Node]:
     return None
 
 
-def _depends_on(n: Any, target: fx.Node, memo: Dict[fx.Node, bool]) -> bool:
-    if not isinstance(n, fx.Node):
-        return False
-    if n is target:
-        return True
-    if n in memo:
-        return memo[n]
-    memo[n] = False
-    r = any(_depends_on(a, target, memo) for a in n.all_input_nodes)
-    memo[n] = r
-    return r
-
-
 def _placeholders_of(n: fx.Node) -> List[fx.Node]:
     seen, out, stack = set(), [], [n]
     while stack:

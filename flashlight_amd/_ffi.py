@@ -44,7 +44,8 @@ class FlAttnParams(C.Structure):
         ("attended_dump", C.c_void_p),
         ("bias_dtype", C.c_int32 * 2),
         ("lse", C.c_void_p),
-        ("reserved", C.c_int32 * 4),
+        ("dropout_threshold", C.c_uint32), ("dropout_seed", C.c_uint32 * 2),
+        ("reserved", C.c_int32 * 1),
     ]
 
 
@@ -173,8 +174,16 @@ def _dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def dropout_threshold(p: float) -> int:
+    """16-bit threshold of dropout rate p (0 = off): the kernels drop a weight when its 16 hash bits are below it, so
+    the rate in effect is threshold / 65536."""
+    if not 0.0 <= p < 1.0:
+        raise ValueError(f"dropout_p must be in [0, 1), got {p}")
+    return min(int(round(p * 65536.0)), 65535)
+
+
 def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases,
-                 gate, diff, lambda_full, attended_dump):
+                 gate, diff, lambda_full, attended_dump, dropout_p=0.0, dropout_seed=0):
     """Fills an `fl_attn_params` for validated 4-D tensors; returns it with the tensors that must outlive the launch."""
     B, _, Lq, Dqk = q.shape
     Lk, Dv = k.shape[2], v.shape[3]
@@ -187,6 +196,8 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
     p.B, p.Hq, p.Hkv, p.Lq, p.Lk, p.Dqk, p.Dv = B, Hq, Hkv, Lq, Lk, Dqk, Dv
     p.scale = float(1.0 / math.sqrt(Dqk) if scale is None else scale)
     p.mask_kind, p.window, p.prefix = int(mask_kind), int(window), int(prefix)
+    p.dropout_threshold = dropout_threshold(float(dropout_p))
+    p.dropout_seed[0], p.dropout_seed[1] = int(dropout_seed) & 0xFFFFFFFF, (int(dropout_seed) >> 32) & 0xFFFFFFFF
     keep = [q, k, v, out]
     if doc_ids is not None:
         if doc_ids.dim() != 2 or doc_ids.shape[1] != Lk or doc_ids.shape[0] not in (1, B):
@@ -272,6 +283,8 @@ def attn_fwd(
     attended_dump: Optional[torch.Tensor] = None,
     validate_only: bool = False,
     lse: Optional[torch.Tensor] = None,
+    dropout_p: float = 0.0,
+    dropout_seed: int = 0,
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
@@ -279,6 +292,8 @@ def attn_fwd(
     [B/batch_div, Hq, Lq, Lk] (size-1 axes broadcast).  q, k, v (and gate, 16-bit biases) are all bf16 or all fp16.  Returns `out` [B, Hq, Lq, Dv]
     in that type, written on the current stream.
     `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
+    `dropout_p` > 0 drops softmax weights (torch.nn.functional.dropout semantics) by a hash of (`dropout_seed`, batch,
+    head, query, key); positional masks and GQA only.
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -315,7 +330,7 @@ def attn_fwd(
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                           biases, gate, diff, lambda_full, attended_dump)
+                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed)
     if lse is not None:
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
             raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")
@@ -334,8 +349,8 @@ def attn_fwd(
 def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, dout: torch.Tensor,
              *, scale: Optional[float] = None, mask_kind: int = MASK_NONE, window: int = 0, prefix: int = 0,
              doc_ids: Optional[torch.Tensor] = None, alibi_heads: int = 0, softcap: float = 0.0,
-             validate_only: bool = False):
-    """Gradients (dq, dk, dv) of `attn_fwd` called with the same arguments; `out` and `lse` are what that call
+             validate_only: bool = False, dropout_p: float = 0.0, dropout_seed: int = 0):
+    """Gradients (dq, dk, dv) of `attn_fwd` called with the same arguments (dropout rate and seed included); `out` and `lse` are what that call
     returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream."""
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
@@ -350,7 +365,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
         raise ValueError("lse must be the contiguous float32 [B, Hq, Lq] tensor the forward filled")
     fwd, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                             (), None, False, 0.0, None)
+                             (), None, False, 0.0, None, dropout_p, dropout_seed)
     fwd.lse = lse.data_ptr()
     dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
         torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)

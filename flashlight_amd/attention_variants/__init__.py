@@ -15,3 +15,4 @@ from .document_mask import attention_pytorch_document_mask, create_document_id  
 from .diff_attn import diffattn  # noqa: F401
 from .evoformer import attention_reference  # noqa: F401
 from .ipa import invariant_point_attention  # noqa: F401
+from ._common import honor_dropout  # noqa: F401

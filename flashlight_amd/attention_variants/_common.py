@@ -32,6 +32,33 @@ def grouped_view(out: torch.Tensor, key: torch.Tensor, enable_gqa: bool) -> torc
     return out.view(n, hkv, hq // hkv, l, ev)
 
 
-def run(query, key, value, *, scale: Optional[float], enable_gqa: bool, **kw) -> torch.Tensor:
+_honor_dropout = False
+
+
+class honor_dropout:
+    """The reference's variants take `dropout_p` and ignore it (attention_variants/causal.py:4-36, alibi.py:13-33,
+    softcap.py:4-53), and so do this package's by default.  `honor_dropout(True)` (also usable as a context manager:
+    `with honor_dropout(): ...`) makes them apply it: softmax weights are dropped with probability `dropout_p` and the
+    kept ones scaled by 1 / (1 - p), as torch.nn.functional.dropout would.  Seeds come from torch's default CPU
+    generator.  The kernels have dropout for positional masks only: the causal variant takes it; ALiBi and soft-cap
+    calls with dropout_p > 0 raise."""
+
+    def __init__(self, enabled: bool = True):
+        global _honor_dropout
+        self._previous = _honor_dropout
+        _honor_dropout = bool(enabled)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        global _honor_dropout
+        _honor_dropout = self._previous
+        return False
+
+
+def run(query, key, value, *, scale: Optional[float], enable_gqa: bool, dropout_p: float = 0.0, **kw) -> torch.Tensor:
     check_heads(query, key, value, enable_gqa)
+    if _honor_dropout and dropout_p:
+        kw["dropout_p"] = float(dropout_p)
     return ops.dispatch(query, key, value, scale=scale, **kw)

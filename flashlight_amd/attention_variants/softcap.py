@@ -43,5 +43,6 @@ def attention_softcapped(query: torch.Tensor, key: torch.Tensor, value: torch.Te
             "score_mod must come from generate_tanh_softcap(): the fused kernel applies cap * tanh(x / cap) in "
             "registers and cannot call an arbitrary Python function on the score matrix")
     out = run(query, key, value, scale=scale, enable_gqa=enable_gqa,
-              mask_kind=_ffi.MASK_CAUSAL if is_causal else _ffi.MASK_NONE, softcap=score_mod.soft_cap)
+              mask_kind=_ffi.MASK_CAUSAL if is_causal else _ffi.MASK_NONE, softcap=score_mod.soft_cap,
+              dropout_p=dropout_p)
     return grouped_view(out, key, enable_gqa)

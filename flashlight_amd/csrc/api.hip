@@ -52,6 +52,7 @@ uint32_t wanted_features(const fl_attn_params* p) {
   if (p->diff) f |= fl::F_DIFF;
   if (p->gate) f |= fl::F_GATE;
   if (p->attended_dump) f |= fl::F_DUMP;
+  if (p->dropout_threshold) f |= fl::F_DROPOUT;
   return f;
 }
 
@@ -133,8 +134,15 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if ((rc = check_strides("q", p->q_strides, 8)) || (rc = check_strides("k", p->k_strides, 8)) ||
       (rc = check_strides("v", p->v_strides, 8)) || (rc = check_strides("o", p->o_strides, 4)))
     return rc;
-  for (int i = 0; i < 4; ++i)
-    if (p->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
+  if (p->reserved[0] != 0) return fail(FL_ERR_ARG, "reserved[0] must be 0");
+  if (p->dropout_threshold) {
+    if (p->dropout_threshold > 65535u)
+      return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
+    if (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind) || p->bias[0] || p->bias[1] || p->gate || p->diff ||
+        p->attended_dump)
+      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional masks only (no ALiBi, soft-cap, document mask, bias, "
+                                      "gate, differential attention, dump)");
+  }
   if (p->lse) {
     if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
     if (p->diff) return fail(FL_ERR_UNSUPPORTED, "lse is not produced for differential attention");
@@ -323,6 +331,10 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   }
   kp.dump = p->attended_dump;
   kp.lse = p->lse;
+  kp.drop_thr = p->dropout_threshold;
+  kp.drop_seed[0] = p->dropout_seed[0];
+  kp.drop_seed[1] = p->dropout_seed[1];
+  kp.drop_rescale = 65536.0f / (65536.0f - (float)p->dropout_threshold);
   const int bm = in->rw * in->nw;
   kp.n_qtiles = (p->Lq + bm - 1) / bm;
   kp.n_ktiles = (p->Lk + in->bn - 1) / in->bn;
@@ -378,6 +390,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     if (want) return fail(FL_ERR_UNSUPPORTED, "backward: document masks cannot be combined with ALiBi or a soft-cap");
     want = fl::F_DOC;
   }
+  if (p->dropout_threshold) want = fl::F_DROPOUT;  // validate() has excluded every other feature
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want) in = &fl::kBwdInstances[i];
@@ -440,6 +453,10 @@ int fl_attn_bwd(const fl_attn_bwd_params* b, void* stream_) {
   bp.doc_stride = p->doc_stride;
   bp.alibi_heads = p->alibi_heads;
   bp.softcap = p->softcap;
+  bp.drop_thr = p->dropout_threshold;
+  bp.drop_seed[0] = p->dropout_seed[0];
+  bp.drop_seed[1] = p->dropout_seed[1];
+  bp.drop_rescale = 65536.0f / (65536.0f - (float)p->dropout_threshold);
   if (is_doc(p->mask_kind)) {
     const int blocks = (p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
     const int total = p->B * blocks;

@@ -46,6 +46,9 @@ struct BParams {
   int32_t doc_blocks;
   int32_t alibi_heads;
   float softcap;
+  uint32_t drop_thr;      // as in KParams: 0 = no dropout
+  uint32_t drop_seed[2];
+  float drop_rescale;
 };
 
 // Delta[b, h, q] = sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
@@ -103,6 +106,7 @@ void bwd_kernel(const BParams p) {
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC;
   constexpr bool kDQ = ROLE == ROLE_DQ;
+  constexpr bool kDrop = FEAT & F_DROPOUT;
   constexpr float kLog2e = 1.4426950408889634f;
   using L = TileLayout<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -329,7 +333,14 @@ void bwd_kernel(const BParams p) {
         return out;
       };
       bf16x8 pf[2 * TB], dsf[2 * TB];
-      float pd[TB][16];  // weight times d(score) / d(qk * scale)
+      float pd[TB][16];  // weight times d(score) / d(qk * scale); with dropout its sign bit marks a dropped weight
+      // dropout: the owner position's share of the hash argument (see drop_pair_hash); the streamed head changes from step
+      // to step in ROLE_DKV
+      uint32_t drop_o = 0;
+      if constexpr (kDrop) {
+        const uint32_t s0 = drop_head_seed(p.drop_seed[0], p.drop_seed[1], (uint32_t)(batch * p.Hq + shead));
+        drop_o = s0 + (kDQ ? (uint32_t)opos * kDropQ : (uint32_t)(opos >> 1) * kDropK);
+      }
       {
         f32x16 x1[TB];
 #pragma unroll
@@ -396,6 +407,27 @@ void bwd_kernel(const BParams p) {
               pd[sb][i] = kSoftcap ? pw * dfac : pw;
             }
           }
+          if constexpr (kDrop) {
+            // ROLE_DQ: registers (i, i + 1), i even, are the key pair (sbase + off) / 2 of this lane's query: one hash.
+            // ROLE_DKV: register i is query sbase + off against this lane's key: its own hash, the key's half of it.
+#pragma unroll
+            for (int i = 0; i < 16; i += kDQ ? 2 : 1) {
+              const int off = 8 * (i / 4) + i % 4;
+              if constexpr (kDQ) {
+                const uint32_t x = drop_pair_hash(drop_o + (uint32_t)((sbase + off) >> 1) * kDropK);
+                const bool keep0 = (x & 0xFFFFu) >= p.drop_thr, keep1 = (x >> 16) >= p.drop_thr;
+                pv[i] = keep0 ? pv[i] : 0.f;
+                pv[i + 1] = keep1 ? pv[i + 1] : 0.f;
+                pd[sb][i] = keep0 ? pd[sb][i] : -pd[sb][i];
+                pd[sb][i + 1] = keep1 ? pd[sb][i + 1] : -pd[sb][i + 1];
+              } else {
+                const uint32_t x = drop_pair_hash(drop_o + (uint32_t)(sbase + off) * kDropQ);
+                const bool keep = ((x >> (16 * (opos & 1))) & 0xFFFFu) >= p.drop_thr;
+                pv[i] = keep ? pv[i] : 0.f;
+                pd[sb][i] = keep ? pd[sb][i] : -pd[sb][i];
+              }
+            }
+          }
 #pragma unroll
           for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -426,7 +458,14 @@ void bwd_kernel(const BParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * g + e;
-              const float ds = pd[sb][i] * (x2[sb][i] - (kDQ ? delta_o : dl4[e]));
+              float ds;
+              if constexpr (kDrop) {
+                // d(loss) / d(weight) is dP / (1 - p) where the weight was kept and 0 where it was dropped
+                const bool kept = __builtin_bit_cast(int, pd[sb][i]) >= 0;
+                ds = __builtin_fabsf(pd[sb][i]) * ((kept ? x2[sb][i] * p.drop_rescale : 0.f) - (kDQ ? delta_o : dl4[e]));
+              } else {
+                ds = pd[sb][i] * (x2[sb][i] - (kDQ ? delta_o : dl4[e]));
+              }
               dsf[2 * sb + i / 8][i % 8] = (bf16_t)ds;
             }
           }
@@ -492,7 +531,7 @@ void bwd_kernel(const BParams p) {
         for (int g = 0; g < 4; ++g) {
           bf16x4 o4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)acc2[db][4 * g + e];
+          for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)(kDrop ? acc2[db][4 * g + e] * p.drop_rescale : acc2[db][4 * g + e]);
           *reinterpret_cast<bf16x4*>(out2 + 32 * db + 8 * g + 4 * h) = o4;
         }
     }

@@ -37,6 +37,7 @@ enum : uint32_t {
   F_DIFF = 16u,    // two softmax branches, out = A0 - lambda * A1
   F_GATE = 32u,    // out *= sigmoid(gate)
   F_DUMP = 64u,    // write the attended-pair bitmap (test hook), skip nothing else
+  F_DROPOUT = 128u,  // softmax weights are dropped by a counter-based hash of (seed, batch, head, query, key)
 };
 
 enum : int { MASK_NONE = 0, MASK_CAUSAL = 1, MASK_SLIDING = 2, MASK_PREFIX = 3, MASK_DOC = 4, MASK_DOC_CAUSAL = 5 };
@@ -79,11 +80,50 @@ struct KParams {
   int64_t q_branch_stride, k_branch_stride;  // element offset of the second softmax branch (diff)
   uint8_t* dump;
   float* lse;        // optional [B, Hq, Lq]: log2 of the row's sum of 2^(logit in log2 units); +inf if nothing attended
+  uint32_t drop_thr;      // a weight is dropped when its 16 hash bits are < drop_thr (1 .. 65535; 0: no dropout)
+  uint32_t drop_seed[2];  // low and high half of the 64-bit seed
+  float drop_rescale;     // 65536 / (65536 - drop_thr), applied to the kept weights
   int32_t n_qtiles;  // ceil(Lq / BM)
   int32_t n_ktiles;  // ceil(Lk / BN)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- dropout decisions ------------------------------------------------------------------------------------------------
+// Whether the weight of (batch, head, query q, key k) survives is a pure function of those and the seed, so that the
+// forward, both backward kernels and a CPU restatement agree without exchanging a mask.  One 32-bit hash serves the
+// key pair (2j, 2j + 1): the even key takes the low 16 bits, the odd key the high 16, and a weight is dropped when its
+// 16 bits are below the threshold.  The hash of x = head_seed + q * kDropQ + (k / 2) * kDropK is two rounds of a
+// 24-bit multiply-add between xor-shifts: full-rate vector instructions only (a 32-bit multiply is quarter rate).
+constexpr uint32_t kDropQ = 0x9E3779B1u, kDropK = 0x85EBCA77u;
+__device__ __forceinline__ uint32_t drop_fmix32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x85EBCA6Bu;
+  x ^= x >> 13;
+  x *= 0xC2B2AE35u;
+  x ^= x >> 16;
+  return x;
+}
+// start value of head bh = batch * Hq + head (once per workgroup: the 32-bit multiplies do not matter here)
+__device__ __forceinline__ uint32_t drop_head_seed(uint32_t seed_lo, uint32_t seed_hi, uint32_t bh) {
+  return drop_fmix32(seed_lo ^ drop_fmix32(seed_hi + 0x9E3779B9u * (bh + 1u)));
+}
+__device__ __forceinline__ uint32_t drop_pair_hash(uint32_t x) {
+  x ^= x >> 16;
+  x = (x & 0xFFFFFFu) * 0xCA6B35u + (x >> 8);
+  x ^= x >> 13;
+  x = ((x >> 8) & 0xFFFFFFu) * 0xB2AE3Du + x;
+  x ^= x >> 16;
+  return x;
+}
+// 0xFFFF in each half of the result whose 16 hash bits are > c (c = threshold - 1 in both halves of c2): three packed
+// 16-bit instructions
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t drop_pair_mask(uint32_t hash, uint32_t c2) {
+  const u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, hash), __builtin_bit_cast(u16x2, c2));
+  const u16x2 one = {1, 1}, all = {0xFFFF, 0xFFFF};
+  return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_elementwise_min(d, one) * all));
+}
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 // Exchange between the two half-waves: returns (x[l % 32], x[l % 32 + 32]) in every lane.
@@ -324,6 +364,7 @@ void fwd_kernel(const KParams p) {
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kBias = FEAT & F_BIAS, kDoc = FEAT & F_DOC;
   constexpr bool kDiff = FEAT & F_DIFF, kGate = FEAT & F_GATE, kDump = FEAT & F_DUMP;
+  constexpr bool kDrop = FEAT & F_DROPOUT;
   constexpr bool kMod = kAlibi || kSoftcap || kBias;  // scores are transformed before the softmax
   constexpr float kLog2e = 1.4426950408889634f;
   using E = typename T::Elem;  // pointers in KParams are typed bf16_t whatever E is: 16 opaque bits
@@ -496,6 +537,15 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
       qdoc[qb] = p.doc_ids[(int64_t)batch * p.doc_stride + min(qrow[qb], p.Lq - 1)];
+  }
+  // dropout: this lane's rows' share of the hash argument, and the threshold (minus one) in both 16-bit halves
+  uint32_t drop_q[QB];
+  uint32_t drop_c2 = 0;
+  if constexpr (kDrop) {
+    const uint32_t s0 = drop_head_seed(p.drop_seed[0], p.drop_seed[1], (uint32_t)(batch * p.Hq + head));
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) drop_q[qb] = s0 + (uint32_t)qrow[qb] * kDropQ;
+    drop_c2 = (p.drop_thr - 1u) * 0x10001u;
   }
   // With dense biases as the only score modification the modified scores stay in natural units (s = qk * scale + bias)
   // and the factor log2(e) rides in the exponential's multiply-add; other modifications produce log2 units directly.
@@ -907,12 +957,16 @@ void fwd_kernel(const KParams p) {
     };
 
     // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
-    auto softmax_p = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], float (&rsum)[QB]) FL_INLINE {
+    // (the row sums take every weight; with dropout the weights that go on to the second product are then thinned:
+    // t is the tile, whose keys enter the hash)
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], float (&rsum)[QB], int t) FL_INLINE {
       const ex2 ones = {(E)1.0f, (E)1.0f};
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
         float rs = 0.f;
+        uint32_t drop_x0 = 0;
+        if constexpr (kDrop) drop_x0 = drop_q[qb] + (uint32_t)(t * (BN / 2) + 2 * h) * kDropK;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
           float pv[16];
@@ -928,6 +982,15 @@ void fwd_kernel(const KParams p) {
             for (int e = 0; e < 8; e += 2) {
               const ex2 pr = {pf[qb][2 * kb + j][e], pf[qb][2 * kb + j][e + 1]};
               rs = dot2acc(pr, ones, rs);
+              if constexpr (kDrop) {
+                // registers 8j + e, 8j + e + 1 are keys t BN + 32 kb + 8 (2j + e / 4) + 4h + e % 4 and the next one
+                // (pair index = (t BN) / 2 + 2h + a constant: one multiply per tile, one add per pair)
+                const uint32_t x = drop_x0 + (uint32_t)((32 * kb + 8 * (2 * j + e / 4) + e % 4) / 2) * kDropK;
+                const uint32_t m = drop_pair_mask(drop_pair_hash(x), drop_c2);
+                const ex2 kept = __builtin_bit_cast(ex2, __builtin_bit_cast(uint32_t, pr) & m);
+                pf[qb][2 * kb + j][e] = kept[0];
+                pf[qb][2 * kb + j][e + 1] = kept[1];
+              }
             }
           }
         }
@@ -944,15 +1007,15 @@ void fwd_kernel(const KParams p) {
     constexpr float kBig = 0x1p24f, kTiny = 0x1p-24f;
     constexpr bool kFastRef = true;
     auto weights_checked = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], bool check, auto in_loop,
-                               ex8 (&vfirst)[DVB], int vslot) FL_INLINE {
+                               ex8 (&vfirst)[DVB], int vslot, int t) FL_INLINE {
       float rs[QB];
-      softmax_p(s, pf, rs);
+      softmax_p(s, pf, rs, t);
       if constexpr (decltype(in_loop)::value) {
         // inside the pipelined step the exponentials share a block with the first product's MFMAs (issued by the
         // caller just before): interleave them
         constexpr int NA = KS * KB * QB;
         constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp per score, one pack and one dot2 per two
-        sched_first_product<NA, (n_exp * 3 + NA - 1) / NA>();
+        sched_first_product<NA, (n_exp * (kDrop ? 9 : 3) + NA - 1) / NA>();
       }
       if constexpr (decltype(in_loop)::value) {
         // the second product's first V fragments are fetched here, ahead of the branch below, so that their LDS
@@ -970,7 +1033,7 @@ void fwd_kernel(const KParams p) {
           float mx[QB];
           row_max(s, mx);
           rescale_if_grown(mx, true);
-          softmax_p(s, pf, rs);
+          softmax_p(s, pf, rs, t);
         }
       }
 #pragma unroll
@@ -1057,7 +1120,8 @@ void fwd_kernel(const KParams p) {
         __builtin_amdgcn_s_setprio(3);
         qk(sn, (slot + 1) % NS);
         ex8 vfirst[DVB];
-        weights_checked(sc, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::true_type{}, vfirst, slot);
+        weights_checked(sc, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::true_type{}, vfirst, slot,
+                        entry_tile(ent[0]));
         pv_mma(pf, slot, vfirst, std::true_type{});
         score_mods(sn, entry_tile(ent[1]), (slot + 1) % NS);
         {
@@ -1096,10 +1160,12 @@ void fwd_kernel(const KParams p) {
         ex8 vfirst[DVB];
         if constexpr (slot % 2 == 0) {
           settle(s_a, ent[0]);
-          weights_checked(s_a, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot);
+          weights_checked(s_a, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot,
+                          entry_tile(ent[0]));
         } else {
           settle(s_b, ent[0]);
-          weights_checked(s_b, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot);
+          weights_checked(s_b, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot,
+                          entry_tile(ent[0]));
         }
         pv_mma(pf, slot, vfirst, std::false_type{});
         return false;
@@ -1110,7 +1176,8 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const float l = xhalf_sum(l_run[qb]);
-      const float inv = l > 0.f ? 1.0f / l : 0.f;  // a row that attends nothing yields zeros
+      float inv = l > 0.f ? 1.0f / l : 0.f;  // a row that attends nothing yields zeros
+      if constexpr (kDrop) inv *= p.drop_rescale;  // the row sum counted every weight; the kept ones are scaled up
       if constexpr (!kDiff) {
         // row statistic for a backward pass: weights were exp2(s * c2 - m_run * c2), so the row's log2-sum-exp2 is
         if (p.lse != nullptr && h == 0 && qrow[qb] < p.Lq) {

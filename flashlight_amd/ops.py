@@ -54,19 +54,23 @@ def _attn_fwd_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_hea
 
 @torch.library.custom_op("flashlight_amd::attn_fwd_lse", mutates_args=())
 def attn_fwd_lse(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, mask_kind: int, window: int, prefix: int,
-                 doc_ids: Optional[torch.Tensor], alibi_heads: int, softcap: float) -> tuple[torch.Tensor, torch.Tensor]:
+                 doc_ids: Optional[torch.Tensor], alibi_heads: int, softcap: float, dropout_p: float = 0.0,
+                 dropout_seed: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
     """The forward for calls that will be differentiated: also returns the row statistics (float32 [B, Hq, Lq], log2 of
     each row's sum of 2^logit) from which `attn_bwd` recomputes the weights.  The reference has no backward; this
-    operator carries the autograd rule registered below."""
+    operator carries the autograd rule registered below.  It is also the operator for a forward with dropout: which
+    weights are dropped is a function of `dropout_seed`, so the backward needs no mask from the forward."""
     out = _alloc_out(q, v, False, False)
     lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
     _ffi.attn_fwd(q, k, v, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window, prefix=prefix,
-                  doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, out=out, lse=lse)
+                  doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, out=out, lse=lse, dropout_p=dropout_p,
+                  dropout_seed=dropout_seed)
     return out, lse
 
 
 @attn_fwd_lse.register_fake
-def _attn_fwd_lse_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap):
+def _attn_fwd_lse_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, dropout_p=0.0,
+                       dropout_seed=0):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, dim]")
     return _alloc_out(q, v, False, False), torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
@@ -75,42 +79,63 @@ def _attn_fwd_lse_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi
 @torch.library.custom_op("flashlight_amd::attn_bwd", mutates_args=())
 def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, dout: torch.Tensor,
              scale: float, mask_kind: int, window: int, prefix: int, doc_ids: Optional[torch.Tensor], alibi_heads: int,
-             softcap: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+             softcap: float, dropout_p: float = 0.0,
+             dropout_seed: int = 0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dq, dk, dv) of `attn_fwd_lse` for the output gradient `dout`."""
     return _ffi.attn_bwd(q, k, v, out, lse, dout, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window,
-                         prefix=prefix, doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap)
+                         prefix=prefix, doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, dropout_p=dropout_p,
+                         dropout_seed=dropout_seed)
 
 
 @attn_bwd.register_fake
-def _attn_bwd_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap):
+def _attn_bwd_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
+                   dropout_p=0.0, dropout_seed=0):
     c = torch.contiguous_format
     return torch.empty_like(q, memory_format=c), torch.empty_like(k, memory_format=c), torch.empty_like(v, memory_format=c)
 
 
 def _setup_context(ctx, inputs, output):
-    q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap = inputs
+    q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, dropout_p, dropout_seed = inputs
     out, lse = output
     ctx.save_for_backward(q, k, v, out, lse)
     ctx.doc_ids = doc_ids
-    ctx.args = (scale, mask_kind, window, prefix, alibi_heads, softcap)
+    ctx.args = (scale, mask_kind, window, prefix, alibi_heads, softcap, dropout_p, dropout_seed)
 
 
 def _backward(ctx, dout, dlse):
     q, k, v, out, lse = ctx.saved_tensors
-    scale, mask_kind, window, prefix, alibi_heads, softcap = ctx.args
+    scale, mask_kind, window, prefix, alibi_heads, softcap, dropout_p, dropout_seed = ctx.args
     dq, dk, dv = attn_bwd(q, k, v, out, lse, dout.to(torch.bfloat16), scale, mask_kind, window, prefix, ctx.doc_ids,
-                          alibi_heads, softcap)
-    return dq, dk, dv, None, None, None, None, None, None, None
+                          alibi_heads, softcap, dropout_p, dropout_seed)
+    return dq, dk, dv, None, None, None, None, None, None, None, None, None
 
 
 attn_fwd_lse.register_autograd(_backward, setup_context=_setup_context)
 
 
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
-             softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False) -> torch.Tensor:
+             softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
+             dropout_seed=None) -> torch.Tensor:
     """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise; the
-    differentiable operator when a gradient with respect to q, k or v will be asked for."""
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+    differentiable operator when a gradient with respect to q, k or v will be asked for.
+
+    `dropout_p` > 0 drops softmax weights (the reference's functions ignore their `dropout_p`; see
+    `attention_variants.honor_dropout`).  `dropout_seed=None` draws a fresh 63-bit seed from torch's default CPU
+    generator, so `torch.manual_seed` reproduces a run; the same seed gives the same decisions in forward and backward."""
+    dropout_p = float(dropout_p)
+    _ffi.dropout_threshold(dropout_p)  # range check
+    if dropout_p > 0.0:
+        if biases or gate is not None or diff or seq_major_out:
+            raise NotImplementedError("dropout is built for positional masks and grouped-query attention only")
+        if dropout_seed is None:
+            if torch.compiler.is_compiling():
+                raise NotImplementedError("dropout under torch.compile needs an explicit dropout_seed (a seed drawn "
+                                          "while tracing would be frozen into the graph)")
+            dropout_seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
+    else:
+        dropout_seed = 0
+    if (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) or \
+            (dropout_p > 0.0 and torch.compiler.is_compiling()):
         if q.dtype != torch.bfloat16:
             raise NotImplementedError("the backward kernels take bfloat16 only: call under torch.no_grad() for a forward "
                                       f"in {q.dtype}")
@@ -119,7 +144,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
                 "no backward is implemented for bias operands, the sigmoid gate or differential attention: call under "
                 "torch.no_grad() (or detach the inputs) if only the forward is wanted")
         out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
-                              int(prefix), doc_ids, int(alibi_heads), float(softcap))
+                              int(prefix), doc_ids, int(alibi_heads), float(softcap), dropout_p, int(dropout_seed))
         return out
     if torch.compiler.is_compiling():
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
@@ -129,4 +154,4 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None
     return _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                          alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
-                         lambda_full=lambda_full, out=out)
+                         lambda_full=lambda_full, out=out, dropout_p=dropout_p, dropout_seed=dropout_seed)

@@ -114,7 +114,17 @@ typedef struct fl_attn_params {
    * the sum over attended keys of 2^(score * log2(e)) (+inf for a row that attends nothing).  Not with diff. */
   float* lse;
 
-  int32_t reserved[4]; /* must be 0 */
+  /* Dropout on the softmax weights (torch.nn.functional.dropout semantics: the row normalisation counts every weight,
+   * kept weights are scaled by 65536 / (65536 - dropout_threshold)).  The reference's functions accept `dropout_p` and
+   * ignore it (attention_variants/causal.py:4-36, alibi.py:13-33, softcap.py:4-53); 0 here does the same.
+   * dropout_threshold = round(p * 65536), 1 .. 65535: a weight is dropped when the 16 bits a counter-based hash of
+   * (dropout_seed, batch * Hq + head, query, key) gives it are below the threshold.  fl_attn_bwd regenerates the same
+   * decisions from the same fields.  Positional masks and GQA only: not with ALiBi, a soft-cap, document masks, bias
+   * operands, gate, differential attention or the dump hook; Dqk = Dv in {64, 128}. */
+  uint32_t dropout_threshold;
+  uint32_t dropout_seed[2]; /* low, high half of a 64-bit seed */
+
+  int32_t reserved[1]; /* must be 0 */
 } fl_attn_params;
 
 /* ABI version of the loaded library (FL_ABI_VERSION it was built with). */

@@ -19,6 +19,10 @@ How each function is pinned (tests/test_oracle_pinned.py) without running the re
   IPA                pure-Python loops over queries, keys and points with math.exp at N <= 6; zero points == SDPA with
                      the pair bias as float mask; a common translation of query and key points changes nothing;
                      two keys at distances d1, d2 get weights in the ratio exp(w (d1^2 - d2^2))
+  dropout            (oracle/dropout.py; the reference ignores dropout_p) all kept == SDPA; the 1 / (1 - p) factor against
+                     torch.nn.functional.dropout; mean over 400 seeds approaches the undropped result; the keep decisions
+                     against a second restatement in plain Python integers, frozen values and correlation statistics;
+                     gradients by central differences (tests/test_dropout.py)
 The committed fixtures under tests/golden/ were produced by tests/golden/make_golden.py from those library
 routines (never from this package), so they pin it from outside as well.
 """

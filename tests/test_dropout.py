@@ -1,0 +1,306 @@
+"""Dropout on the softmax weights.  The reference's variants accept `dropout_p` and ignore it (attention_variants/
+causal.py:4-36, alibi.py:13-33, softcap.py:4-53), so there is no reference output to compare with.  What is pinned:
+
+  * the semantics (oracle/dropout.py) against library routines: all weights kept == scaled_dot_product_attention; the
+    1 / (1 - p) convention against torch.nn.functional.dropout; the mean over many seeds approaches the undropped result;
+  * the decision function: a second restatement in plain Python integers, frozen known values, and its statistics
+    (rate, uniformity, no correlation along rows, columns, diagonals, heads or seeds);
+  * its gradients: autograd through the oracle against central differences in float64;
+  * the kernels (GPU tests): forward and gradients, through the C ABI, against the oracle given the same seed.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import flashlight_amd.attention_variants as A
+from flashlight_amd import _ffi, ops
+from oracle import dropout as OD
+from tests.conftest import assert_parity
+from tests.test_abi import good_params
+
+DEV = "cuda"
+
+
+# ---- the decision function -------------------------------------------------------------------------------------------------
+
+def _scalar_random16(seed, bh, q, k):
+    """The same 16 bits in plain Python integers (no numpy), written from the description in oracle/dropout.py."""
+    m = 0xFFFFFFFF
+
+    def fmix(x):
+        x &= m
+        x ^= x >> 16
+        x = (x * 0x85EBCA6B) & m
+        x ^= x >> 13
+        x = (x * 0xC2B2AE35) & m
+        return x ^ (x >> 16)
+
+    s0 = fmix((seed & m) ^ fmix(((seed >> 32) + 0x9E3779B9 * (bh + 1)) & m))
+    x = (s0 + q * 0x9E3779B1 + (k // 2) * 0x85EBCA77) & m
+    x ^= x >> 16
+    x = ((x & 0xFFFFFF) * 0xCA6B35 + (x >> 8)) & m
+    x ^= x >> 13
+    x = (((x >> 8) & 0xFFFFFF) * 0xB2AE3D + x) & m
+    x ^= x >> 16
+    return (x >> 16) if k % 2 else (x & 0xFFFF)
+
+
+def test_decision_bits_two_restatements_and_known_values():
+    for seed, bh in ((0, 0), (1234, 3), (2 ** 63 + 12345, 63), (0xFFFFFFFFFFFFFFFF, 7)):
+        r = OD.random16(seed, bh, 9, 14)
+        for q in range(9):
+            for k in range(14):
+                assert r[q, k] == _scalar_random16(seed, bh, q, k), (seed, bh, q, k)
+    # frozen values: a change of any constant, shift or operand order shows up here
+    assert OD.head_seed(0, 0) == 2856213345 and OD.head_seed(1, 5) == 4171907236
+    assert OD.random16(1234, 3, 2, 8).tolist() == [[12170, 21700, 45079, 30570, 41986, 25535, 54504, 33553],
+                                                    [45153, 33049, 5915, 51856, 49463, 23721, 16504, 11248]]
+    # positions far out (32-bit wrap-around of the products)
+    r = OD.random16(99, 1, 70000, 6)[-1]
+    assert [int(x) for x in r] == [_scalar_random16(99, 1, 69999, k) for k in range(6)]
+
+
+def test_threshold_and_effective_rate():
+    assert OD.threshold16(0.0) == 0 and OD.threshold16(0.5) == 32768 and OD.threshold16(0.1) == 6554
+    assert OD.threshold16(0.9999999) == 65535
+    assert _ffi.dropout_threshold(0.1) == OD.threshold16(0.1) and _ffi.dropout_threshold(0.25) == 16384
+    for bad in (-0.1, 1.0, 2.0):
+        with pytest.raises(ValueError):
+            OD.threshold16(bad)
+        with pytest.raises(ValueError):
+            _ffi.dropout_threshold(bad)
+    assert abs(OD.effective_rate(0.1) - 0.1) < 2 ** -16
+
+
+def test_decision_bits_statistics():
+    def corr(a, b):
+        return abs(np.corrcoef(a.ravel(), b.ravel())[0, 1])
+
+    n = 512
+    noise = 5.0 / n  # five standard deviations of a sample correlation over n * n pairs
+    for seed, bh in ((0, 0), (1, 5), (987654321987, 63)):
+        u = OD.random16(seed, bh, n, n) / 65536.0
+        assert abs(u.mean() - 0.5) < 0.003
+        hist = np.bincount((u * 16).astype(int).ravel(), minlength=16) / u.size
+        assert np.abs(hist - 1 / 16).max() < 0.002
+        for a, b in ((u[:, :-1], u[:, 1:]), (u[:, :-2], u[:, 2:]), (u[:, :-4], u[:, 4:]), (u[:-1], u[1:]), (u[:-2], u[2:]),
+                     (u[:-4], u[4:]), (u[:-1, :-1], u[1:, 1:]), (u[:-1, 1:], u[1:, :-1]), (u[:-1, :-2], u[1:, 2:])):
+            assert corr(a, b) < noise
+        assert corr(u, OD.random16(seed, bh + 1, n, n) / 65536.0) < noise
+        assert corr(u, OD.random16(seed + 1, bh, n, n) / 65536.0) < noise
+        for p in (0.1, 0.5):
+            keep = u >= OD.effective_rate(p)
+            assert abs(keep.mean() - (1 - p)) < 0.003
+            sd = np.sqrt(p * (1 - p) / n)  # of a row's or column's keep rate
+            assert 0.8 * sd < keep.mean(1).std() < 1.2 * sd and 0.8 * sd < keep.mean(0).std() < 1.2 * sd
+
+
+# ---- the semantics ---------------------------------------------------------------------------------------------------------
+
+def _rand(B, Hq, Hkv, L, S, E, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=dtype)  # noqa: E731
+    return mk(B, Hq, L, E), mk(B, Hkv, S, E), mk(B, Hkv, S, E)
+
+
+def test_oracle_dropout_semantics_against_library_routines():
+    q, k, v = _rand(2, 4, 2, 7, 9, 8)
+    ones = torch.ones(2, 4, 7, 9, dtype=torch.bool)
+    # nothing dropped: plain attention (p only sets the scale, 1 here)
+    ref = F.scaled_dot_product_attention(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1))
+    assert torch.allclose(OD.attention_dropout(q, k, v, ones, 0.0), ref, atol=1e-6)
+    causal = torch.tril(torch.ones(7, 9, dtype=torch.bool))
+    ref = F.scaled_dot_product_attention(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), attn_mask=causal)
+    assert torch.allclose(OD.attention_dropout(q, k, v, ones, 0.0, attend=causal), ref, atol=1e-6)
+    # everything dropped: zeros; kept weights carry the factor torch's own dropout uses
+    assert OD.attention_dropout(q, k, v, ~ones, 0.25).abs().max() == 0
+    kept_value = F.dropout(torch.ones(1000), 0.25, training=True).max().item()
+    assert abs(kept_value - 1 / (1 - OD.effective_rate(0.25))) < 1e-6
+    # one key kept per row: that key's value times weight / (1 - p)
+    keep = torch.zeros(2, 4, 7, 9, dtype=torch.bool)
+    keep[..., 3] = True
+    w = torch.softmax(q @ k.repeat_interleave(2, 1).transpose(-1, -2) / 8 ** 0.5, -1)[..., 3:4]
+    want = w * v.repeat_interleave(2, 1)[:, :, 3:4, :] / (1 - OD.effective_rate(0.25))
+    assert torch.allclose(OD.attention_dropout(q, k, v, keep, 0.25), want, atol=1e-6)
+    # unbiased: the mean over seeds approaches the undropped result
+    ref = OD.attention_dropout(q, k, v, ones, 0.0)
+    acc = torch.zeros_like(ref)
+    n = 400
+    for seed in range(n):
+        acc += OD.attention_dropout(q, k, v, OD.keep_mask(seed, 2, 4, 7, 9, 0.3), 0.3)
+    assert (acc / n - ref).abs().max() < 0.15 and (acc / n - ref).abs().mean() < 0.03
+
+
+def test_oracle_dropout_gradients_against_finite_differences():
+    q, k, v = (t.requires_grad_(True) for t in _rand(1, 2, 1, 5, 6, 4, dtype=torch.float64))
+    keep = OD.keep_mask(5, 1, 2, 5, 6, 0.4)
+    causal = torch.tril(torch.ones(5, 6, dtype=torch.bool))
+    assert 0.2 < keep.float().mean() < 0.9
+    assert torch.autograd.gradcheck(lambda a, b, c: OD.attention_dropout(a, b, c, keep, 0.4, attend=causal), (q, k, v),
+                                    eps=1e-6, atol=1e-5, rtol=1e-4)
+
+
+# ---- the boundary ----------------------------------------------------------------------------------------------------------
+
+def test_abi_validation_of_dropout_fields():
+    lib = _ffi.load_library()
+    rc = lambda p: lib.fl_attn_validate(C.byref(p))  # noqa: E731
+    for D in (64, 128):
+        p = good_params(D=D)
+        p.dropout_threshold = 6554
+        p.dropout_seed[0], p.dropout_seed[1] = 0xFFFFFFFF, 0x7FFFFFFF
+        p.mask_kind = _ffi.MASK_CAUSAL
+        assert rc(p) == 0, _ffi.last_error()
+    p = good_params()
+    p.dropout_threshold = 65536
+    assert rc(p) == -5 and "dropout_threshold" in _ffi.last_error()
+    for mutate in (lambda p: setattr(p, "alibi_heads", 4), lambda p: setattr(p, "softcap", 30.0),
+                   lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000)),
+                   lambda p: setattr(p, "diff", 1)):
+        p = good_params()
+        p.dropout_threshold = 100
+        mutate(p)
+        assert rc(p) == -4 and "dropout" in _ffi.last_error(), _ffi.last_error()
+    p = good_params(D=32)  # no dropout kernel at head dim 32
+    p.dropout_threshold = 100
+    assert rc(p) == -4, _ffi.last_error()
+    p = good_params()
+    p.reserved[0] = 1
+    assert rc(p) == -5 and "reserved" in _ffi.last_error()
+
+
+def test_front_end_switch_and_refusals():
+    q = torch.zeros(1, 2, 8, 64)
+    # default: dropout_p is ignored like the reference does, so a CPU call fails for the usual reason, not for dropout
+    with pytest.raises(Exception) as e:
+        A.attention_pytorch_causal(q, q, q, dropout_p=0.5)
+    assert "dropout" not in str(e.value)
+    with pytest.raises(NotImplementedError, match="dropout"):
+        ops.dispatch(q, q, q, dropout_p=0.1, gate=q)
+    with pytest.raises(ValueError, match="dropout_p"):
+        ops.dispatch(q, q, q, dropout_p=1.5)
+    with A.honor_dropout():
+        from flashlight_amd.attention_variants import _common
+        assert _common._honor_dropout
+    assert not _common._honor_dropout
+
+
+# ---- the kernels -----------------------------------------------------------------------------------------------------------
+
+def _gpu_inputs(B, Hq, Hkv, L, S, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)  # noqa: E731
+    return mk(B, Hq, L, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, L, D)
+
+
+def _attend(mask_kind, L, S, window=0, prefix=0):
+    qi = torch.arange(L)[:, None]
+    ki = torch.arange(S)[None, :]
+    if mask_kind == _ffi.MASK_CAUSAL:
+        return ki <= qi
+    if mask_kind == _ffi.MASK_SLIDING:
+        return (ki <= qi) & (qi - ki <= window)
+    if mask_kind == _ffi.MASK_PREFIX_LM:
+        return (ki < prefix) | (ki <= qi)
+    return None
+
+
+CASES = [
+    # B, Hq, Hkv, L, S, D, mask, window, prefix, p
+    (2, 4, 2, 200, 200, 64, _ffi.MASK_NONE, 0, 0, 0.1),
+    (1, 4, 1, 257, 257, 128, _ffi.MASK_CAUSAL, 0, 0, 0.25),
+    (2, 2, 2, 130, 300, 128, _ffi.MASK_NONE, 0, 0, 0.5),
+    (1, 2, 1, 300, 130, 64, _ffi.MASK_CAUSAL, 0, 0, 0.1),
+    (1, 2, 2, 400, 400, 64, _ffi.MASK_SLIDING, 50, 0, 0.2),
+    (1, 2, 2, 333, 333, 128, _ffi.MASK_PREFIX_LM, 0, 70, 0.3),
+    (1, 1, 1, 1, 1, 64, _ffi.MASK_NONE, 0, 0, 0.1),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(map(str, c)))
+def test_forward_and_gradients_with_dropout_match_the_oracle(case):
+    B, Hq, Hkv, L, S, D, mask_kind, window, prefix, p = case
+    seed = 0x1234567 * (L + 1) + (S << 40)
+    q, k, v, dout = _gpu_inputs(B, Hq, Hkv, L, S, D, seed=L + D)
+    kw = dict(mask_kind=mask_kind, window=window, prefix=prefix, dropout_p=p, dropout_seed=seed)
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, **kw)
+    torch.cuda.synchronize()
+
+    keep = OD.keep_mask(seed, B, Hq, L, S, p)
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    ref = OD.attention_dropout(qf, kf, vf, keep, p, attend=_attend(mask_kind, L, S, window, prefix))
+    ref.backward(dout.float().cpu())
+    assert_parity(out, ref, "forward with dropout")
+    for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{what} with dropout")
+    # the row statistics do not see the dropout
+    lse0 = torch.empty_like(lse)
+    _ffi.attn_fwd(q, k, v, lse=lse0, mask_kind=mask_kind, window=window, prefix=prefix)
+    assert torch.allclose(lse, lse0, atol=2e-2, rtol=0)  # sums of bf16-rounded weights over different tile sizes
+
+
+@pytest.mark.gpu
+def test_dropout_fp16_forward_and_determinism():
+    q, k, v, _ = _gpu_inputs(1, 2, 2, 192, 192, 128, seed=3)
+    q, k, v = (t.to(torch.float16) for t in (q, k, v))
+    a = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.2, dropout_seed=77)
+    b = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.2, dropout_seed=77)
+    c = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.2, dropout_seed=78)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    keep = OD.keep_mask(77, 1, 2, 192, 192, 0.2)
+    ref = OD.attention_dropout(q.float().cpu(), k.float().cpu(), v.float().cpu(), keep, 0.2,
+                               attend=_attend(_ffi.MASK_CAUSAL, 192, 192))
+    assert_parity(a, ref, "fp16 forward with dropout")
+
+
+@pytest.mark.gpu
+def test_dropout_through_autograd_and_the_variant_switch():
+    q, k, v, dout = _gpu_inputs(1, 4, 2, 160, 160, 64, seed=9)
+    # default: the variant ignores dropout_p, as the reference does
+    base = A.attention_pytorch_causal(q, k, v, enable_gqa=True)
+    assert torch.equal(A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True), base)
+    with A.honor_dropout():
+        torch.manual_seed(11)
+        a = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
+        torch.manual_seed(11)
+        b = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
+        c = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
+        assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a, base)
+        with pytest.raises(_ffi.FlashlightError, match="dropout"):
+            A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(30.0), dropout_p=0.1, enable_gqa=True)
+    # autograd: the backward regenerates the forward's decisions from the seed
+    qg, kg, vg = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    out = ops.dispatch(qg, kg, vg, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.3, dropout_seed=2024)
+    out.backward(dout)
+    keep = OD.keep_mask(2024, 1, 4, 160, 160, 0.3)
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    ref = OD.attention_dropout(qf, kf, vf, keep, 0.3, attend=_attend(_ffi.MASK_CAUSAL, 160, 160))
+    ref.backward(dout.float().cpu())
+    assert_parity(out, ref, "autograd forward with dropout")
+    for what, got, want in (("dq", qg.grad, qf.grad), ("dk", kg.grad, kf.grad), ("dv", vg.grad, vf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"autograd {what} with dropout")
+
+
+@pytest.mark.gpu
+def test_dropout_rate_at_benchmark_size_through_a_ones_value():
+    # with V = 1 every output element is (sum of kept weights) / (1 - p): its mean over rows is 1, its spread that of the
+    # kept weight mass; keys attended uniformly (q = 0) make the weights 1 / S, so out = kept fraction / (1 - p)
+    B, H, S, D = 1, 4, 4096, 128
+    q = torch.zeros(B, H, S, D, dtype=torch.bfloat16, device=DEV)
+    k = torch.randn(B, H, S, D, device=DEV).to(torch.bfloat16)
+    v = torch.ones(B, H, S, D, dtype=torch.bfloat16, device=DEV)
+    for p in (0.1, 0.5):
+        out = _ffi.attn_fwd(q, k, v, dropout_p=p, dropout_seed=31337).float()
+        assert (out[..., 0:1] - out).abs().max() < 1e-2           # every column of a row sees the same decisions
+        frac = out[..., 0] * (1 - OD.effective_rate(p))             # kept fraction per row
+        assert abs(frac.mean().item() - (1 - p)) < 2e-3
+        sd = (p * (1 - p) / S) ** 0.5
+        assert 0.7 * sd < frac.std().item() < 1.4 * sd + 2e-3       # binomial spread (plus bf16 rounding of the weights)

@@ -103,6 +103,23 @@ def registry() -> Dict[str, Callable]:
     }
 
 
+def dropout_registry(dropout_p: float) -> Dict[str, Callable]:
+    """The variants that have a dropout kernel (positional masks), with `--dropout_p` applied.  The reference records
+    the flag in its CSV and never applies it (benchmarks/_utils.py:231-233); its own variants are timed with
+    `--dropout_p 0`.  One fixed seed: the decisions cost the same whatever it is."""
+    from flashlight_amd import _ffi, ops
+
+    def variant(**kw):
+        return lambda q, k, v, enable_gqa=False: ops.dispatch(q, k, v, dropout_p=dropout_p, dropout_seed=1, **kw)
+
+    return {
+        "full": variant(),
+        "full_with_causal": variant(mask_kind=_ffi.MASK_CAUSAL),
+        "full_with_sliding_window": variant(mask_kind=_ffi.MASK_SLIDING, window=256),
+        "full_with_prefix_lm": variant(mask_kind=_ffi.MASK_PREFIX_LM, prefix=256),
+    }
+
+
 def make_qkv(batch: int, seqlen: int, nheads: int, headdim: int, group_size: int):
     """benchmarks/_utils.py:226-247: bf16 N(0,1); without GQA the three tensors are unbound from one packed
     [B, S, 3, H, D] draw and made contiguous in [B, H, S, D] order."""
@@ -183,7 +200,7 @@ def main(argv=None) -> List[tuple]:
         rows = _run_backward_suite(args) if args.suite == "backward" else _run_other_suite(args)
         write_results_csv(rows, f"{args.output}.csv")
         return rows
-    variants = registry()
+    variants = registry() if args.dropout_p == 0.0 else dropout_registry(args.dropout_p)
     for group_size in args.group_size:
         for headdim in args.headdim:
             for batch, seqlen in zip(args.batch_size, args.seqlen):
@@ -230,6 +247,9 @@ def _run_backward_suite(args) -> List[tuple]:
                     "full_with_document_mask": dict(mask_kind=_ffi.MASK_DOCUMENT,
                                                     doc_ids=create_document_id(batch, seqlen, num_docs=12)),
                 }
+                if args.dropout_p > 0.0:  # the positional-mask cases have a dropout kernel
+                    cases = {n: dict(kw, dropout_p=args.dropout_p, dropout_seed=1) for n, kw in cases.items()
+                             if not ({"alibi_heads", "softcap", "doc_ids"} & set(kw))}
                 for name, kw in cases.items():
                     if args.filter and all(key not in name for key in args.filter):
                         continue

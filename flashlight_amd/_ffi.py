@@ -354,7 +354,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream."""
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
-        _require_gpu_bf16(name, t)
+        _require_gpu_half(name, t, q if isinstance(q, torch.Tensor) and q.dtype in _HALF_TYPES else None)
         if t.dim() != 4:
             raise ValueError(f"{name} must be 4-D [batch, heads, seq, dim], got shape {tuple(t.shape)}")
     q, k, v, out, dout = (_dim_contiguous(t) for t in (q, k, v, out, dout))

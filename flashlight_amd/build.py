@@ -114,11 +114,12 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
     # backward kernels: one unit per (head dim, feature bits) of FL_BWD_LIST in bwd_instances.h
     bwd_list = re.search(r"#define FL_BWD_LIST\(X\)(.*)", (CSRC / "bwd_instances.h").read_text()).group(1)
     for d, feat in re.findall(r"X\((\d+),\s*(\d+)\)", bwd_list):
-        o = objdir / f"bwd_{d}_{feat}.o"
-        objs.append(o)
-        if not o.exists():
-            tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_BWD_D={d}", f"-DFL_BWD_FEAT={feat}", "-c", str(CSRC / "bwd_unit.hip"),
-                           "-o", str(o)], o))
+        for f16 in (0, 1):
+            o = objdir / f"bwd_{d}_{feat}{'_f16' if f16 else ''}.o"
+            objs.append(o)
+            if not o.exists():
+                tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_BWD_D={d}", f"-DFL_BWD_FEAT={feat}", f"-DFL_INST_F16={f16}", "-c",
+                               str(CSRC / "bwd_unit.hip"), "-o", str(o)], o))
     # the instance tables are host data only: compiling them for the device would reference the host launchers
     for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("bwd_table.hip", ["--cuda-host-only"]),
                        ("api.hip", []), ("probe.hip", [])):

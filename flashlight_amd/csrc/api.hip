@@ -366,7 +366,6 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
     return fail(FL_ERR_UNSUPPORTED, "backward: bias operands, gate, differential attention and the dump hook are not supported");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
-  if (p->dtype != FL_BF16) return fail(FL_ERR_UNSUPPORTED, "backward: bf16 only");
   if ((rc = check_ptr("dout", b->dout, 16)) || (rc = check_ptr("dq", b->dq, 8)) || (rc = check_ptr("dk", b->dk, 8)) ||
       (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 16)) ||
       (rc = check_ptr("fwd.lse", p->lse, 16)))
@@ -393,7 +392,8 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (p->dropout_threshold) want = fl::F_DROPOUT;  // validate() has excluded every other feature
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
-    if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want) in = &fl::kBwdInstances[i];
+    if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)
+      in = &fl::kBwdInstances[i];
   if (!in) return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d (64 and 128 are compiled)", p->Dqk);
   if (out) *out = in;
   g_err[0] = 0;

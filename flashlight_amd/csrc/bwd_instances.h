@@ -10,6 +10,7 @@ namespace fl {
 struct BwdInstance {
   int d;
   uint32_t feat;
+  int dtype;  // element type of q, k, v, o, dout and the gradients: FL_BF16 (0) or FL_F16 (2)
   hipError_t (*launch_dq)(const BParams&, hipStream_t);
   hipError_t (*launch_dkv)(const BParams&, hipStream_t);
   hipError_t (*launch_delta)(const BParams&, hipStream_t);
@@ -29,11 +30,11 @@ hipError_t launch_bwd(const BParams& bp, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int DV>
+template <int DV, class E>
 hipError_t launch_delta(const BParams& bp, hipStream_t stream) {
   const int64_t rows = (int64_t)bp.B * bp.Hq * bp.Lq;
   const int rows_per_block = 256 / (DV / 8);
-  hipLaunchKernelGGL(bwd_delta_kernel<DV>, dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
+  hipLaunchKernelGGL((bwd_delta_kernel<DV, E>), dim3((unsigned)((rows + rows_per_block - 1) / rows_per_block)), dim3(256), 0,
                      stream, bp);
   return hipGetLastError();
 }
@@ -44,20 +45,24 @@ hipError_t launch_delta(const BParams& bp, hipStream_t stream) {
 // 8 = document ids in the element predicate, 128 = dropout.
 #define FL_BWD_LIST(X) X(64, 0) X(64, 3) X(64, 8) X(64, 128) X(128, 0) X(128, 3) X(128, 8) X(128, 128)
 
-#define FL_BWD_DECL(D, FEAT)                                           \
-  namespace fl {                                                       \
-  hipError_t launch_bwd_dq_##D##_##FEAT(const BParams&, hipStream_t);  \
-  hipError_t launch_bwd_dkv_##D##_##FEAT(const BParams&, hipStream_t); \
-  hipError_t launch_bwd_delta_##D##_##FEAT(const BParams&, hipStream_t); \
+// Every (D, FEAT) pair is compiled for bf16 and for fp16 elements (suffix _bf16 / _f16).
+#define FL_BWD_DECL_(D, FEAT, SFX)                                            \
+  namespace fl {                                                              \
+  hipError_t launch_bwd_dq_##D##_##FEAT##SFX(const BParams&, hipStream_t);    \
+  hipError_t launch_bwd_dkv_##D##_##FEAT##SFX(const BParams&, hipStream_t);   \
+  hipError_t launch_bwd_delta_##D##_##FEAT##SFX(const BParams&, hipStream_t); \
   }
-#define FL_BWD_DEF(D, FEAT)                                                                                  \
-  namespace fl {                                                                                             \
-  hipError_t launch_bwd_dq_##D##_##FEAT(const BParams& bp, hipStream_t s) {                                  \
-    return launch_bwd<BwdTraits<D, ROLE_DQ, FEAT>>(bp, s);                                                   \
-  }                                                                                                          \
-  hipError_t launch_bwd_dkv_##D##_##FEAT(const BParams& bp, hipStream_t s) {                                 \
-    return launch_bwd<BwdTraits<D, ROLE_DKV, FEAT>>(bp, s);                                                  \
-  }                                                                                                          \
-  hipError_t launch_bwd_delta_##D##_##FEAT(const BParams& bp, hipStream_t s) { return launch_delta<D>(bp, s); } \
+#define FL_BWD_DECL(D, FEAT) FL_BWD_DECL_(D, FEAT, _bf16) FL_BWD_DECL_(D, FEAT, _f16)
+#define FL_BWD_DEF(D, FEAT, SFX, ELEM)                                                                              \
+  namespace fl {                                                                                                    \
+  hipError_t launch_bwd_dq_##D##_##FEAT##SFX(const BParams& bp, hipStream_t s) {                                    \
+    return launch_bwd<BwdTraits<D, ROLE_DQ, FEAT, ELEM>>(bp, s);                                                    \
+  }                                                                                                                 \
+  hipError_t launch_bwd_dkv_##D##_##FEAT##SFX(const BParams& bp, hipStream_t s) {                                   \
+    return launch_bwd<BwdTraits<D, ROLE_DKV, FEAT, ELEM>>(bp, s);                                                   \
+  }                                                                                                                 \
+  hipError_t launch_bwd_delta_##D##_##FEAT##SFX(const BParams& bp, hipStream_t s) { return launch_delta<D, ELEM>(bp, s); } \
   }
-#define FL_BWD_ROW(D, FEAT) {D, FEAT, &fl::launch_bwd_dq_##D##_##FEAT, &fl::launch_bwd_dkv_##D##_##FEAT, &fl::launch_bwd_delta_##D##_##FEAT},
+#define FL_BWD_ROW_(D, FEAT, SFX, DT) \
+  {D, FEAT, DT, &fl::launch_bwd_dq_##D##_##FEAT##SFX, &fl::launch_bwd_dkv_##D##_##FEAT##SFX, &fl::launch_bwd_delta_##D##_##FEAT##SFX},
+#define FL_BWD_ROW(D, FEAT) FL_BWD_ROW_(D, FEAT, _bf16, 0) FL_BWD_ROW_(D, FEAT, _f16, 2)

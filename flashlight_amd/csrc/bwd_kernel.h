@@ -52,8 +52,9 @@ struct BParams {
 };
 
 // Delta[b, h, q] = sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
-template <int DV>
+template <int DV, class E>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
+  typedef E ex8 __attribute__((ext_vector_type(8)));
   constexpr int LPR = DV / 8;  // lanes per row, 16 bytes each
   const int64_t rows = (int64_t)p.B * p.Hq * p.Lq;
   const int64_t row = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
@@ -61,8 +62,8 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
   float s = 0.f;
   if (row < rows) {
     const int q = (int)(row % p.Lq), h = (int)((row / p.Lq) % p.Hq), b = (int)(row / ((int64_t)p.Lq * p.Hq));
-    const bf16x8 a = *reinterpret_cast<const bf16x8*>(p.dout + b * p.dos[0] + h * p.dos[1] + q * p.dos[2] + 8 * c);
-    const bf16x8 o = *reinterpret_cast<const bf16x8*>(p.o + b * p.os[0] + h * p.os[1] + q * p.os[2] + 8 * c);
+    const ex8 a = *reinterpret_cast<const ex8*>(p.dout + b * p.dos[0] + h * p.dos[1] + q * p.dos[2] + 8 * c);
+    const ex8 o = *reinterpret_cast<const ex8*>(p.o + b * p.os[0] + h * p.os[1] + q * p.os[2] + 8 * c);
 #pragma unroll
     for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)o[e];
   }
@@ -71,8 +72,9 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
   if (row < rows && c == 0) p.delta[row] = s;
 }
 
-template <int D_, int ROLE_, uint32_t FEAT_>
+template <int D_, int ROLE_, uint32_t FEAT_, class Elem_ = bf16_t>
 struct BwdTraits {
+  using Elem = Elem_;  // element type of q, k, v, o, dout and the gradients: bf16_t or f16_t
   static constexpr int D = D_, ROLE = ROLE_;
   static constexpr uint32_t FEAT = FEAT_;
   static constexpr int OWN = 128;                          // owner positions per workgroup: 4 waves x 32
@@ -106,6 +108,9 @@ void bwd_kernel(const BParams p) {
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC;
   constexpr bool kDQ = ROLE == ROLE_DQ;
+  using E = typename T::Elem;  // pointers in BParams are typed bf16_t whatever E is: 16 opaque bits
+  typedef E ex8 __attribute__((ext_vector_type(8)));
+  typedef E ex4 __attribute__((ext_vector_type(4)));
   constexpr bool kDrop = FEAT & F_DROPOUT;
   constexpr float kLog2e = 1.4426950408889634f;
   using L = TileLayout<D>;
@@ -182,7 +187,7 @@ void bwd_kernel(const BParams p) {
   // ---- owner operands ---------------------------------------------------------------------------------------------------
   // ROLE_DQ: Q and dO fragments of this lane's query row live in registers (B operands), with its LSE and Delta.
   // ROLE_DKV: the workgroup's K and V rows are staged in LDS once and read as B operands where they are used.
-  bf16x8 o1f[kDQ ? KS : 1], o2f[kDQ ? KS : 1];
+  ex8 o1f[kDQ ? KS : 1], o2f[kDQ ? KS : 1];
   float lse_o = 0.f, delta_o = 0.f;
   const bf16_t* kptr = p.k + (int64_t)batch * p.ks[0] + (int64_t)kvh * p.ks[1];
   const bf16_t* vptr = p.v + (int64_t)batch * p.vs[0] + (int64_t)kvh * p.vs[1];
@@ -192,8 +197,8 @@ void bwd_kernel(const BParams p) {
     const bf16_t* dp = p.dout + (int64_t)batch * p.dos[0] + (int64_t)ohead * p.dos[1] + (int64_t)qr * p.dos[2];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      o1f[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16 + 8 * h);
-      o2f[ks] = *reinterpret_cast<const bf16x8*>(dp + ks * 16 + 8 * h);
+      o1f[ks] = *reinterpret_cast<const ex8*>(qp + ks * 16 + 8 * h);
+      o2f[ks] = *reinterpret_cast<const ex8*>(dp + ks * 16 + 8 * h);
     }
     const int64_t row = ((int64_t)batch * p.Hq + ohead) * p.Lq + qr;
     lse_o = p.lse[row];
@@ -244,13 +249,13 @@ void bwd_kernel(const BParams p) {
   // ---- LDS operand reads --------------------------------------------------------------------------------------------------
   // row-wise: 8 consecutive elements [row][16 ks + 8 h, +8) (A operand of X1/X2 from a streamed tile, or B operand from
   // an owner tile)
-  auto frag_row = [&](unsigned tile_off, int row, int ks) FL_INLINE -> bf16x8 {
-    return *reinterpret_cast<const bf16x8*>(smem + tile_off + row * (D * 2) + L::swz_kv(row, 2 * ks + h) * 16);
+  auto frag_row = [&](unsigned tile_off, int row, int ks) FL_INLINE -> ex8 {
+    return *reinterpret_cast<const ex8*>(smem + tile_off + row * (D * 2) + L::swz_kv(row, 2 * ks + h) * 16);
   };
   // transposing: A operand of the accumulating products for 16-position chunk c and column block db; slot j of lane
   // (r, h) is streamed position 16 c + 8 (j / 4) + 4 h + j % 4, the order in which the weights are packed
-  auto frag_tr = [&](unsigned tile_off, int c, int db) FL_INLINE -> bf16x8 {
-    bf16x8 f;
+  auto frag_tr = [&](unsigned tile_off, int c, int db) FL_INLINE -> ex8 {
+    ex8 f;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int i16 = lane % 16, g = (lane / 16) % 2;
@@ -259,7 +264,7 @@ void bwd_kernel(const BParams p) {
       const unsigned char* ap = smem + tile_off + row * (D * 2) + L::swz_kv(row, col / 8) * 16 + (col % 8) * 2;
       typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
       const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
-      const bf16x4 b4 = __builtin_bit_cast(bf16x4, t4);
+      const ex4 b4 = __builtin_bit_cast(ex4, t4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) f[4 * j + e] = b4[e];
     }
@@ -332,7 +337,7 @@ void bwd_kernel(const BParams p) {
         for (int e = 0; e < 4; ++e) out[e] = base[srow0 + min(q4 + e, p.Lq - 1)];  // clamped rows are masked
         return out;
       };
-      bf16x8 pf[2 * TB], dsf[2 * TB];
+      ex8 pf[2 * TB], dsf[2 * TB];
       float pd[TB][16];  // weight times d(score) / d(qk * scale); with dropout its sign bit marks a dropped weight
       // dropout: the owner position's share of the hash argument (see drop_pair_hash); the streamed head changes from step
       // to step in ROLE_DKV
@@ -349,11 +354,11 @@ void bwd_kernel(const BParams p) {
           for (int i = 0; i < 16; ++i) x1[sb][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          bf16x8 b1;
+          ex8 b1;
           if constexpr (kDQ) b1 = o1f[ks]; else b1 = frag_row(T::O1_OFF, ow * 32 + r, ks);
 #pragma unroll
           for (int sb = 0; sb < TB; ++sb)
-            x1[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t1, (qh * TB + sb) * 32 + r, ks), b1, x1[sb], 0, 0, 0);
+            x1[sb] = mfma32(frag_row(t1, (qh * TB + sb) * 32 + r, ks), b1, x1[sb]);
         }
 #pragma unroll
         for (int sb = 0; sb < TB; ++sb) {
@@ -431,7 +436,7 @@ void bwd_kernel(const BParams p) {
 #pragma unroll
           for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pf[2 * sb + j][e] = (bf16_t)pv[8 * j + e];
+            for (int e = 0; e < 8; ++e) pf[2 * sb + j][e] = (E)pv[8 * j + e];
         }
       }
       {
@@ -442,11 +447,11 @@ void bwd_kernel(const BParams p) {
           for (int i = 0; i < 16; ++i) x2[sb][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          bf16x8 b2;
+          ex8 b2;
           if constexpr (kDQ) b2 = o2f[ks]; else b2 = frag_row(T::O2_OFF, ow * 32 + r, ks);
 #pragma unroll
           for (int sb = 0; sb < TB; ++sb)
-            x2[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_row(t2, (qh * TB + sb) * 32 + r, ks), b2, x2[sb], 0, 0, 0);
+            x2[sb] = mfma32(frag_row(t2, (qh * TB + sb) * 32 + r, ks), b2, x2[sb]);
         }
 #pragma unroll
         for (int sb = 0; sb < TB; ++sb) {
@@ -466,7 +471,7 @@ void bwd_kernel(const BParams p) {
               } else {
                 ds = pd[sb][i] * (x2[sb][i] - (kDQ ? delta_o : dl4[e]));
               }
-              dsf[2 * sb + i / 8][i % 8] = (bf16_t)ds;
+              dsf[2 * sb + i / 8][i % 8] = (E)ds;
             }
           }
         }
@@ -476,9 +481,9 @@ void bwd_kernel(const BParams p) {
       for (int c = 0; c < 2 * TB; ++c)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          acc1[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t1, 2 * TB * qh + c, db), dsf[c], acc1[db], 0, 0, 0);
+          acc1[db] = mfma32(frag_tr(t1, 2 * TB * qh + c, db), dsf[c], acc1[db]);
           if constexpr (!kDQ)
-            acc2[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(t2, 2 * TB * qh + c, db), pf[c], acc2[db], 0, 0, 0);
+            acc2[db] = mfma32(frag_tr(t2, 2 * TB * qh + c, db), pf[c], acc2[db]);
         }
     }
     dma_wait<0>();
@@ -518,10 +523,10 @@ void bwd_kernel(const BParams p) {
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        bf16x4 o4;
+        ex4 o4;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)(acc1[db][4 * g + e] * p.scale);
-        *reinterpret_cast<bf16x4*>(out1 + 32 * db + 8 * g + 4 * h) = o4;
+        for (int e = 0; e < 4; ++e) o4[e] = (E)(acc1[db][4 * g + e] * p.scale);
+        *reinterpret_cast<ex4*>(out1 + 32 * db + 8 * g + 4 * h) = o4;
       }
     if constexpr (!kDQ) {
       bf16_t* out2 = p.dv + (int64_t)batch * p.dvs[0] + (int64_t)ohead * p.dvs[1] + (int64_t)opos * p.dvs[2];
@@ -529,10 +534,10 @@ void bwd_kernel(const BParams p) {
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          bf16x4 o4;
+          ex4 o4;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)(kDrop ? acc2[db][4 * g + e] * p.drop_rescale : acc2[db][4 * g + e]);
-          *reinterpret_cast<bf16x4*>(out2 + 32 * db + 8 * g + 4 * h) = o4;
+          for (int e = 0; e < 4; ++e) o4[e] = (E)(kDrop ? acc2[db][4 * g + e] * p.drop_rescale : acc2[db][4 * g + e]);
+          *reinterpret_cast<ex4*>(out2 + 32 * db + 8 * g + 4 * h) = o4;
         }
     }
   }

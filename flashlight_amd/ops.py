@@ -105,7 +105,7 @@ def _setup_context(ctx, inputs, output):
 def _backward(ctx, dout, dlse):
     q, k, v, out, lse = ctx.saved_tensors
     scale, mask_kind, window, prefix, alibi_heads, softcap, dropout_p, dropout_seed = ctx.args
-    dq, dk, dv = attn_bwd(q, k, v, out, lse, dout.to(torch.bfloat16), scale, mask_kind, window, prefix, ctx.doc_ids,
+    dq, dk, dv = attn_bwd(q, k, v, out, lse, dout.to(q.dtype), scale, mask_kind, window, prefix, ctx.doc_ids,
                           alibi_heads, softcap, dropout_p, dropout_seed)
     return dq, dk, dv, None, None, None, None, None, None, None, None, None
 
@@ -136,9 +136,6 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         dropout_seed = 0
     if (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) or \
             (dropout_p > 0.0 and torch.compiler.is_compiling()):
-        if q.dtype != torch.bfloat16:
-            raise NotImplementedError("the backward kernels take bfloat16 only: call under torch.no_grad() for a forward "
-                                      f"in {q.dtype}")
         if biases or gate is not None or diff or seq_major_out:
             raise NotImplementedError(
                 "no backward is implemented for bias operands, the sigmoid gate or differential attention: call under "

@@ -98,7 +98,7 @@ typedef struct fl_attn_params {
   float lambda;
 
   int32_t dtype; /* element type of q, k, v, o and gate: FL_BF16 or FL_F16 (the reference's typing admits both,
-                  * monkeypatch/fusion/_reduction.py:55-57); the backward takes FL_BF16 only */
+                  * monkeypatch/fusion/_reduction.py:55-57) */
 
   /* Scratch for the document-mask tile table; size from fl_workspace_bytes(); may be NULL otherwise. */
   void* workspace;
@@ -158,7 +158,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * kind, grouped-query heads, ALiBi, the tanh soft-cap; Dqk == Dv in {64, 128}.  Not supported (FL_ERR_UNSUPPORTED):
  * bias operands, gate, differential attention, the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
- * receive the gradients (bf16, strides in elements, last stride 1, others multiples of 8).
+ * receive the gradients (element type fwd.dtype like dout; strides in elements, last stride 1, others multiples of 8).
  * delta: caller-provided scratch of B * Hq * Lq floats; delta and fwd.lse must be 16-byte aligned.
  * fwd.workspace as for the forward (document masks). */
 typedef struct fl_attn_bwd_params {

@@ -156,6 +156,25 @@ def test_gradients_match_the_oracle(name, D):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name", ["vanilla", "causal", "alibi+softcap+causal"])
+def test_gradients_fp16(name, D):
+    """fp16 elements: same kernels compiled for the other MFMA / conversion instructions; fp16 keeps three more
+    mantissa bits than bf16, so the bf16 tolerance holds with room."""
+    hip_fn, oracle_fn = VARIANTS[name]
+    q, k, v, dout = (t.to(torch.float16) for t in _inputs(2, 4, 2, 200, D, seed=sum(map(ord, name)) + D + 1))
+    out, dq, dk, dv = _grads(hip_fn, q, k, v, dout, torch.float16)
+    ref, rq, rk, rv = _grads(oracle_fn, q, k, v, dout, torch.float32)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    assert_parity(out.reshape(ref.shape), ref, f"{name} fp16: forward")
+    for what, got, want in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        assert got.dtype == torch.float16 and got.shape == want.shape
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{name} fp16: {what}")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("D", [64, 128])
 def test_gradients_document_mask(D, causal):

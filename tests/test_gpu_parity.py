@@ -453,14 +453,12 @@ def test_fp16_differential_evoformer_and_mixed_types():
     out = A.attention_reference(Q, K, V, [mask, pair.float()], gate=G)  # one fp16 operand, one fp32 operand
     assert out.dtype == torch.float16
     assert_parity(out, O.attention_evoformer(*f32(Q, K, V), [mask.float(), pair.float()], gate=G.float()), "fp16 evoformer")
-    # element types do not mix, and the backward is bf16 only
+    # element types do not mix
     qb, kb, vb = qkv(1, 2, 2, 64, 64, seed=53)
     with pytest.raises(NotImplementedError, match="mixed element types"):
         A.attention_pytorch(qb, kb.to(torch.float16), vb)
     with pytest.raises(NotImplementedError, match="mixed element types"):
         A.attention_reference(Q, K, V, [pair.bfloat16()])
-    with pytest.raises(NotImplementedError, match="bfloat16 only"):
-        A.attention_pytorch_causal(qb.to(torch.float16).requires_grad_(True), kb.to(torch.float16), vb.to(torch.float16))
 
 
 def test_fp16_large_weights_take_the_exact_path():

@@ -224,10 +224,9 @@ void bwd_kernel(const BParams p) {
       dma16(base, off, lds0 + it * NT * 16);
     }
   };
-  // ROLE_DKV: the statistics of the streamed rows ride the tile transfers when every row block starts on a 16-byte
-  // boundary (then a tile's valid rows are a multiple of 4 too); otherwise they are read from global memory in place
-  const bool stats_staged = !kDQ && p.Lq % 4 == 0;
-  // streamed step s -> (query head of the group, tile)
+  // streamed step s -> (query head of the group, tile).  ROLE_DKV: the statistics of the streamed rows (LSE, Delta) ride
+  // the tile transfers into LDS, 4 bytes per lane, so that the loop holds no ordinary global load: the wait such a load
+  // needs would also wait for the tile transfers that are in flight for the next step.
   auto step_head = [&](int s) FL_INLINE { return kDQ ? ohead : kvh * p.group + s / n_tiles; };
   auto step_tile = [&](int s) FL_INLINE { return t_lo + (kDQ ? s : s % n_tiles); };
   auto load_step = [&](int s, int slot) FL_INLINE {
@@ -241,14 +240,15 @@ void bwd_kernel(const BParams p) {
                 T::T1_OFF + slot * T::TBYTES, T::T_PER_T);
       load_tile(p.dout + (int64_t)batch * p.dos[0] + (int64_t)hd * p.dos[1] + (int64_t)t0 * p.dos[2], p.dos[2], valid,
                 T::T2_OFF + slot * T::TBYTES, T::T_PER_T);
-      if (stats_staged && wave == 0) {
-        // one wave brings both arrays (every wave waits for all of its own transfers before the barrier, so the
-        // counts need not match).  Lane l fetches rows 4 l .. 4 l + 3; lanes past the end of the sequence repeat its
-        // last four rows.
+      if (wave == 0) {
+        // one wave brings both arrays (every wave waits for all of its own transfers before the barrier, so the counts
+        // need not match).  Lane l fetches row t0 + l; lanes past the end of the tile or of the sequence repeat the last
+        // valid row (those rows are masked).
+        static_assert(BT <= 64, "one lane per streamed row");
         const int64_t row0 = ((int64_t)batch * p.Hq + hd) * p.Lq + t0;
-        const unsigned off = (unsigned)min(lane, valid / 4 - 1) * 16u;
-        dma16(uniform_ptr(p.lse + row0), off, (unsigned)(uintptr_t)smem + T::S1_OFF + slot * T::SBYTES);
-        dma16(uniform_ptr(p.delta + row0), off, (unsigned)(uintptr_t)smem + T::S2_OFF + slot * T::SBYTES);
+        const unsigned off = (unsigned)min(lane, valid - 1) * 4u;
+        dma4(uniform_ptr(p.lse + row0), off, (unsigned)(uintptr_t)smem + T::S1_OFF + slot * T::SBYTES);
+        dma4(uniform_ptr(p.delta + row0), off, (unsigned)(uintptr_t)smem + T::S2_OFF + slot * T::SBYTES);
       }
     }
   };
@@ -334,15 +334,9 @@ void bwd_kernel(const BParams p) {
       float slope_l2 = 0.f;
       if constexpr (kAlibi)
         slope_l2 = p.alibi_heads > 0 ? exp2f(-8.0f * (float)(shead + 1) / (float)p.alibi_heads) * kLog2e : 0.f;
-      const int64_t srow0 = ((int64_t)batch * p.Hq + shead) * p.Lq;  // ROLE_DKV: row statistics of the streamed head
-      // 4 consecutive streamed rows of a per-row fp32 array: one 16-byte load when aligned and inside the sequence
-      auto rows4 = [&](const float* base, unsigned staged_off, int q4) FL_INLINE -> f32x4 {
-        if (stats_staged)  // rows past the end hold copies of valid rows; they are masked
-          return *reinterpret_cast<const f32x4*>(smem + staged_off + slot * T::SBYTES + (q4 - t0) * 4);
-        f32x4 out;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = base[srow0 + min(q4 + e, p.Lq - 1)];  // clamped rows are masked
-        return out;
+      // 4 consecutive streamed rows of a staged per-row fp32 array
+      auto rows4 = [&](unsigned staged_off, int q4) FL_INLINE -> f32x4 {
+        return *reinterpret_cast<const f32x4*>(smem + staged_off + slot * T::SBYTES + (q4 - t0) * 4);
       };
       // X2 = T2 . O2^T (dP).  At D = 128 its fp32 tile is declared out here, next to X1's, and (ROLE_DQ) its MFMAs are issued
       // right after X1's, before the weights' vector work; at D = 64 it lives in the block that consumes it.  Both choices
@@ -408,7 +402,7 @@ void bwd_kernel(const BParams p) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             f32x4 lse4;
-            if constexpr (!kDQ) lse4 = rows4(p.lse, T::S1_OFF, sbase + 8 * g);
+            if constexpr (!kDQ) lse4 = rows4(T::S1_OFF, sbase + 8 * g);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * g + e, off = 8 * g + e;
@@ -491,7 +485,7 @@ void bwd_kernel(const BParams p) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             f32x4 dl4;
-            if constexpr (!kDQ) dl4 = rows4(p.delta, T::S2_OFF, sbase + 8 * g);
+            if constexpr (!kDQ) dl4 = rows4(T::S2_OFF, sbase + 8 * g);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * g + e;

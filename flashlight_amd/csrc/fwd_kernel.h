@@ -169,6 +169,14 @@ __device__ __forceinline__ void dma16(uint64_t gbase_uniform, unsigned voff, uns
                : "m0");
 }
 
+// The same with 4 bytes per lane (lane l writes LDS bytes [4 l, 4 l + 4)): for fp32 rows whose start is only 4-byte aligned.
+__device__ __forceinline__ void dma4(uint64_t gbase_uniform, unsigned voff, unsigned lds_base) {
+  const unsigned lds_base_uniform = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_base);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, %0" ::"s"(gbase_uniform), "v"(voff),
+               "s"(lds_base_uniform)
+               : "m0");
+}
+
 // Waits until at most N of this wave's vector-memory operations (the transfers above included) are outstanding;
 // they complete in issue order.  Leaves the LDS/scalar and export counters alone.
 template <int N>

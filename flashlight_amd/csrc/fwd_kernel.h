@@ -755,6 +755,30 @@ void fwd_kernel(const KParams p) {
             const int kbase = k0 + 32 * kb + 4 * h;
             const float rel0 = (float)(kbase - qrow[qb]);
             float bv[16];
+            // (called once on every path below, so that the path without global loads does not meet the other one
+            // before the scores are final: a wait for those loads after the join would run on every tile, and would
+            // also wait for the K/V transfers in flight)
+            auto combine = [&]() FL_INLINE {
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const float x = s[kb][qb][i];
+                float tl2;
+                if constexpr (kNatural) {
+                  tl2 = __builtin_fmaf(x, p.scale, bv[i]);  // natural units: one operation per score
+                } else {
+                  if constexpr (kSoftcap) {
+                    const float e = fast_exp2(x * cap_k1);
+                    const float rc = fast_rcp(e + 1.0f);
+                    tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
+                  } else {
+                    tl2 = x * p.scale_log2;
+                  }
+                  if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
+                  if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
+                }
+                s[kb][qb][i] = tl2;
+              }
+            };
             if constexpr (kBias) {
 #pragma unroll
               for (int i = 0; i < 16; ++i) bv[i] = 0.f;
@@ -818,26 +842,12 @@ void fwd_kernel(const KParams p) {
                     }
                   }
                 }
-              }
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float x = s[kb][qb][i];
-              float tl2;
-              if constexpr (kNatural) {
-                tl2 = __builtin_fmaf(x, p.scale, bv[i]);  // natural units: one operation per score
+                combine();
               } else {
-                if constexpr (kSoftcap) {
-                  const float e = fast_exp2(x * cap_k1);
-                  const float rc = fast_rcp(e + 1.0f);
-                  tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
-                } else {
-                  tl2 = x * p.scale_log2;
-                }
-                if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
-                if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
+                combine();
               }
-              s[kb][qb][i] = tl2;
+            } else {
+              combine();
             }
           }
       }
@@ -856,36 +866,45 @@ void fwd_kernel(const KParams p) {
         const int kbase = k0 + 32 * kb + 4 * h;
         const int t_len = p.Lk - kbase;   // off < t_len   <=> key < Lk
         const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
+        // the positional test, and one of three document tests: none; one id for the whole block; an id per key
+        auto mask_block = [&](auto doc_mode, int64_t block_doc, const int64_t (&kdoc)[16]) FL_INLINE {
+          constexpr int kMode = decltype(doc_mode)::value;
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            const int rel = kbase - qrow[qb];
+            // off <= hi <=> key < Lk && (key - q <= dmax || key < pfx);  off >= lo <=> key - q >= dmin
+            int hi = min(t_len - 1, max(p.dmax - rel, t_pfx - 1));
+            const int lo = p.dmin - rel;
+            if constexpr (kMode == 1) hi = (block_doc == qdoc[qb]) ? hi : -1;  // another document: nothing passes
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int off = 8 * (i / 4) + (i % 4);
+              bool ok = (off <= hi) & (off >= lo);
+              if constexpr (kMode == 2) ok = ok & (kdoc[i] == qdoc[qb]);
+              s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
+            }
+          }
+        };
         int64_t kdoc[16];
         if constexpr (kDoc) {
           // a 32-key block lies inside one document far more often than not, and the (min, max) table says so with two
-          // scalar loads: only blocks that hold a boundary read their keys' ids one by one
+          // scalar loads: only blocks that hold a boundary read their keys' ids one by one.  The two cases do not share
+          // the code that consumes the ids: a wait for those loads placed after the join would run in the common case
+          // too, and would also wait for the K/V transfers in flight.
           static_assert(kDocBlock == 32, "one table entry per 32-key block of a tile");
           // (a block that starts past the last key reads the last entry: all of its keys are masked anyway)
           const int64_t* tb = p.doc_table + ((int64_t)batch * p.doc_blocks + min((k0 + 32 * kb) / kDocBlock, p.doc_blocks - 1)) * 2;
           const int64_t bmn = tb[0], bmx = tb[1];
           if (bmn == bmx) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) kdoc[i] = bmn;
+            mask_block(std::integral_constant<int, 1>{}, bmn, kdoc);
           } else {
 #pragma unroll
             for (int i = 0; i < 16; ++i)
               kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
+            mask_block(std::integral_constant<int, 2>{}, 0, kdoc);
           }
-        }
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          const int rel = kbase - qrow[qb];
-          // off <= hi <=> key < Lk && (key - q <= dmax || key < pfx);  off >= lo <=> key - q >= dmin
-          const int hi = min(t_len - 1, max(p.dmax - rel, t_pfx - 1));
-          const int lo = p.dmin - rel;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int off = 8 * (i / 4) + (i % 4);
-            bool ok = (off <= hi) & (off >= lo);
-            if constexpr (kDoc) ok = ok & (kdoc[i] == qdoc[qb]);
-            s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
-          }
+        } else {
+          mask_block(std::integral_constant<int, 0>{}, 0, kdoc);
         }
       }
     };

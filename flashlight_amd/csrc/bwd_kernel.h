@@ -83,7 +83,7 @@ struct BwdTraits {
   // through LDS at the end (one workgroup per CU, 128 KB of LDS).
   static constexpr int QH = (ROLE == ROLE_DKV && D_ > 64) ? 2 : 1;   // waves per owner block
   static constexpr int NW = 4 * QH, NT = 64 * NW;
-  static constexpr int TB = (ROLE == ROLE_DQ && D_ <= 64) ? 2 : 1;  // 32-position blocks per wave and step (register budget)
+  static constexpr int TB = (D_ <= 64) ? 2 : 1;  // 32-position blocks per wave and step (register budget)
   static constexpr int BT = 32 * TB * QH;                  // streamed positions per step
   static constexpr int KS = D / 16, DB = D / 32;
   static constexpr int TBYTES = BT * D * 2;                // one streamed tile

@@ -296,37 +296,36 @@ void bwd_kernel(const BParams p) {
       load_tile(kptr + (int64_t)o0 * p.ks[2], p.ks[2], valid, T::O1_OFF, T::O_PER_T);
       load_tile(vptr + (int64_t)o0 * p.vs[2], p.vs[2], valid, T::O2_OFF, T::O_PER_T);
     }
-    load_step(0, 0);
-    dma_wait<0>();
   }
 
-  for (int s = 0; s < n_steps; ++s) {
-    const int slot = s & 1;
-    __syncthreads();  // publishes slot `slot` (every wave waited for its own transfers) and frees the other slot
-    if (s + 1 < n_steps) load_step(s + 1, slot ^ 1);
+  // Workgroup-level class of a step: nothing of its tile is attended by the workgroup's owner range (`skip`: document
+  // ranges apart; positional emptiness inside [t_lo, t_hi] only occurs for a prefix-LM mask), everything is (`full`),
+  // or every position of the tile and of the owner range carries one and the same document id (`doc_uniform`).
+  // Steps that are skipped are never transferred: the loop goes from one live step to the next (under a document mask
+  // most steps of the range are dead).
+  auto classify_step = [&](int s, bool& full, bool& doc_uniform) FL_INLINE -> bool {
+    const int t0 = step_tile(s) * BT;
+    const int s1 = min(t0 + BT, slen);
+    const int qa = kDQ ? o0 : t0, qb_ = kDQ ? o1 : s1, ka = kDQ ? t0 : o0, kb_ = kDQ ? s1 : o1;
+    const int cls = classify_positional(p.mask_kind, qa, qb_, ka, kb_, p.window, p.prefix);
+    bool skip = cls == TILE_EMPTY;
+    // every pair of the step attended: the positional mask holds everywhere and both ranges lie inside the sequences
+    full = cls == TILE_FULL && t0 + BT <= slen && o0 + T::OWN <= olen;
+    doc_uniform = false;
+    if constexpr (kDoc) {
+      int64_t mn, mx;
+      doc_range(p.doc_table + (int64_t)batch * p.doc_blocks * 2, t0, s1, mn, mx);
+      skip = skip || mx < own_mn || mn > own_mx;
+      doc_uniform = mn == mx && own_mn == own_mx && mn == own_mn;
+      full = full && doc_uniform;
+    }
+    return skip;
+  };
+  // One step: the tile in ring slot `slot` against the owner operands.
+  auto run_step = [&](int s, int slot, bool full, bool doc_uniform) FL_INLINE {
     const int t0 = step_tile(s) * BT;
     const int shead = step_head(s);  // the query head of this step
-
-    // workgroup-level skip: nothing of this tile is attended by the workgroup's owner range (document ranges apart;
-    // positional emptiness inside [t_lo, t_hi] only occurs for a prefix-LM mask)
-    bool skip = false, full = false;
-    bool doc_uniform = false;  // every position of the tile and of the owner range carries one and the same document id
     {
-      const int s1 = min(t0 + BT, slen);
-      const int qa = kDQ ? o0 : t0, qb_ = kDQ ? o1 : s1, ka = kDQ ? t0 : o0, kb_ = kDQ ? s1 : o1;
-      const int cls = classify_positional(p.mask_kind, qa, qb_, ka, kb_, p.window, p.prefix);
-      skip = cls == TILE_EMPTY;
-      // every pair of the step attended: the positional mask holds everywhere and both ranges lie inside the sequences
-      full = cls == TILE_FULL && t0 + BT <= slen && o0 + T::OWN <= olen;
-      if constexpr (kDoc) {
-        int64_t mn, mx;
-        doc_range(p.doc_table + (int64_t)batch * p.doc_blocks * 2, t0, s1, mn, mx);
-        skip = skip || mx < own_mn || mn > own_mx;
-        doc_uniform = mn == mx && own_mn == own_mx && mn == own_mn;
-        full = full && doc_uniform;
-      }
-    }
-    if (!skip) {
       const unsigned t1 = T::T1_OFF + slot * T::TBYTES, t2 = T::T2_OFF + slot * T::TBYTES;
       // ---- X1 = T1 . O1^T, then the weights; X2 = T2 . O2^T, then dS (one after the other: the two fp32 tiles are
       // never live together, which is what lets 128 accumulator registers fit) ----------------------------------------------
@@ -512,7 +511,40 @@ void bwd_kernel(const BParams p) {
             acc2[db] = mfma32(frag_tr(t2, 2 * TB * qh + c, db), pf[c], acc2[db]);
         }
     }
+  };
+  if constexpr (kDoc) {
+    // (the class of a step is worked out before its transfers are issued: the table reads must not wait on them)
+    auto next_live = [&](int s, bool& full, bool& doc_uniform) FL_INLINE -> int {
+      while (s < n_steps && classify_step(s, full, doc_uniform)) ++s;
+      return s;
+    };
+    bool full = false, doc_uniform = false;
+    int s = next_live(0, full, doc_uniform);
+    if (s < n_steps) load_step(s, 0);
     dma_wait<0>();
+    for (int slot = 0; s < n_steps; slot ^= 1) {
+      __syncthreads();  // publishes slot `slot` (every wave waited for its own transfers) and frees the other slot
+      bool full_next = false, doc_uniform_next = false;
+      const int s_next = next_live(s + 1, full_next, doc_uniform_next);
+      if (s_next < n_steps) load_step(s_next, slot ^ 1);
+      run_step(s, slot, full, doc_uniform);
+      dma_wait<0>();
+      s = s_next;
+      full = full_next;
+      doc_uniform = doc_uniform_next;
+    }
+  } else {
+    // positional masks: every step of [t_lo, t_hi] is visited (a dead one only occurs under a prefix-LM mask)
+    if (n_steps > 0) load_step(0, 0);
+    dma_wait<0>();
+    for (int s = 0; s < n_steps; ++s) {
+      const int slot = s & 1;
+      __syncthreads();  // publishes slot `slot` (every wave waited for its own transfers) and frees the other slot
+      if (s + 1 < n_steps) load_step(s + 1, slot ^ 1);
+      bool full, doc_uniform;
+      if (!classify_step(s, full, doc_uniform)) run_step(s, slot, full, doc_uniform);
+      dma_wait<0>();
+    }
   }
 
   // ---- the waves of one owner block add up their partial sums: the second wave parks its accumulators in LDS (element

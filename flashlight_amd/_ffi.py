@@ -90,7 +90,8 @@ _MAX_DV_DIFF = 128  # widest value slab of a differential-attention kernel insta
 
 
 def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
-    """Loads the in-tree shared library once.  Raises if it has not been built (no silent fallback)."""
+    """Loads the in-tree shared library once (or the library at `path`, which then serves every later call).  Raises if
+    it has not been built (no silent fallback)."""
     global _lib
     if _lib is not None and path is None:
         return _lib
@@ -127,8 +128,7 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     if lib.fl_bwd_params_sizeof() != C.sizeof(FlAttnBwdParams):
         raise RuntimeError(f"{p}: fl_attn_bwd_params is {lib.fl_bwd_params_sizeof()} bytes, binding expects "
                            f"{C.sizeof(FlAttnBwdParams)}")
-    if path is None:
-        _lib = lib
+    _lib = lib
     return lib
 
 

@@ -54,3 +54,19 @@ def test_tiny_sweep_on_gpu(tmp_path):
     assert len(rows) == 14 and {r[0] for r in rows} == set(R.registry())
     assert all(r[1] > 0 and r[2] > 0 for r in rows)
     assert (tmp_path / "b.csv").exists()
+
+
+def test_dropout_registry_is_a_subset_with_the_same_names():
+    # --dropout_p > 0 times the variants that have a dropout kernel, under the forward sweep's names
+    assert set(R.dropout_registry(0.1)) == {"full", "full_with_causal", "full_with_sliding_window", "full_with_prefix_lm"}
+    assert set(R.dropout_registry(0.1)) <= set(R.registry())
+
+
+@pytest.mark.gpu
+def test_tiny_sweep_with_dropout_on_gpu(tmp_path):
+    rows = R.main(["--batch_size", "2", "--seqlen", "512", "--group_size", "1", "--dropout_p", "0.1", "--output",
+                   str(tmp_path / "d")])
+    assert {r[0] for r in rows} == set(R.dropout_registry(0.1)) and all(r[-1] == 0.1 and r[1] > 0 for r in rows)
+    rows = R.main(["--suite", "backward", "--batch_size", "2", "--seqlen", "512", "--group_size", "1", "--dropout_p", "0.1",
+                   "--output", str(tmp_path / "e")])
+    assert {r[0] for r in rows} == {n + "_bwd" for n in R.dropout_registry(0.1)}

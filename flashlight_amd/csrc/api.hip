@@ -138,10 +138,9 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   if (p->dropout_threshold) {
     if (p->dropout_threshold > 65535u)
       return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
-    if (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind) || p->bias[0] || p->bias[1] || p->gate || p->diff ||
-        p->attended_dump)
-      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional masks only (no ALiBi, soft-cap, document mask, bias, "
-                                      "gate, differential attention, dump)");
+    if (is_doc(p->mask_kind) || p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
+      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional masks, ALiBi and the soft-cap only (no document mask, "
+                                      "bias, gate, differential attention, dump)");
   }
   if (p->lse) {
     if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
@@ -389,7 +388,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     if (want) return fail(FL_ERR_UNSUPPORTED, "backward: document masks cannot be combined with ALiBi or a soft-cap");
     want = fl::F_DOC;
   }
-  if (p->dropout_threshold) want = fl::F_DROPOUT;  // validate() has excluded every other feature
+  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() has excluded document masks
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)

@@ -126,7 +126,8 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     _ffi.dropout_threshold(dropout_p)  # range check
     if dropout_p > 0.0:
         if biases or gate is not None or diff or seq_major_out:
-            raise NotImplementedError("dropout is built for positional masks and grouped-query attention only")
+            raise NotImplementedError("dropout is built for positional masks, the in-kernel ALiBi term and the soft-cap; not "
+                                      "for bias operands, the gate or differential attention")
         if dropout_seed is None:
             if torch.compiler.is_compiling():
                 raise NotImplementedError("dropout under torch.compile needs an explicit dropout_seed (a seed drawn "

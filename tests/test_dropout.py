@@ -158,7 +158,12 @@ def test_abi_validation_of_dropout_fields():
     p.dropout_threshold = 65536
     assert rc(p) == -5 and "dropout_threshold" in _ffi.last_error()
     for mutate in (lambda p: setattr(p, "alibi_heads", 4), lambda p: setattr(p, "softcap", 30.0),
-                   lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000)),
+                   lambda p: (setattr(p, "alibi_heads", 4), setattr(p, "softcap", 30.0))):
+        p = good_params()
+        p.dropout_threshold = 100
+        mutate(p)
+        assert rc(p) == 0, _ffi.last_error()
+    for mutate in (lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000)),
                    lambda p: setattr(p, "diff", 1)):
         p = good_params()
         p.dropout_threshold = 100
@@ -247,6 +252,33 @@ def test_forward_and_gradients_with_dropout_match_the_oracle(case):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("alibi,softcap", [(True, None), (False, 3.0), (True, 5.0)])
+def test_dropout_with_alibi_and_softcap(D, alibi, softcap):
+    B, Hq, Hkv, L = 1, 4, 2, 230
+    q, k, v, dout = _gpu_inputs(B, Hq, Hkv, L, L, D, seed=D + (7 if alibi else 0))
+    p, seed = 0.2, 0xABCDEF0123
+    kw = dict(mask_kind=_ffi.MASK_CAUSAL, alibi_heads=Hq if alibi else 0, softcap=softcap or 0.0, dropout_p=p, dropout_seed=seed)
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, **kw)
+    torch.cuda.synchronize()
+    import oracle as O
+    bias = None
+    if alibi:
+        rel = (torch.arange(L)[None, :] - torch.arange(L)[:, None]).float()
+        bias = O.alibi_slopes(Hq)[:, None, None] * rel[None]
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    ref = OD.attention_dropout(qf, kf, vf, OD.keep_mask(seed, B, Hq, L, L, p), p, attend=_attend(_ffi.MASK_CAUSAL, L, L),
+                               bias=bias, softcap=softcap)
+    ref.backward(dout.float().cpu())
+    assert_parity(out, ref, "forward with dropout and score modifications")
+    for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{what} with dropout and score modifications")
+
+
+@pytest.mark.gpu
 def test_dropout_fp16_forward_and_determinism():
     q, k, v, _ = _gpu_inputs(1, 2, 2, 192, 192, 128, seed=3)
     q, k, v = (t.to(torch.float16) for t in (q, k, v))
@@ -273,8 +305,9 @@ def test_dropout_through_autograd_and_the_variant_switch():
         b = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
         c = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
         assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a, base)
-        with pytest.raises(_ffi.FlashlightError, match="dropout"):
-            A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(30.0), dropout_p=0.1, enable_gqa=True)
+        with pytest.raises(NotImplementedError, match="dropout"):  # a dense score_mod tensor goes through the bias path
+            A.attention_pytorch_alibi(q, k, v, score_mod=lambda L, S: torch.zeros(4, L, S, device=DEV), dropout_p=0.1,
+                                      enable_gqa=True)
     # autograd: the backward regenerates the forward's decisions from the seed
     qg, kg, vg = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
     out = ops.dispatch(qg, kg, vg, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.3, dropout_seed=2024)

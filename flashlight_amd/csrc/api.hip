@@ -312,11 +312,12 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   kp.bias_row = -1;
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb] || p->bias_strides[nb][3] != 1 || reinterpret_cast<uintptr_t>(p->bias[nb]) % 16 != 0) continue;
-    if (p->Lk % 8 != 0 || kp.bias_f32[nb]) continue;
+    if (p->Lk % 8 != 0) continue;
+    if (kp.bias_f32[nb] && p->bias_strides[nb][2] != 0) continue;  // fp32: only a row-broadcast operand is staged
     bool ok = true;
     for (int i = 0; i < 3; ++i) ok = ok && p->bias_strides[nb][i] % 8 == 0;
     // per-lane byte offsets inside one (batch, head) slice are 32-bit
-    ok = ok && ((int64_t)p->Lq * p->bias_strides[nb][2] + p->Lk) * 2 < ((int64_t)1 << 31);
+    ok = ok && ((int64_t)p->Lq * p->bias_strides[nb][2] + p->Lk) * 4 < ((int64_t)1 << 31);
     if (!ok) continue;
     if (p->bias_strides[nb][2] == 0 && kp.bias_row < 0) kp.bias_row = nb;
     else if (kp.bias_lds < 0) kp.bias_lds = nb;

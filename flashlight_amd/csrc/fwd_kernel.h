@@ -685,9 +685,14 @@ void fwd_kernel(const KParams p) {
     }
     const int nbr = kBias ? p.bias_row : -1;
     const bf16_t* rptr = nullptr;
+    bool row_f32 = false;  // the staged row operand holds fp32 elements (4 keys per 16-byte chunk instead of 8)
     const unsigned lds_r = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::R_OFF + wave * 1024);
     if constexpr (kBias) {
-      if (nbr >= 0) rptr = p.bias[nbr] + (int64_t)(batch / p.bdiv[nbr]) * p.bs[nbr][0] + (int64_t)head * p.bs[nbr][1];
+      if (nbr >= 0) {
+        row_f32 = p.bias_f32[nbr] != 0;
+        // (element offsets; the pointer is typed bf16_t, so an fp32 operand's offset counts twice)
+        rptr = p.bias[nbr] + ((int64_t)(batch / p.bdiv[nbr]) * p.bs[nbr][0] + (int64_t)head * p.bs[nbr][1]) * (row_f32 ? 2 : 1);
+      }
     }
     bool any_direct = false;
     if constexpr (kBias) {
@@ -699,7 +704,12 @@ void fwd_kernel(const KParams p) {
         if (nbr >= 0) {
           // lanes repeat the row's BN / 8 chunks; chunks past Lk repeat the last one
           const int last_chunk = (min(p.Lk - t * BN, BN)) / 8 - 1;
-          dma16(uniform_ptr(rptr + (int64_t)t * BN), (unsigned)min(lane % LB::CPR, last_chunk) * 16u, lds_r + slot * T::RBYTES);
+          if (row_f32) {
+            const int last4 = (min(p.Lk - t * BN, BN)) / 4 - 1;
+            dma16(uniform_ptr(rptr + (int64_t)t * BN * 2), (unsigned)min(lane % (BN / 4), last4) * 16u, lds_r + slot * T::RBYTES);
+          } else {
+            dma16(uniform_ptr(rptr + (int64_t)t * BN), (unsigned)min(lane % LB::CPR, last_chunk) * 16u, lds_r + slot * T::RBYTES);
+          }
         }
         if (!stage_bias) return;
         const uint64_t base = uniform_ptr(bptr + (int64_t)t * BN);
@@ -784,12 +794,21 @@ void fwd_kernel(const KParams p) {
               for (int i = 0; i < 16; ++i) bv[i] = 0.f;
               if (nbr >= 0) {
                 // row-broadcast operand: keys 32 kb + 8 g + 4 h .. + 4 of this wave's staged row
-                const unsigned char* bl = smem + T::R_OFF + bslot * T::RBYTES + wave * 1024 + 8 * h;
+                const unsigned char* bl = smem + T::R_OFF + bslot * T::RBYTES + wave * 1024;
+                if (row_f32) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                  const ex4 b4 = *reinterpret_cast<const ex4*>(bl + (4 * kb + g) * 16);
+                  for (int g = 0; g < 4; ++g) {
+                    const f32x4 b4 = *reinterpret_cast<const f32x4*>(bl + (32 * kb + 8 * g + 4 * h) * 4);
 #pragma unroll
-                  for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                    for (int e = 0; e < 4; ++e) bv[4 * g + e] += b4[e];
+                  }
+                } else {
+#pragma unroll
+                  for (int g = 0; g < 4; ++g) {
+                    const ex4 b4 = *reinterpret_cast<const ex4*>(bl + 8 * h + (4 * kb + g) * 16);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) bv[4 * g + e] += (float)b4[e];
+                  }
                 }
               }
               if (nbl >= 0) {

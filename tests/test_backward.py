@@ -192,6 +192,22 @@ def test_gradients_document_mask(D, causal):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+def test_gradients_document_mask_many_dead_tiles(D):
+    """Several documents over many tiles: most (owner block, streamed tile) pairs are dead, and the backward hops from
+    one live step to the next; one document has a single position, one ends on a tile edge."""
+    L = 1500
+    lengths = [128, 1, 300, 255, 416, 400]
+    assert sum(lengths) == L
+    ids = torch.repeat_interleave(torch.arange(len(lengths)), torch.tensor(lengths))[None].expand(2, L).contiguous().to(DEV)
+    q, k, v, dout = _inputs(2, 4, 2, L, D, seed=99 + D)
+    for causal in (False, True):
+        _check(f"document long causal={causal} D={D}",
+               lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal),
+               lambda q, k, v: O.attention_document_mask(q, k, v, ids, enable_gqa=True, is_causal=causal), q, k, v, dout)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("L,S", [(1, 1), (31, 31), (64, 200), (200, 64), (129, 257), (1000, 1000)])
 def test_gradients_ragged_and_cross_lengths(L, S):
     for D in (64, 128):

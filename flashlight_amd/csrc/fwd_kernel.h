@@ -768,6 +768,10 @@ void fwd_kernel(const KParams p) {
             // (called once on every path below, so that the path without global loads does not meet the other one
             // before the scores are final: a wait for those loads after the join would run on every tile, and would
             // also wait for the K/V transfers in flight)
+            // ALiBi: slope * (rel0 + off) with off a per-register constant; slope * rel0 rides in the addend of the
+            // multiply-add that precedes it, leaving one multiply-add with a literal per score
+            const float alibi0 = kAlibi ? slope_l2 * rel0 : 0.f;
+            const float cap_shift = cap_c + alibi0;
             auto combine = [&]() FL_INLINE {
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
@@ -779,11 +783,11 @@ void fwd_kernel(const KParams p) {
                   if constexpr (kSoftcap) {
                     const float e = fast_exp2(x * cap_k1);
                     const float rc = fast_rcp(e + 1.0f);
-                    tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_c);
+                    tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_shift);
                   } else {
-                    tl2 = x * p.scale_log2;
+                    tl2 = kAlibi ? __builtin_fmaf(x, p.scale_log2, alibi0) : x * p.scale_log2;
                   }
-                  if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, rel0 + (float)(8 * (i / 4) + (i % 4)), tl2);
+                  if constexpr (kAlibi) tl2 = __builtin_fmaf(slope_l2, (float)(8 * (i / 4) + (i % 4)), tl2);
                   if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
                 }
                 s[kb][qb][i] = tl2;

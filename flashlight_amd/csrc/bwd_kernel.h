@@ -398,6 +398,11 @@ void bwd_kernel(const BParams p) {
             if (opos >= p.Lk) hi = -(1 << 29);
           }
           float pv[16];
+          // what does not depend on the register goes into one addend: minus the row's LSE, and the ALiBi term at
+          // off = 0 (key - q = rel0 + off in ROLE_DQ, rel0 - off in ROLE_DKV), which leaves slope * off as one
+          // multiply-add with a literal per score
+          const float alibi0 = kAlibi ? slope_l2 * (float)(kDQ ? sbase - opos : opos - sbase) : 0.f;
+          const float slope_off = kDQ ? slope_l2 : -slope_l2;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             f32x4 lse4;
@@ -406,21 +411,19 @@ void bwd_kernel(const BParams p) {
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * g + e, off = 8 * g + e;
               const float x = x1[sb][i];
-              float s2, dfac = 1.0f;  // logit in log2 units; d(score) / d(qk * scale)
+              const float c0 = alibi0 - (kDQ ? lse_o : lse4[e]);
+              float s2, dfac = 1.0f;  // logit in log2 units minus the LSE; d(score) / d(qk * scale)
               if constexpr (kSoftcap) {
                 const float ex = fast_exp2(x * cap_k1);
                 const float rc = fast_rcp(ex + 1.0f);
                 const float th = __builtin_fmaf(rc, -2.0f, 1.0f);  // tanh(x * scale / cap)
-                s2 = cap_on ? th * cap_c : x * p.scale_log2;
+                s2 = cap_on ? __builtin_fmaf(th, cap_c, c0) : __builtin_fmaf(x, p.scale_log2, c0);
                 dfac = cap_on ? __builtin_fmaf(-th, th, 1.0f) : 1.0f;
               } else {
-                s2 = x * p.scale_log2;
+                s2 = __builtin_fmaf(x, p.scale_log2, c0);
               }
-              if constexpr (kAlibi) {
-                const float rel_f = kDQ ? (float)(sbase + off - opos) : (float)(opos - sbase - off);
-                s2 = __builtin_fmaf(slope_l2, rel_f, s2);
-              }
-              float pw = fast_exp2(s2 - (kDQ ? lse_o : lse4[e]));
+              if constexpr (kAlibi) s2 = __builtin_fmaf(slope_off, (float)off, s2);
+              float pw = fast_exp2(s2);
               if (!full) {  // workgroup-uniform
                 bool ok = (off <= hi) & (off >= lo);
                 if constexpr (kDoc) {

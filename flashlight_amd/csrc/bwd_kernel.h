@@ -31,7 +31,7 @@ struct BParams {
   const bf16_t* o;
   const bf16_t* dout;
   const float* lse;    // [B, Hq, Lq], log2 units; +inf for a row that attends nothing
-  float* delta;        // [B, Hq, Lq] scratch: rowsum(dO o O)
+  float* delta;        // [B, Hq, Lq] scratch: minus rowsum(dO o O)
   bf16_t* dq;
   bf16_t* dk;
   bf16_t* dv;
@@ -51,7 +51,7 @@ struct BParams {
   float drop_rescale;
 };
 
-// Delta[b, h, q] = sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
+// delta[b, h, q] = -sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
 template <int DV, class E>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
   typedef E ex8 __attribute__((ext_vector_type(8)));
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BParams p) {
   }
 #pragma unroll
   for (int d = 1; d < LPR; d *= 2) s += __shfl_xor(s, d);
-  if (row < rows && c == 0) p.delta[row] = s;
+  if (row < rows && c == 0) p.delta[row] = -s;  // stored negated: the consumers add it (or start dP's accumulators from it)
 }
 
 template <int D_, int ROLE_, uint32_t FEAT_, class Elem_ = bf16_t>
@@ -195,7 +195,7 @@ void bwd_kernel(const BParams p) {
   // ROLE_DQ: Q and dO fragments of this lane's query row live in registers (B operands), with its LSE and Delta.
   // ROLE_DKV: the workgroup's K and V rows are staged in LDS once and read as B operands where they are used.
   ex8 o1f[kDQ ? KS : 1], o2f[kDQ ? KS : 1];
-  float lse_o = 0.f, delta_o = 0.f;
+  float lse_o = 0.f, delta_o = 0.f;  // delta_o: minus this row's rowsum(dO o O)
   const bf16_t* kptr = p.k + (int64_t)batch * p.ks[0] + (int64_t)kvh * p.ks[1];
   const bf16_t* vptr = p.v + (int64_t)batch * p.vs[0] + (int64_t)kvh * p.vs[1];
   if constexpr (kDQ) {
@@ -341,11 +341,22 @@ void bwd_kernel(const BParams p) {
       // right after X1's, before the weights' vector work; at D = 64 it lives in the block that consumes it.  Both choices
       // are measured: the first is 15 % faster at D = 128 and 1-2 % slower at D = 64.
       f32x16 x2_wide[TB];
-      auto second_product = [&](f32x16 (&x2)[TB]) FL_INLINE {
+      // dP's accumulators start from zero, or (ROLE_DKV without dropout) from the staged -Delta of their rows, which saves
+      // the subtraction per score later
+      constexpr bool kDeltaInit = !kDQ && !kDrop;
+      auto init_x2 = [&](f32x16 (&x2)[TB]) FL_INLINE {
 #pragma unroll
         for (int sb = 0; sb < TB; ++sb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) x2[sb][i] = 0.f;
+          for (int g = 0; g < 4; ++g) {
+            f32x4 nd = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (kDeltaInit) nd = rows4(T::S2_OFF, t0 + 32 * (qh * TB + sb) + 4 * h + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x2[sb][4 * g + e] = nd[e];
+          }
+      };
+      auto second_product = [&](f32x16 (&x2)[TB]) FL_INLINE {
+        init_x2(x2);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           ex8 b2;
@@ -466,10 +477,7 @@ void bwd_kernel(const BParams p) {
         f32x16 x2_here[TB];
         f32x16 (&x2)[TB] = pick<T::WIDE_X2>(x2_wide, x2_here);
         if constexpr (!T::WIDE_X2) {
-#pragma unroll
-          for (int sb = 0; sb < TB; ++sb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) x2[sb][i] = 0.f;
+          init_x2(x2);
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
             ex8 b2;
@@ -486,8 +494,8 @@ void bwd_kernel(const BParams p) {
           const int sbase = t0 + 32 * (qh * TB + sb) + 4 * h;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            f32x4 dl4;
-            if constexpr (!kDQ) dl4 = rows4(T::S2_OFF, sbase + 8 * g);
+            f32x4 dl4 = {0.f, 0.f, 0.f, 0.f};  // minus Delta of the four rows, unless dP already started from it
+            if constexpr (!kDQ && !kDeltaInit) dl4 = rows4(T::S2_OFF, sbase + 8 * g);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int i = 4 * g + e;
@@ -495,9 +503,9 @@ void bwd_kernel(const BParams p) {
               if constexpr (kDrop) {
                 // d(loss) / d(weight) is dP / (1 - p) where the weight was kept and 0 where it was dropped
                 const bool kept = __builtin_bit_cast(int, pd[sb][i]) >= 0;
-                ds = __builtin_fabsf(pd[sb][i]) * ((kept ? x2[sb][i] * p.drop_rescale : 0.f) - (kDQ ? delta_o : dl4[e]));
+                ds = __builtin_fabsf(pd[sb][i]) * ((kept ? x2[sb][i] * p.drop_rescale : 0.f) + (kDQ ? delta_o : dl4[e]));
               } else {
-                ds = pd[sb][i] * (x2[sb][i] - (kDQ ? delta_o : dl4[e]));
+                ds = kDeltaInit ? pd[sb][i] * x2[sb][i] : pd[sb][i] * (x2[sb][i] + (kDQ ? delta_o : dl4[e]));
               }
               dsf[2 * sb + i / 8][i % 8] = (E)ds;
             }

@@ -37,18 +37,25 @@ def parse_args():
 # commands and raw values: profiles/fwd_kernel_d128_cfg1_counters.md
 MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 410.6e6, "cfg1/sliding_window": 311.4e6}
 
+FLUSH_BYTES = 512 << 20  # twice the 256 MB memory-side cache: zeroing it evicts the operands of the previous launch
+CPU_CAP_S = 12.0         # wall-clock cap per configuration for the eager CPU timing
+
 
 def event_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def time_launches(fn, iters: int, warmup: int = 20):
+def time_launches(fn, iters: int, warmup: int = 20, flush=None):
     """Trimmed mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
-    current stream (the stream the kernels are launched on)."""
+    current stream (the stream the kernels are launched on).  With `flush` (a device buffer larger than the caches)
+    the buffer is zeroed before every bracketed launch, like the reference's harness does (benchmarks/_utils.py:145-151
+    there): the launch then reads its operands from HBM."""
     for _ in range(warmup):
         fn()
     pairs = [event_pair() for _ in range(iters)]
     for a, b in pairs:
+        if flush is not None:
+            flush.zero_()
         a.record()
         fn()
         b.record()
@@ -71,32 +78,60 @@ def time_back_to_back(fn, iters: int, warmup: int = 10) -> float:
     return a.elapsed_time(b) / iters
 
 
-def cpu_baseline(threads_hint: int = 0) -> dict:
-    """The eager fp32 restatement of the reference's CPU-runnable path (oracle/), timed on this host's cores on a
-    bounded sample of the benchmark workload: the same three variants at the same S and D, on 1 batch x 2 heads."""
-    import oracle as O  # the checker, imported here only to be timed as the CPU baseline
+def roofline_entry(w, ms: float, W) -> dict:
+    """Fraction of the roofline that bounds workload `w` at a launch duration of `ms`: unmasked FLOPs against the bf16
+    MFMA peak, or algorithmic bytes (every operand and the result touched once) against the HBM peak."""
+    if w.bound == "hbm":
+        gbps = w.min_bytes / ms / 1e6
+        return {"bound": "hbm", "achieved": gbps, "peak": W.PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / W.PEAK_HBM_GBPS}
+    tf = w.flops / ms / 1e9
+    return {"bound": "mfma", "achieved": tf, "peak": W.PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / W.PEAK_BF16_TFLOPS}
+
+
+def _cpu_chunks(t: dict):
+    """Independent slices of a workload's CPU tensors: one per batch element, or per 32 N_seq rows of the 5-D
+    Evoformer layout [B, N_seq, S, H, D] (whose pair bias [B, 1, H, S, S] is shared by all of them)."""
+    q = t["q"]
+    if q.dim() == 5:
+        for a in range(0, q.size(1), 32):
+            yield {k: (v if k == "pair_bias" else v[:, a:a + 32]) for k, v in t.items()}
+    else:
+        for b in range(q.size(0)):
+            yield {k: v[b:b + 1] for k, v in t.items()}
+
+
+def cpu_baseline() -> dict:
+    """The eager fp32 restatement of the reference's CPU-runnable path (oracle/), timed on this host's cores: once over
+    every benchmark configuration, in independent slices (one batch element at a time) and query blocks of 512 rows so
+    that the dense score matrices fit, under a wall-clock cap per configuration.  `value` is the headline step
+    (configuration 1: vanilla + causal + sliding window); a configuration that hits the cap reports the rate of the
+    slices it finished and says so."""
+    from oracle.benchmark_cases import evaluate  # the checker, imported here only to be timed as the CPU baseline
+    import oracle as O
     from flashlight_amd import workloads as W
 
-    B, H, S, D = 1, 2, 4096, 128
-    g = torch.Generator().manual_seed(1001)
-    q, k, v = (torch.randn(B, H, S, D, generator=g) for _ in range(3))
-    fns = {"vanilla": lambda: O.attention_vanilla(q, k, v),
-           "causal": lambda: O.attention_causal(q, k, v),
-           "sliding_window": lambda: O.attention_sliding_window(q, k, v, window_size=256)}
-    pairs = {"vanilla": W.pairs_none(S), "causal": W.pairs_causal(S), "sliding_window": W.pairs_sliding(S, 256)}
-    flops = sum(4 * D * p * B * H for p in pairs.values())
-    for f in fns.values():
-        f()  # warm-up
-    reps, t_total = 0, 0.0
-    per = {n: [] for n in fns}
-    while reps < 3 or (t_total < 10.0 and reps < 40):
-        for n, f in fns.items():
+    cpu = torch.device("cpu")
+    per = {}
+    for w in W.build_workloads():
+        t = {k: (v.float() if v.is_floating_point() else v) for k, v in w.make(cpu).items()}
+        chunks = list(_cpu_chunks(t))
+        done, elapsed = 0, 0.0
+        for c in chunks:
             t0 = time.perf_counter()
-            f()
-            per[n].append(time.perf_counter() - t0)
-        t_total = sum(sum(x) for x in per.values())
-        reps += 1
-    step_s = sum(statistics.fmean(x) for x in per.values())
+            evaluate(w.name, c, w.params, q_block=512)
+            elapsed += time.perf_counter() - t0
+            done += 1
+            if elapsed > CPU_CAP_S:
+                break
+        full_s = elapsed * len(chunks) / done
+        per[w.name] = {"ms": 1e3 * full_s, "unmasked_TFLOPs": w.flops / full_s / 1e12, "slices_timed": done,
+                       "slices_total": len(chunks)}
+        if done < len(chunks):
+            per[w.name]["note"] = (f"skipped: over cap ({CPU_CAP_S:.0f} s) after {done} of {len(chunks)} slices; ms is "
+                                   "extrapolated from the slices timed")
+        del t, chunks
+    cfg1 = [w for w in W.build_workloads() if w.config == 1]
+    step_s = sum(per[w.name]["ms"] for w in cfg1) / 1e3
     # configuration 0 of the baseline file: causal, B=2 H=8 S=512 D=64 fp32, the reference's own CPU-sized case
     g0 = torch.Generator().manual_seed(1000)
     q0, k0, v0 = (torch.randn(2, 8, 512, 64, generator=g0) for _ in range(3))
@@ -108,11 +143,12 @@ def cpu_baseline(threads_hint: int = 0) -> dict:
         t0s.append(time.perf_counter() - t0)
     cfg0_flops = 4 * 64 * W.pairs_causal(512) * 16
     return {
-        "value": flops / step_s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"eager fp32 oracle, dense scores like the reference, vanilla+causal+sliding(256) at B={B} H={H} "
-                  f"S={S} D={D} ({reps} reps, {t_total:.1f} s); unmasked FLOPs",
-        "ms_per_variant": {n: 1e3 * statistics.fmean(x) for n, x in per.items()},
-        "host_cpus": os.cpu_count(),
+        "value": sum(w.flops for w in cfg1) / step_s / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "eager fp32 oracle (dense scores like the reference, 512 query rows at a time), one pass over the "
+                  "whole of configuration 1 (vanilla + causal + sliding window 256 at B=4 H=16 S=4096 D=128), "
+                  f"{step_s:.1f} s; unmasked FLOPs.  per_config holds one pass over each other configuration",
+        "per_config": per, "cap_s_per_config": CPU_CAP_S, "host_cpus": os.cpu_count(),
         "cfg0_causal_fp32_B2_H8_S512_D64": {"ms": 1e3 * statistics.median(t0s),
                                               "unmasked_GFLOPs": cfg0_flops / statistics.median(t0s) / 1e9},
     }
@@ -158,21 +194,27 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # per-launch durations of each variant, HIP events on the launch stream
+    # per-launch durations of each variant, HIP events on the launch stream: warm (the same operands launch after
+    # launch, partly served by the 256 MB memory-side cache) and flushed (a 512 MB buffer zeroed before each launch)
+    flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
     variants = {}
     for w in cfg1:
         mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(50, args.steps))
+        cold_ms, cold_med = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush)
         tf = w.flops / mean_ms / 1e9
         variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
                             "ms_back_to_back": time_back_to_back(lambda w=w: w.call(tens), iters=max(50, args.steps), warmup=20),
+                            "ms_flushed": cold_ms, "ms_flushed_median": cold_med, "tflops_flushed": w.flops / cold_ms / 1e9,
                             "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
-                            "hbm_floor_GBps_at_this_time": w.min_bytes / mean_ms / 1e6}
+                            "roofline": roofline_entry(w, mean_ms, W), "roofline_flushed": roofline_entry(w, cold_ms, W)}
     dom = max(cfg1, key=lambda w: variants[w.name]["ms"])  # the launch that dominates the step
     dv = variants[dom.name]
     roofline = {"bound": "mfma", "kernel": f"fl::fwd_kernel ({dom.name})", "achieved": dv["tflops"],
                 "peak": W.PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dv["tflops"] / W.PEAK_BF16_TFLOPS,
+                "frac_flushed": dv["tflops_flushed"] / W.PEAK_BF16_TFLOPS,
                 "traffic": MEASURED_HBM_BYTES.get(dom.name), "traffic_unit": "bytes/launch (rocprofv3, see profiles/)",
                 "launch_ms": dv["ms"], "flops_per_launch": dom.flops}
+    step_flushed_ms = sum(v["ms_flushed"] for v in variants.values())
 
     others = {}
     if not args.no_other_configs:
@@ -182,12 +224,17 @@ def main():
                 continue
             t = w.make(dev)
             mean_ms = time_back_to_back(lambda: w.call(t), iters=100, warmup=50)
+            cold_ms, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush)
             tf = w.flops / mean_ms / 1e9
-            others[w.name] = {"ms": mean_ms, "timing": "100 launches back to back after 50 warm-up launches", "tflops": tf,
+            others[w.name] = {"ms": mean_ms, "timing": "warm: 100 launches back to back after 50 warm-up launches; "
+                                                       "flushed: 50 launches, 512 MB zeroed before each",
+                              "ms_flushed": cold_ms, "tflops": tf, "tflops_flushed": w.flops / cold_ms / 1e9,
                               "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS, "unmasked_flops": w.flops,
-                              "min_bytes": w.min_bytes, "GBps_on_min_bytes": w.min_bytes / mean_ms / 1e6}
+                              "min_bytes": w.min_bytes, "roofline": roofline_entry(w, mean_ms, W),
+                              "roofline_flushed": roofline_entry(w, cold_ms, W)}
             del t
             torch.cuda.empty_cache()
+    del flush
 
     # What the matrix pipe alone sustains on this part (same MFMA instruction, operands in registers, nothing else
     # running), on N(0,1) operands like the benchmark's and on zeros, and the forward itself on all-zero inputs: the
@@ -210,6 +257,8 @@ def main():
         zeros = {k: torch.zeros_like(v) for k, v in tens.items()}
         ms = time_back_to_back(lambda: cfg1[0].call(zeros), iters=100, warmup=30)
         context["vanilla_on_zero_inputs_TFLOPs"] = cfg1[0].flops / ms / 1e9
+        # the dominant launch against what the matrix pipe alone sustains on the same kind of data in this run
+        context["roofline_frac_vs_mfma_only_randn"] = roofline["achieved"] / context["mfma_only_randn_operands_TFLOPs"]
         del tens, zeros, ops
 
     if args.calibrate_copy:
@@ -226,6 +275,9 @@ def main():
                                "B=4 H=16 S=4096 D=128, one launch each per step",
                    "seed": cfg1[0].seed, "unmasked_flops_per_step": step_flops},
         "pct_mfma_peak": 100 * step_flops / wall_ms / 1e9 / W.PEAK_BF16_TFLOPS,
+        "cache_state": "value and ms_per_step: warm (steps back to back on the same operands); *_flushed: 512 MB zeroed "
+                       "before each launch",
+        "ms_per_step_flushed": step_flushed_ms, "value_flushed": step_flops / step_flushed_ms / 1e9,
         "peak_used_TFLOPs": W.PEAK_BF16_TFLOPS,
         "variants": variants, "roofline": roofline, "other_configs": others, "power_context": context,
         "device": torch.cuda.get_device_name(0),

@@ -322,6 +322,9 @@ def attn_fwd(
         # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,
         # so wide values go in slabs of _MAX_DV_DIFF columns, one launch each, through strided views of v and out
         # (the reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38).
+        if lse is not None or dropout_p > 0.0:
+            # what the single launch refuses for differential attention is refused here too, instead of dropped
+            raise NotImplementedError("differential attention produces no lse and takes no dropout")
         for c in range(0, Dv, _MAX_DV_DIFF):
             attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
                      doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,

@@ -65,8 +65,15 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   int best_extra = 1 << 30;
   // Tuning knob: FL_TILE=<rows per wave>x<keys per tile>x<waves>x<ring depth>, e.g. 32x32x4x4, restricts the choice
   // to instances of that shape (the default is the first listed instance that fits).
-  int want_rw = 0, want_bn = 0, want_nw = 0, want_ns = 0;
-  if (const char* e = std::getenv("FL_TILE")) std::sscanf(e, "%dx%dx%dx%d", &want_rw, &want_bn, &want_nw, &want_ns);
+  // The environment is read once, when the first launch is planned.
+  struct TileKnob {
+    int rw = 0, bn = 0, nw = 0, ns = 0;
+    TileKnob() {
+      if (const char* e = std::getenv("FL_TILE")) std::sscanf(e, "%dx%dx%dx%d", &rw, &bn, &nw, &ns);
+    }
+  };
+  static const TileKnob knob;
+  const int want_rw = knob.rw, want_bn = knob.bn, want_nw = knob.nw, want_ns = knob.ns;
   // keys one workgroup of 128 query rows visits: the window plus its own rows for a sliding window, else up to Lk
   const int64_t visited = p->mask_kind == FL_MASK_SLIDING ? std::min<int64_t>(p->Lk, (int64_t)p->window + 128) : p->Lk;
   const bool short_loop = p->mask_kind == FL_MASK_SLIDING && visited <= 640;

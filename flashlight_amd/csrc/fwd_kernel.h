@@ -1054,7 +1054,10 @@ void fwd_kernel(const KParams p) {
     // reference, weights again.  Any reference gives the same O / l; fp32 sums keep their relative precision.
     // ALiBi moves the scores by a large, steady amount from tile to tile; its kernels visit the tiles in descending key
     // order (see list_entry), so that the amount is downwards and the first reference holds.
-    constexpr float kBig = 0x1p24f, kTiny = 0x1p-24f;
+    // The underflow bound follows the element type: a bf16 weight keeps its 8 bits down to 2^-126, an fp16 weight is
+    // subnormal below 2^-14 (absolute error up to 2^-25) and zero below 2^-25.  With a row sum of at least 2^-4 the
+    // rounding of one tile's 64 subnormal weights stays below 2^-15 of the sum.
+    constexpr float kBig = 0x1p24f, kTiny = std::is_same<typename T::Elem, f16_t>::value ? 0x1p-4f : 0x1p-24f;
     constexpr bool kFastRef = true;
     auto weights_checked = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], bool check, auto in_loop,
                                ex8 (&vfirst)[DVB], int vslot, int t) FL_INLINE {

@@ -66,6 +66,8 @@ class Workload:
     min_bytes: int       # q + k + v + out (+ bias + gate + ids), each touched once
     make: Callable[[torch.device], dict] = field(repr=False, default=None)
     call: Callable[[dict], torch.Tensor] = field(repr=False, default=None)
+    params: Dict[str, float] = field(default_factory=dict)  # the variant's own arguments (window, prefix, cap, lambda)
+    bound: str = "mfma"  # the roofline that bounds the launch: "mfma", or "hbm" where a head's work is a few key tiles
 
     @property
     def flops(self) -> int:
@@ -105,7 +107,8 @@ def build_workloads(scale_down: int = 1) -> List[Workload]:
             ("sliding_window", pairs_sliding(S, win),
              lambda t, win=win: attention_pytorch_sliding_window(t["q"], t["k"], t["v"], window_size=win))):
         W.append(Workload(f"cfg1/{name}", 1, 1001, {"q": (B, H, S, D), "kv": (B, H, S, D)}, pairs, B * H, 4 * D, io,
-                          _qkv(1001, B, H, H, S, D), fn))
+                          _qkv(1001, B, H, H, S, D), fn, params={"window": win} if name == "sliding_window" else {},
+                          bound="hbm" if name == "sliding_window" else "mfma"))
 
     # cfg2: GQA + ALiBi + softcap 50 + causal, B=2 Hq=32 Hkv=8 S=8192 D=128
     B, Hq, Hkv, S, D = 2, 32, 8, 8192 // sd, 128
@@ -114,7 +117,8 @@ def build_workloads(scale_down: int = 1) -> List[Workload]:
                       pairs_causal(S), B * Hq, 4 * D, io, _qkv(1002, B, Hq, Hkv, S, D),
                       lambda t: attention_pytorch_alibi(t["q"], t["k"], t["v"],
                                                         score_mod=generate_alibi_bias_pytorch(t["q"].size(1)),
-                                                        is_causal=True, enable_gqa=True, softcap=50.0)))
+                                                        is_causal=True, enable_gqa=True, softcap=50.0),
+                      params={"softcap": 50.0}))
 
     # cfg3a: document mask, causal within each document, B=1 H=16 S=16384 D=64
     B, H, S, D = 1, 16, 16384 // sd, 64
@@ -135,7 +139,8 @@ def build_workloads(scale_down: int = 1) -> List[Workload]:
     io = 2 * 4 * B * H * S * D
     W.append(Workload("cfg3/prefix_lm", 3, 1013, {"q": (B, H, S, D), "kv": (B, H, S, D)}, pairs_prefix(S, P), B * H,
                       4 * D, io, _qkv(1013, B, H, H, S, D),
-                      lambda t, P=P: attention_pytorch_prefix_lm(t["q"], t["k"], t["v"], prefix_lengths=P)))
+                      lambda t, P=P: attention_pytorch_prefix_lm(t["q"], t["k"], t["v"], prefix_lengths=P),
+                      params={"prefix": P}))
 
     # cfg4a: differential attention, B=2 H=16 (q, k: 32 heads x 64; v: 16 heads x 128), S=4096, causal, lambda 0.8
     B, H, S, d = 2, 16, 4096 // sd, 64
@@ -147,7 +152,8 @@ def build_workloads(scale_down: int = 1) -> List[Workload]:
                 "v": _randn(g, (B, H, S, 2 * d), device)}
     W.append(Workload("cfg4/diff_attn_causal", 4, 1004, {"q": (B, 2 * H, S, d), "v": (B, H, S, 2 * d)}, pairs_causal(S),
                       B * H, 2 * (2 * d + 2 * 2 * d), io, make_diff,
-                      lambda t: diffattn(t["q"], t["k"], t["v"], lambda_full=0.8, is_causal=True)))
+                      lambda t: diffattn(t["q"], t["k"], t["v"], lambda_full=0.8, is_causal=True),
+                      params={"lambda_full": 0.8}))
 
     # cfg4b: Evoformer row attention, B=1 N_seq=256 N_res=384 H=8 D=32, pair bias + sigmoid gate
     B, Nseq, S, H, D = 1, 256 // sd, 384, 8, 32
@@ -161,7 +167,8 @@ def build_workloads(scale_down: int = 1) -> List[Workload]:
         return t
     W.append(Workload("cfg4/evoformer_bias_gate", 4, 1014, {"qkv": (B, Nseq, S, H, D), "bias": (B, 1, H, S, S)},
                       pairs_none(S), B * Nseq * H, 4 * D, io, make_evo,
-                      lambda t: attention_reference(t["q"], t["k"], t["v"], [t["pair_bias"]], gate=t["gate"])))
+                      lambda t: attention_reference(t["q"], t["k"], t["v"], [t["pair_bias"]], gate=t["gate"]),
+                      bound="hbm"))
     return W
 
 

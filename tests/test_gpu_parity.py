@@ -42,31 +42,8 @@ def test_known_answer_vectors(golden, name):
 
 def oracle_for(w: W.Workload, t: dict, q_block):
     """fp32 oracle evaluation of a benchmark workload, on the tensors' device (plain eager PyTorch either way)."""
-    q, k, v = f32(t["q"], t["k"], t["v"])
-    n = w.name.split("/")[1]
-    if n == "vanilla":
-        return O.attention_vanilla(q, k, v, q_block=q_block)
-    if n == "causal":
-        return O.attention_causal(q, k, v, q_block=q_block)
-    if n == "sliding_window":
-        win = W.pairs_sliding  # noqa: F841  (window recovered from the pair count below)
-        S = q.size(2)
-        window = next(x for x in (256, 128, 64, 32, 16) if W.pairs_sliding(S, x) == w.pairs_per_head)
-        return O.attention_sliding_window(q, k, v, window_size=window, q_block=q_block)
-    if n == "gqa_alibi_softcap_causal":
-        return O.attention_alibi(q, k, v, score_mod=q.size(1), is_causal=True, honor_causal=True, enable_gqa=True,
-                                 softcap=50.0, q_block=q_block)
-    if n == "document_mask_causal":
-        return O.attention_document_mask(q, k, v, t["document_id"], is_causal=True, q_block=q_block)
-    if n == "prefix_lm":
-        S = q.size(2)
-        P = next(x for x in (1024, 512, 256, 128, 64) if W.pairs_prefix(S, x) == w.pairs_per_head)
-        return O.attention_prefix_lm(q, k, v, prefix_lengths=P, q_block=q_block)
-    if n == "diff_attn_causal":
-        return O.diff_attention(q, k, v, lambda_full=0.8, is_causal=True, q_block=q_block)
-    if n == "evoformer_bias_gate":
-        return O.attention_evoformer(q, k, v, [t["pair_bias"].float()], gate=t["gate"].float(), q_block=q_block)
-    raise KeyError(w.name)
+    from oracle.benchmark_cases import evaluate
+    return evaluate(w.name, {k: (v.float() if v.is_floating_point() else v) for k, v in t.items()}, w.params, q_block)
 
 
 WORKLOAD_NAMES = [w.name for w in W.build_workloads()]
@@ -103,17 +80,16 @@ def test_benchmark_configs_full_size(name):
 # ---- assert_close(atol=2e-2, rtol=1e-2) (e.g. tests/test_causal.py:36 of the reference).
 
 def assert_script_tolerance(out, ref, what=""):
-    """|out - ref| <= 2e-2 + 1e-2 |ref| like the reference's scripts.  With inputs in [-9, 9] a softmax row is close to
-    one-hot and an output near zero is a cancellation of values of magnitude 9 whose bf16 weights carry 2^-9 relative
-    rounding each, so a handful of elements land just past the bound (the reference's scripts note the same, e.g.
-    "~4/4M elements exceed 1e-2", tests/test_alibi.py:37-39 there): at most 1 element in 10^5 may exceed it, and
-    none by more than a factor of two."""
+    """The reference scripts' own check, every element: |out - ref| <= 2e-2 + 1e-2 |ref|
+    (torch.testing.assert_close(atol=2e-2, rtol=1e-2), e.g. tests/test_causal.py:36, tests/test_alibi.py:40 there).
+    On failure the message carries the worst excess over the bound and how many elements are past it."""
     assert tuple(out.shape) == tuple(ref.shape), what
     o, r = out.float(), ref.float().to(out.device)
     assert torch.isfinite(o).all(), what
     excess = (o - r).abs() / (2e-2 + 1e-2 * r.abs())
-    frac = (excess > 1).float().mean().item()
-    assert excess.max().item() <= 2.0 and frac <= 1e-5, f"{what}: worst {excess.max().item():.2f}x bound, {frac:.2e} over"
+    n_over = int((excess > 1).sum().item())
+    print(f"[script tolerance] {what}: worst {excess.max().item():.3f} x bound, {n_over} of {excess.numel()} over")
+    assert n_over == 0, f"{what}: worst {excess.max().item():.3f} x bound, {n_over} of {excess.numel()} elements over"
 
 
 def test_reference_script_vanilla_and_causal():   # tests/test_vanilla.py:21-36, tests/test_causal.py:21-36
@@ -473,3 +449,41 @@ def test_fp16_large_weights_take_the_exact_path():
     q, k, v = (t.to(torch.float16).to(DEV) for t in (q * 4, k * 4, v))
     out = A.attention_pytorch(q, k, v, scale=1.0)
     assert_parity(out, O.attention_vanilla(*f32(q, k, v), scale=1.0), "fp16 large logits")
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("via_bias", [False, True])
+def test_fp16_weights_in_the_subnormal_band(D, via_bias):
+    # every logit sits 12 to 18 nats below zero, the reference a row starts with: weights formed against it are fp16
+    # subnormals (2^-17 .. 2^-26, a few bits or none), so the kernel has to notice the small row sums and settle a
+    # reference from the row maxima before it trusts them.  Driven once through q.k itself (plain instances) and once
+    # through a dense fp32 score_mod (bias instances).
+    g = torch.Generator().manual_seed(77)
+    S = 1024
+    q = torch.randn(1, 2, S, D, generator=g) * 0.5
+    k = torch.randn(1, 2, S, D, generator=g) * 0.5
+    v = torch.randn(1, 2, S, D, generator=g)
+    low = -(12.0 + 5.0 * torch.rand(S, generator=g))  # per key, natural units
+    if not via_bias:
+        q[..., 0] = math.sqrt(D)
+        k[..., 0] = low  # q0 * k0 / sqrt(D) = low
+    q, k, v = (t.to(torch.float16).to(DEV) for t in (q, k, v))
+    qf, kf, vf = f32(q, k, v)
+    if via_bias:
+        bias = low.view(1, 1, 1, S).expand(1, 2, S, S).contiguous().to(DEV)
+        out = A.attention_pytorch_alibi(q, k, v, score_mod=lambda l, s: bias)
+        ref = O.attention_alibi(qf, kf, vf, score_mod=lambda l, s: bias)
+        assert_parity(out, ref, "dense score_mod")
+        return
+    assert_parity(A.attention_pytorch(q, k, v), O.attention_vanilla(qf, kf, vf), "vanilla")
+    assert_parity(A.attention_pytorch_causal(q, k, v), O.attention_causal(qf, kf, vf), "causal")
+
+
+def test_config0_shape_causal():
+    # configuration 0 of the baseline file (the reference's CPU-sized case): causal, B=2 H=8 S=512 D=64, fp32 N(0,1)
+    # inputs from seed 1000; the kernel takes their bf16 rounding, the oracle the fp32 originals
+    g = torch.Generator().manual_seed(1000)
+    q, k, v = (torch.randn(2, 8, 512, 64, generator=g) for _ in range(3))
+    out = A.attention_pytorch_causal(*(t.to(torch.bfloat16).to(DEV) for t in (q, k, v)))
+    assert out.shape == (2, 8, 512, 64)
+    assert_parity(out, O.attention_causal(q, k, v), "config 0")

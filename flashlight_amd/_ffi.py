@@ -112,6 +112,9 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_plan.argtypes = [C.POINTER(FlAttnParams), C.POINTER(C.c_int64)]
     lib.fl_attn_fwd.restype = C.c_int
     lib.fl_attn_fwd.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
+    lib.fl_attn_fwd_static.restype = C.c_int
+    lib.fl_attn_fwd_static.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
+    lib.fl_static_scratch_bytes.restype = C.c_uint64
     lib.fl_bwd_params_sizeof.restype = C.c_uint64
     lib.fl_attn_bwd_validate.restype = C.c_int
     lib.fl_attn_bwd_validate.argtypes = [C.POINTER(FlAttnBwdParams)]
@@ -183,7 +186,7 @@ def dropout_threshold(p: float) -> int:
 
 
 def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases,
-                 gate, diff, lambda_full, attended_dump, dropout_p=0.0, dropout_seed=0):
+                 gate, diff, lambda_full, attended_dump, dropout_p=0.0, dropout_seed=0, alloc_workspace=True):
     """Fills an `fl_attn_params` for validated 4-D tensors; returns it with the tensors that must outlive the launch."""
     B, _, Lq, Dqk = q.shape
     Lk, Dv = k.shape[2], v.shape[3]
@@ -255,7 +258,7 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
                 not attended_dump.is_contiguous() or attended_dump.device != q.device:
             raise ValueError("attended_dump must be a contiguous uint8 [B, Hq, Lq, Lk] tensor on the inputs' device")
         p.attended_dump = attended_dump.data_ptr()
-    need = lib.fl_workspace_bytes(C.byref(p))
+    need = lib.fl_workspace_bytes(C.byref(p)) if alloc_workspace else 0
     if need:
         ws = torch.empty(need, dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), need
@@ -285,6 +288,7 @@ def attn_fwd(
     lse: Optional[torch.Tensor] = None,
     dropout_p: float = 0.0,
     dropout_seed: int = 0,
+    static_scratch: bool = False,
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
@@ -294,6 +298,8 @@ def attn_fwd(
     `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
     `dropout_p` > 0 drops softmax weights (torch.nn.functional.dropout semantics) by a hash of (`dropout_seed`, batch,
     head, query, key); positional masks and GQA only.
+    `static_scratch` goes through `fl_attn_fwd_static`: no workspace is allocated here, the library's own static
+    device array serves as scratch (calls that may overlap on one GPU must not both use it).
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -329,11 +335,12 @@ def attn_fwd(
             attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
                      doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
                      gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
-                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
+                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only, static_scratch=static_scratch)
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed)
+                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed,
+                           alloc_workspace=validate_only or not static_scratch)
     if lse is not None:
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
             raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")
@@ -343,7 +350,8 @@ def attn_fwd(
         return out
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.fl_attn_fwd(C.byref(p), C.c_void_p(stream)))
+        entry = lib.fl_attn_fwd_static if static_scratch else lib.fl_attn_fwd
+        _check(entry(C.byref(p), C.c_void_p(stream)))
     # tensors in `keep` were last used on the current stream; the caching allocator orders their reuse after it
     del keep
     return out

@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "flashlight_amd.h"
 #include "bwd_instances.h"
@@ -29,6 +30,12 @@ static __global__ void doc_table_kernel(const int64_t* ids, int64_t ids_stride, 
 
 }  // namespace fl
 
+// Scratch of the entry point that allocates nothing (fl_attn_fwd_static): one copy per GPU the library runs on, held
+// until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels and memory calls
+// take the device address that call returns (static_scratch_ptr below).
+constexpr size_t kStaticScratchBytes = (size_t)FL_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -39,6 +46,26 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+int static_scratch_ptr(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail((int)e, "hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(FL_ERR_UNSUPPORTED, "device ordinal %d is beyond the %d this library tracks", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail((int)(e != hipSuccess ? e : hipErrorInvalidSymbol), "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
 }
 
 bool is_doc(int kind) { return kind == FL_MASK_DOCUMENT || kind == FL_MASK_DOCUMENT_CAUSAL; }
@@ -362,6 +389,30 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));
   return 0;
 }
+
+int fl_attn_fwd_static(const fl_attn_params* p, void* stream) {
+  if (!p) return fail(FL_ERR_NULL, "params is null");
+  fl_attn_params q = *p;
+  const uint64_t need = fl_workspace_bytes(&q);
+  if (need > kStaticScratchBytes)
+    return fail(FL_ERR_WORKSPACE,
+                "fl_attn_fwd_static: this call needs %llu bytes of scratch, the library's static scratch holds %llu "
+                "(document masks up to B * ceil(Lk / 32) = %llu blocks); use fl_attn_fwd with a caller workspace",
+                (unsigned long long)need, (unsigned long long)kStaticScratchBytes,
+                (unsigned long long)(kStaticScratchBytes / 16));
+  q.workspace = nullptr;
+  q.workspace_bytes = 0;
+  if (need) {
+    void* ptr = nullptr;
+    int rc = static_scratch_ptr(&ptr);
+    if (rc) return rc;
+    q.workspace = ptr;
+    q.workspace_bytes = kStaticScratchBytes;
+  }
+  return fl_attn_fwd(&q, stream);
+}
+
+uint64_t fl_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 uint64_t fl_bwd_params_sizeof(void) { return sizeof(fl_attn_bwd_params); }
 

@@ -146,6 +146,20 @@ uint64_t fl_workspace_bytes(const fl_attn_params* p);
  * Replaces torch.compile(fn)(q, k, v, ...) for the functions of attention_variants/. */
 int fl_attn_fwd(const fl_attn_params* p, void* stream);
 
+/* fl_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as fl_attn_fwd,
+ * except that p->workspace / p->workspace_bytes are ignored: the scratch a document mask needs lives in a static
+ * device array inside the library (FL_STATIC_SCRATCH_BYTES per GPU, held until the process ends), looked up once per
+ * device on the first call made with that device current.  A call whose fl_workspace_bytes() exceeds that size returns
+ * FL_ERR_WORKSPACE and launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine.  All calls
+ * on one GPU share the array: two such calls that may overlap on that GPU (different streams, or different threads)
+ * race; calls queued on one stream are ordered and safe.  Nothing in the array needs clearing between calls: each call
+ * rewrites the part it reads. */
+#define FL_STATIC_SCRATCH_BYTES (4u << 20)
+int fl_attn_fwd_static(const fl_attn_params* p, void* stream);
+/* FL_STATIC_SCRATCH_BYTES of the loaded library. */
+uint64_t fl_static_scratch_bytes(void);
+
 /* Describes the kernel instance fl_attn_fwd would pick for *p: tile sizes and launch shape.
  * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
 int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);

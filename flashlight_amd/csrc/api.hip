@@ -28,6 +28,65 @@ static __global__ void doc_table_kernel(const int64_t* ids, int64_t ids_stride, 
   table[2 * (int64_t)i + 1] = mx;
 }
 
+// Forward pre-pass for document masks, one workgroup of 256 threads per (batch, query tile of `bm` rows): lists the key
+// tiles (of `bn` keys) that some row of the query tile attends, with the class of each for every wave (`rw` rows per
+// wave), from the (min, max) table; the lists are the same for every head.  Output per workgroup: word 0 = number of
+// entries, then the entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).  Also writes
+// the workgroup's share of the padded copy of the ids ([B][nk * bn], positions past L repeat the last id).
+static __global__ __launch_bounds__(256) void doc_lists_kernel(const int64_t* ids, int64_t ids_stride, const int64_t* table,
+                                                               int blocks, int L, int mask_kind, int bm, int rw, int bn,
+                                                               int n_qtiles, int nk, int list_stride, uint32_t* lists,
+                                                               int64_t* ids_padded) {
+  extern __shared__ uint32_t tl[];  // nk words
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int b = blockIdx.x / n_qtiles, qt = blockIdx.x % n_qtiles;
+  const int nw = bm / rw, q0 = qt * bm;
+  const int64_t* dtab = table + (int64_t)b * blocks * 2;
+  for (int i = tid; i < bm; i += 256) {
+    const int pos = q0 + i;
+    if (pos < nk * bn) ids_padded[(int64_t)b * nk * bn + pos] = ids[(int64_t)b * ids_stride + min(pos, L - 1)];
+  }
+  int64_t qmn[8], qmx[8];
+  for (int w = 0; w < 8; ++w) {
+    qmn[w] = qmx[w] = 0;
+    const int a = q0 + w * rw, e = min(a + rw, L);
+    if (w < nw && a < e) doc_range(dtab, a, e, qmn[w], qmx[w]);
+  }
+  for (int t = tid; t < nk; t += 256) {
+    const int k0 = t * bn, k1 = min(k0 + bn, L);
+    int64_t kmn, kmx;
+    doc_range(dtab, k0, k1, kmn, kmx);
+    unsigned c = 0;
+    for (int w = 0; w < nw; ++w) {
+      const int a = q0 + w * rw, e = min(a + rw, L);
+      int cw = TILE_EMPTY;
+      if (a < e) {
+        cw = classify_positional(mask_kind, a, e, k0, k1, 0, 0);
+        if (kmx < qmn[w] || kmn > qmx[w]) cw = TILE_EMPTY;
+        else if (!(kmn == kmx && qmn[w] == qmx[w] && kmn == qmn[w]) && cw == TILE_FULL) cw = TILE_PARTIAL;
+        if (cw == TILE_FULL && k0 + bn > L) cw = TILE_PARTIAL;  // ragged tail: keys >= L are masked
+      }
+      c |= (unsigned)cw << (2 * w);
+    }
+    tl[t] = (c << 16) | (unsigned)t;
+  }
+  __syncthreads();
+  if (tid < 64) {
+    uint32_t* out = lists + (int64_t)blockIdx.x * list_stride;
+    int count = 0;
+    for (int base = 0; base < nk; base += 64) {
+      const int t = base + lane;
+      const uint32_t e = t < nk ? tl[t] : 0u;
+      const bool keep = (e >> 16) != 0;
+      const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
+      const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+      if (keep) out[1 + pos] = e;
+      count += __builtin_popcountll(m);
+    }
+    if (lane == 0) out[0] = (uint32_t)count;
+  }
+}
+
 }  // namespace fl
 
 // Scratch of the entry point that allocates nothing (fl_attn_fwd_static): one copy per GPU the library runs on, held
@@ -122,14 +181,38 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   return best;
 }
 
-// LDS bytes of a launch: the instance's fixed part plus 4 bytes per key tile for the tile list.
+// Device scratch of a document-mask call, in this order (every part a multiple of 16 bytes):
+//   table   [B][ceil(L / 32)][2] int64   (min, max) id per 32 positions (forward pre-pass and backward)
+//   lists   [B][query tiles][stride] u32 the key tiles each query tile visits (forward)
+//   ids     [B][key tiles * bn] int64    the ids padded to whole key tiles (forward)
+// bm / bn: query rows per workgroup and keys per tile of the forward instance.
+struct DocScratch {
+  int64_t blocks, n_qtiles, nk, list_stride;
+  uint64_t table_bytes, lists_bytes, ids_bytes;
+  uint64_t total() const { return table_bytes + lists_bytes + ids_bytes; }
+};
+DocScratch doc_scratch(int64_t B, int64_t L, int64_t bm, int64_t bn) {
+  DocScratch d;
+  d.blocks = (L + fl::kDocBlock - 1) / fl::kDocBlock;
+  d.n_qtiles = (L + bm - 1) / bm;
+  d.nk = (L + bn - 1) / bn;
+  d.list_stride = (d.nk + 1 + 3) / 4 * 4;
+  d.table_bytes = (uint64_t)B * d.blocks * 2 * sizeof(int64_t);
+  d.lists_bytes = (uint64_t)B * d.n_qtiles * d.list_stride * sizeof(uint32_t);
+  d.ids_bytes = (uint64_t)B * d.nk * bn * sizeof(int64_t);
+  return d;
+}
+
+// LDS bytes of a launch: the instance's fixed part plus, under a document mask, the tile list in whole 1 KiB wave
+// transfers.
 int64_t lds_bytes_for(const fl::Instance* in, const fl_attn_params* p) {
-  const int64_t nkt = ((int64_t)p->Lk + in->bn - 1) / in->bn;
-  return in->lds_fixed_bytes + 4 * nkt;
+  if (!(in->feat & fl::F_DOC)) return in->lds_fixed_bytes;
+  const DocScratch d = doc_scratch(p->B, p->Lk, (int64_t)in->rw * in->nw, in->bn);
+  return in->lds_fixed_bytes + (d.list_stride * 4 + 1023) / 1024 * 1024;
 }
 int64_t max_keys_for(const fl::Instance* in) {
-  int64_t tiles = (fl::kMaxLdsBytes - in->lds_fixed_bytes) / 4;
-  if (tiles > fl::kMaxKeyTiles) tiles = fl::kMaxKeyTiles;
+  int64_t tiles = fl::kMaxKeyTiles;
+  if (in->feat & fl::F_DOC) tiles = std::min<int64_t>(tiles, (fl::kMaxLdsBytes - in->lds_fixed_bytes) / 1024 * 256 - 4);
   return tiles * in->bn;
 }
 
@@ -242,7 +325,7 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
     if (!p->workspace || p->workspace_bytes < need)
       return fail(FL_ERR_WORKSPACE, "document mask needs a %llu-byte workspace (got %llu)", (unsigned long long)need,
                   (unsigned long long)(p->workspace ? p->workspace_bytes : 0));
-    if (reinterpret_cast<uintptr_t>(p->workspace) % 8) return fail(FL_ERR_ALIGN, "workspace must be 8-byte aligned");
+    if (reinterpret_cast<uintptr_t>(p->workspace) % 16) return fail(FL_ERR_ALIGN, "workspace must be 16-byte aligned");
   }
   if (out) *out = in;
   g_err[0] = 0;
@@ -261,8 +344,9 @@ uint64_t fl_params_sizeof(void) { return sizeof(fl_attn_params); }
 
 uint64_t fl_workspace_bytes(const fl_attn_params* p) {
   if (!p || !is_doc(p->mask_kind) || p->B <= 0 || p->Lk <= 0) return 0;
-  const uint64_t blocks = ((uint64_t)p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
-  return (uint64_t)p->B * blocks * 2 * sizeof(int64_t);
+  // tile shape of the instance the forward would run (the largest shapes compiled, if the call names no valid one)
+  const fl::Instance* in = select_instance(p);
+  return doc_scratch(p->B, p->Lk, in ? (int64_t)in->rw * in->nw : 128, in ? in->bn : 32).total();
 }
 
 int fl_attn_validate(const fl_attn_params* p) { return validate(p, nullptr); }
@@ -375,15 +459,24 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   const int grid = p->B * p->Hq * kp.n_qtiles;
 
   if (is_doc(p->mask_kind)) {
-    const int blocks = (p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
-    const int total = p->B * blocks;
-    int64_t* table = static_cast<int64_t*>(p->workspace);
+    const DocScratch d = doc_scratch(p->B, p->Lk, bm, in->bn);
+    const int total = p->B * (int)d.blocks;
+    unsigned char* ws = static_cast<unsigned char*>(p->workspace);
+    int64_t* table = reinterpret_cast<int64_t*>(ws);
+    uint32_t* lists = reinterpret_cast<uint32_t*>(ws + d.table_bytes);
+    int64_t* ids_padded = reinterpret_cast<int64_t*>(ws + d.table_bytes + d.lists_bytes);
     hipLaunchKernelGGL(fl::doc_table_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, p->doc_ids, p->doc_stride,
-                       p->Lk, blocks, total, table);
+                       p->Lk, (int)d.blocks, total, table);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail((int)e, "doc_table_kernel launch failed: %s", hipGetErrorString(e));
-    kp.doc_table = table;
-    kp.doc_blocks = blocks;
+    hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(256), (size_t)kp.n_ktiles * 4, stream,
+                       p->doc_ids, p->doc_stride, table, (int)d.blocks, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles,
+                       kp.n_ktiles, (int)d.list_stride, lists, ids_padded);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "doc_lists_kernel launch failed: %s", hipGetErrorString(e));
+    kp.doc_lists = lists;
+    kp.doc_list_stride = (int)d.list_stride;
+    kp.doc_ids_padded = ids_padded;
   }
   hipError_t e = in->launch(kp, grid, (int)lds_bytes_for(in, p), stream);
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));

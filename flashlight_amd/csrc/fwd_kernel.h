@@ -63,8 +63,14 @@ struct KParams {
   int32_t dmin, dmax, pfx;
   const int64_t* doc_ids;
   int64_t doc_stride;
-  const int64_t* doc_table;  // [B][ceil(L/kDocBlock)][2] = (min, max)
-  int32_t doc_blocks;
+  // Document masks: the key tiles each query tile visits, listed by doc_lists_kernel before the launch (the lists are
+  // the same for every head): per (batch, query tile) doc_list_stride words, word 0 = number of entries, then the
+  // entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).
+  const uint32_t* doc_lists;
+  int32_t doc_list_stride;  // words per (batch, query tile): a multiple of 4, at least n_ktiles + 1
+  // the ids again, written by the same pre-pass as [B][n_ktiles * BN] (positions past Lk repeat the last id), so that
+  // a tile's ids are one aligned run whatever Lk is
+  const int64_t* doc_ids_padded;
   int32_t alibi_heads;
   float softcap;
   const bf16_t* bias[2];
@@ -346,14 +352,19 @@ struct FwdTraits {
   static constexpr int BBYTES = (FEAT & F_BIAS) ? BM * BN * 2 : 0;
   static constexpr int B_PER_T = (FEAT & F_BIAS) ? RW * BN / 8 / 64 : 0;  // 16-byte transfers per lane per tile
   static_assert(!(FEAT & F_BIAS) || ((RW * BN / 8) % 64 == 0 && NS == 2), "staged bias: whole transfers, ring of two");
-  // LDS: K tiles [NS], V tiles [NS], bias tiles [NS], 16 bytes of counters, then the tile list (4 bytes per key tile,
-  // sized at launch)
+  // LDS: K tiles [NS], V tiles [NS], bias tiles [NS], row-bias images [NS], document-id images [NS], then (document
+  // masks only) the tile list, sized at launch: 4 bytes per entry plus the count, rounded up to whole wave transfers
   // A second, row-broadcast operand (query stride 0, e.g. a key-padding bias) is staged as one row of BN keys per wave
   // and slot; the transfer is a whole 1 KiB wave transfer whose lanes repeat the row.
   static constexpr int RBYTES = (FEAT & F_BIAS) ? NW * 1024 : 0;
   static constexpr int R_PER_T = (FEAT & F_BIAS) ? 1 : 0;
+  // Document ids of a tile's keys ride with its V tile: per ring slot and wave a private 1 KiB image (one wave
+  // transfer: BN int64 ids, repeated to fill it).
+  static constexpr int IBYTES = (FEAT & F_DOC) ? NW * 1024 : 0;
+  static constexpr int I_PER_T = (FEAT & F_DOC) ? 1 : 0;
+  static_assert(!(FEAT & F_DOC) || BN * 8 <= 1024, "the ids of one tile fit one wave transfer");
   static constexpr int K_OFF = 0, V_OFF = NS * KBYTES, B_OFF = NS * (KBYTES + VBYTES), R_OFF = B_OFF + NS * BBYTES,
-                       META_OFF = R_OFF + NS * RBYTES, LIST_OFF = META_OFF + 16;
+                       I_OFF = R_OFF + NS * RBYTES, LIST_OFF = I_OFF + NS * IBYTES;
   static constexpr int LDS_FIXED_BYTES = LIST_OFF;
 };
 
@@ -383,10 +394,9 @@ void fwd_kernel(const KParams p) {
   using LV = TileLayout<DV>;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // tile list: one entry per key tile that is not empty for the whole workgroup, in key order:
-  // bits 0-15 tile index, bits 16.. two class bits per wave
-  int* meta = reinterpret_cast<int*>(smem + T::META_OFF);  // [0] = number of list entries
-  uint32_t* tlist = reinterpret_cast<uint32_t*>(smem + T::LIST_OFF);
+  // tile list (document masks): word 0 = number of entries, then one entry per key tile that is not empty for the
+  // whole workgroup, in key order: bits 0-15 tile index, bits 16.. two class bits per wave
+  const uint32_t* tlist = reinterpret_cast<const uint32_t*>(smem + T::LIST_OFF) + 1;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
@@ -426,58 +436,14 @@ void fwd_kernel(const KParams p) {
   // tile is classified for every wave and the non-empty ones are compacted into the LDS tile list.
   int n_list = 0, t_lo = 0;
   if constexpr (kDoc) {
-    {
-      const int64_t* dtab = kDoc ? p.doc_table + (int64_t)batch * p.doc_blocks * 2 : nullptr;
-      int64_t qmn[NW], qmx[NW];
-      if constexpr (kDoc) {
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-          int a = q0 + w * RW, b = min(a + RW, p.Lq);
-          qmn[w] = 0;
-          qmx[w] = 0;
-          if (a < b) doc_range(dtab, a, b, qmn[w], qmx[w]);
-        }
-      }
-      for (int t = tid; t < nk; t += NT) {
-        const int k0 = t * BN, k1 = min(k0 + BN, p.Lk);
-        int64_t kmn = 0, kmx = 0;
-        if constexpr (kDoc) doc_range(dtab, k0, k1, kmn, kmx);
-        unsigned c = 0;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-          int a = q0 + w * RW, b = min(a + RW, p.Lq);
-          int cw = TILE_EMPTY;
-          if (a < b) {
-            cw = classify_positional(p.mask_kind, a, b, k0, k1, p.window, p.prefix);
-            if constexpr (kDoc) {
-              if (kmx < qmn[w] || kmn > qmx[w]) cw = TILE_EMPTY;
-              else if (!(kmn == kmx && qmn[w] == qmx[w] && kmn == qmn[w]) && cw == TILE_FULL) cw = TILE_PARTIAL;
-            }
-            if (cw == TILE_FULL && k0 + BN > p.Lk) cw = TILE_PARTIAL;  // ragged tail: keys >= Lk are masked
-          }
-          c |= (unsigned)cw << (2 * w);
-        }
-        tlist[t] = (c << 16) | (unsigned)t;
-      }
-    }
-    __syncthreads();
-    if (wave == 0) {
-      // in-place compaction by one wave, 64 tiles at a time: an entry never moves to a higher index, and every chunk
-      // is read completely before it is written
-      int count = 0;
-      for (int base = 0; base < nk; base += 64) {
-        const int t = base + lane;
-        const uint32_t e = t < nk ? tlist[t] : 0u;
-        const bool keep = (e >> 16) != 0;
-        const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
-        const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-        if (keep) tlist[pos] = e;
-        count += __builtin_popcountll(m);
-      }
-      if (lane == 0) meta[0] = count;
-    }
-    __syncthreads();
-    n_list = __builtin_amdgcn_readfirstlane(meta[0]);
+    // the list of this (batch, query tile) goes global -> LDS in whole wave transfers (64 chunks of 16 bytes each; chunks
+    // past the end repeat the last one); it is awaited, together with the first K/V transfers' predecessors, right
+    // before the key loop, so that the query loads below run under its latency
+    const int n_chunks = p.doc_list_stride / 4;
+    const uint64_t lbase = uniform_ptr(p.doc_lists + ((int64_t)batch * p.n_qtiles + qt) * p.doc_list_stride);
+    const unsigned lds_l = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::LIST_OFF);
+    for (int c0 = wave * 64; c0 < n_chunks; c0 += NW * 64)
+      dma16(lbase, (unsigned)min(c0 + lane, n_chunks - 1) * 16u, lds_l + c0 * 16);
   } else {
     const int q1 = min(q0 + BM, p.Lq);
     int hi_key = p.Lk - 1, lo_key = 0;  // first / last key position some row of the workgroup may attend
@@ -620,6 +586,7 @@ void fwd_kernel(const KParams p) {
     // LDS byte addresses this wave's transfers of slot 0, first transfer, land at
     const unsigned lds_k = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::K_OFF + wave * 1024);
     const unsigned lds_v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::V_OFF + wave * 1024);
+    const unsigned lds_i = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::I_OFF + wave * 1024);
     unsigned koff[T::K_PER_T], voff[T::V_PER_T];
 #pragma unroll
     for (int it = 0; it < T::K_PER_T; ++it) {
@@ -651,6 +618,11 @@ void fwd_kernel(const KParams p) {
       }
     };
     auto load_v = [&](int t, int slot) FL_INLINE  {
+      if constexpr (kDoc) {
+        // this wave's copy of the tile's key ids: lane l brings ids 2l, 2l + 1 (mod BN)
+        dma16(uniform_ptr(p.doc_ids_padded + ((int64_t)batch * nk + t) * BN), (unsigned)((2 * lane) % BN) * 8u,
+              lds_i + slot * T::IBYTES);
+      }
       const uint64_t base = vbase + (uint64_t)(uint32_t)t * v_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
@@ -882,52 +854,41 @@ void fwd_kernel(const KParams p) {
     // With off = key - kbase a compile-time constant per register, the positional predicate is lo <= off <= hi for
     // per-lane bounds: every mask is one interval of key - q cut at Lk; the prefix-LM mask is the union of two
     // intervals that both start at -inf, i.e. again one (dmin is far below any offset unless a window is set).
-    auto apply_mask = [&](f32x16 (&s)[KB][QB], int t) FL_INLINE {
+    auto apply_mask = [&](f32x16 (&s)[KB][QB], int t, int vslot) FL_INLINE {
       const int k0 = t * BN;
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         const int kbase = k0 + 32 * kb + 4 * h;
         const int t_len = p.Lk - kbase;   // off < t_len   <=> key < Lk
         const int t_pfx = p.pfx - kbase;  // off < t_pfx   <=> key < pfx
-        // the positional test, and one of three document tests: none; one id for the whole block; an id per key
-        auto mask_block = [&](auto doc_mode, int64_t block_doc, const int64_t (&kdoc)[16]) FL_INLINE {
-          constexpr int kMode = decltype(doc_mode)::value;
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            const int rel = kbase - qrow[qb];
-            // off <= hi <=> key < Lk && (key - q <= dmax || key < pfx);  off >= lo <=> key - q >= dmin
-            int hi = min(t_len - 1, max(p.dmax - rel, t_pfx - 1));
-            const int lo = p.dmin - rel;
-            if constexpr (kMode == 1) hi = (block_doc == qdoc[qb]) ? hi : -1;  // another document: nothing passes
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int off = 8 * (i / 4) + (i % 4);
-              bool ok = (off <= hi) & (off >= lo);
-              if constexpr (kMode == 2) ok = ok & (kdoc[i] == qdoc[qb]);
-              s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
-            }
-          }
-        };
+        // Under a document mask the ids of this lane's 16 keys come from the wave's LDS image of the tile's ids (it
+        // arrived with the V tile in ring slot `vslot`): four runs of four consecutive keys.
         int64_t kdoc[16];
         if constexpr (kDoc) {
-          // a 32-key block lies inside one document far more often than not, and the (min, max) table says so with two
-          // scalar loads: only blocks that hold a boundary read their keys' ids one by one.  The two cases do not share
-          // the code that consumes the ids: a wait for those loads placed after the join would run in the common case
-          // too, and would also wait for the K/V transfers in flight.
-          static_assert(kDocBlock == 32, "one table entry per 32-key block of a tile");
-          // (a block that starts past the last key reads the last entry: all of its keys are masked anyway)
-          const int64_t* tb = p.doc_table + ((int64_t)batch * p.doc_blocks + min((k0 + 32 * kb) / kDocBlock, p.doc_blocks - 1)) * 2;
-          const int64_t bmn = tb[0], bmx = tb[1];
-          if (bmn == bmx) {
-            mask_block(std::integral_constant<int, 1>{}, bmn, kdoc);
-          } else {
+          typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
+          const unsigned char* il = smem + T::I_OFF + vslot * T::IBYTES + wave * 1024 + (32 * kb + 4 * h) * 8;
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-              kdoc[i] = p.doc_ids[(int64_t)batch * p.doc_stride + min(kbase + 8 * (i / 4) + (i % 4), p.Lk - 1)];
-            mask_block(std::integral_constant<int, 2>{}, 0, kdoc);
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int e2 = 0; e2 < 2; ++e2) {
+              const i64x2 two = *reinterpret_cast<const i64x2*>(il + (8 * g + 2 * e2) * 8);
+              kdoc[4 * g + 2 * e2] = two[0];
+              kdoc[4 * g + 2 * e2 + 1] = two[1];
+            }
+        }
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          const int rel = kbase - qrow[qb];
+          // off <= hi <=> key < Lk && (key - q <= dmax || key < pfx);  off >= lo <=> key - q >= dmin
+          const int hi = min(t_len - 1, max(p.dmax - rel, t_pfx - 1));
+          const int lo = p.dmin - rel;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int off = 8 * (i / 4) + (i % 4);
+            bool ok = (off <= hi) & (off >= lo);
+            if constexpr (kDoc) ok = ok & (kdoc[i] == qdoc[qb]);
+            s[kb][qb][i] = ok ? s[kb][qb][i] : -INFINITY;
           }
-        } else {
-          mask_block(std::integral_constant<int, 0>{}, 0, kdoc);
         }
       }
     };
@@ -1110,10 +1071,12 @@ void fwd_kernel(const KParams p) {
         }
     };
 
+    if constexpr (kDoc) dma_wait<0>();  // the tile list (issued first thing) has landed
     __syncthreads();  // the previous branch (if any) is done with the LDS buffers
+    if constexpr (kDoc) n_list = __builtin_amdgcn_readfirstlane((int)tlist[-1]);
     if (n_list > 0) {
       constexpr int NS = T::NS;
-      constexpr int LPS = T::K_PER_T + T::V_PER_T + T::B_PER_T + T::R_PER_T;  // transfers per thread per step
+      constexpr int LPS = T::K_PER_T + T::V_PER_T + T::B_PER_T + T::R_PER_T + T::I_PER_T;  // transfers per thread per step
       // ent[j] = tile-list entry of list position pos + j (the last entry again past the end of the list).  Entries are
       // read from LDS NS steps before they are needed, so the read latency never shows.
       int pos = 0;
@@ -1139,11 +1102,11 @@ void fwd_kernel(const KParams p) {
 
       // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
       // maxima, and the (rare) rescale.
-      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e) FL_INLINE {
+      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e, int vslot) FL_INLINE {
         const int t = entry_tile(e);
         const bool full = entry_class(e) == TILE_FULL;
         if (!full || !kFastRef) {
-          if (!full) apply_mask(sc, t);
+          if (!full) apply_mask(sc, t, vslot);
           float mx[QB];
           row_max(sc, mx);
           rescale_if_grown(mx, false);
@@ -1165,7 +1128,7 @@ void fwd_kernel(const KParams p) {
           load_b(entry_tile(ent[NS]), slot);  // the bias of this step's tile was consumed at the end of the previous step
         }
         if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
-        settle(sc, ent[0]);
+        settle(sc, ent[0], slot);
         ex8 pf[QB][2 * KB];
         // Raised issue priority while this wave has matrix work: of the two waves sharing a SIMD, the one that is in
         // its MFMA phase wins the issue port, which drives the pair into opposite phases (one on the matrix pipe while
@@ -1212,11 +1175,11 @@ void fwd_kernel(const KParams p) {
         ex8 pf[QB][2 * KB];
         ex8 vfirst[DVB];
         if constexpr (slot % 2 == 0) {
-          settle(s_a, ent[0]);
+          settle(s_a, ent[0], slot);
           weights_checked(s_a, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot,
                           entry_tile(ent[0]));
         } else {
-          settle(s_b, ent[0]);
+          settle(s_b, ent[0], slot);
           weights_checked(s_b, pf, kFastRef && entry_class(ent[0]) == TILE_FULL, std::false_type{}, vfirst, slot,
                           entry_tile(ent[0]));
         }

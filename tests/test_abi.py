@@ -130,15 +130,23 @@ def test_workspace_size_for_document_masks(lib):
     p = good_params(B=3, L=1000)
     assert lib.fl_workspace_bytes(C.byref(p)) == 0
     p.mask_kind = _ffi.MASK_DOCUMENT_CAUSAL
-    assert lib.fl_workspace_bytes(C.byref(p)) == 3 * ((1000 + 31) // 32) * 16
-    p.doc_ids, p.workspace, p.workspace_bytes = 0x50000, 0x80000, 3 * 32 * 16
+    # (min, max) table per 32 positions + per (batch, query tile) the list of key tiles (count + entries, rounded up to
+    # 4 words) + the ids padded to whole key tiles, for the tile shape the library reports for this call
+    shape = _ffi.plan(good_params(B=3, L=1000))
+    bm, bn = shape["rows_per_workgroup"], shape["keys_per_tile"]
+    nq, nk = -(-1000 // bm), -(-1000 // bn)
+    need = 3 * ((1000 + 31) // 32) * 16 + 3 * nq * ((nk + 1 + 3) // 4 * 4) * 4 + 3 * nk * bn * 8
+    assert lib.fl_workspace_bytes(C.byref(p)) == need
+    p.doc_ids, p.workspace, p.workspace_bytes = 0x50000, 0x80000, need
     assert rc(lib, p) == 0, _ffi.last_error()
     p.workspace_bytes -= 1
     assert rc(lib, p) == -6
+    p.workspace, p.workspace_bytes = 0x80008, need
+    assert rc(lib, p) == -7  # 16-byte alignment
 
 
 def test_too_many_keys_is_an_error_not_a_fault(lib):
-    # the tile list (4 bytes per key tile) must fit in LDS next to the K/V ring
+    # key tiles are numbered in 16 bits
     p = good_params(B=1, Hq=1, Hkv=1, L=1 << 26, D=64)
     assert rc(lib, p) == -2 and "maximum" in _ffi.last_error()
     p = good_params(B=1, Hq=1, Hkv=1, L=1 << 20, D=64)

@@ -112,14 +112,14 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_plan.argtypes = [C.POINTER(FlAttnParams), C.POINTER(C.c_int64)]
     lib.fl_attn_fwd.restype = C.c_int
     lib.fl_attn_fwd.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
-    lib.fl_attn_fwd_static.restype = C.c_int
-    lib.fl_attn_fwd_static.argtypes = [C.POINTER(FlAttnParams), C.c_void_p]
     lib.fl_static_scratch_bytes.restype = C.c_uint64
     lib.fl_bwd_params_sizeof.restype = C.c_uint64
     lib.fl_attn_bwd_validate.restype = C.c_int
     lib.fl_attn_bwd_validate.argtypes = [C.POINTER(FlAttnBwdParams)]
     lib.fl_attn_bwd.restype = C.c_int
     lib.fl_attn_bwd.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
+    lib.fl_attn_bwd_static.restype = C.c_int
+    lib.fl_attn_bwd_static.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
     lib.fl_ipa_pack.restype = C.c_int
     lib.fl_ipa_pack.argtypes = [C.POINTER(FlIpaPackParams), C.c_void_p]
     lib.fl_probe_mfma_rate.restype = C.c_int
@@ -288,7 +288,6 @@ def attn_fwd(
     lse: Optional[torch.Tensor] = None,
     dropout_p: float = 0.0,
     dropout_seed: int = 0,
-    static_scratch: bool = False,
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
@@ -298,8 +297,6 @@ def attn_fwd(
     `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
     `dropout_p` > 0 drops softmax weights (torch.nn.functional.dropout semantics) by a hash of (`dropout_seed`, batch,
     head, query, key); positional masks and GQA only.
-    `static_scratch` goes through `fl_attn_fwd_static`: no workspace is allocated here, the library's own static
-    device array serves as scratch (calls that may overlap on one GPU must not both use it).
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -335,12 +332,11 @@ def attn_fwd(
             attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
                      doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
                      gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
-                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only, static_scratch=static_scratch)
+                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed,
-                           alloc_workspace=validate_only or not static_scratch)
+                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed)
     if lse is not None:
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
             raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")
@@ -350,8 +346,7 @@ def attn_fwd(
         return out
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream().cuda_stream
-        entry = lib.fl_attn_fwd_static if static_scratch else lib.fl_attn_fwd
-        _check(entry(C.byref(p), C.c_void_p(stream)))
+        _check(lib.fl_attn_fwd(C.byref(p), C.c_void_p(stream)))
     # tensors in `keep` were last used on the current stream; the caching allocator orders their reuse after it
     del keep
     return out
@@ -360,9 +355,13 @@ def attn_fwd(
 def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor, dout: torch.Tensor,
              *, scale: Optional[float] = None, mask_kind: int = MASK_NONE, window: int = 0, prefix: int = 0,
              doc_ids: Optional[torch.Tensor] = None, alibi_heads: int = 0, softcap: float = 0.0,
-             validate_only: bool = False, dropout_p: float = 0.0, dropout_seed: int = 0):
+             validate_only: bool = False, dropout_p: float = 0.0, dropout_seed: int = 0, static_scratch: bool = False,
+             grads: Optional[Sequence[torch.Tensor]] = None):
     """Gradients (dq, dk, dv) of `attn_fwd` called with the same arguments (dropout rate and seed included); `out` and `lse` are what that call
-    returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream."""
+    returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream.
+    `grads` = (dq, dk, dv) receives the results when given.  `static_scratch` goes through `fl_attn_bwd_static`: nothing
+    is allocated here beyond the results, the library's own static device array serves as scratch (calls that may
+    overlap on one GPU must not both use it)."""
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
         _require_gpu_half(name, t, q if isinstance(q, torch.Tensor) and q.dtype in _HALF_TYPES else None)
@@ -376,14 +375,23 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
         raise ValueError("lse must be the contiguous float32 [B, Hq, Lq] tensor the forward filled")
     fwd, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                             (), None, False, 0.0, None, dropout_p, dropout_seed)
+                             (), None, False, 0.0, None, dropout_p, dropout_seed,
+                             alloc_workspace=validate_only or not static_scratch)
     fwd.lse = lse.data_ptr()
-    dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
-        torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
-    delta = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
+    if grads is not None:
+        dq, dk, dv = grads
+        for g, like in ((dq, q), (dk, k), (dv, v)):
+            if tuple(g.shape) != tuple(like.shape) or g.dtype != like.dtype or g.device != like.device or g.stride(-1) != 1:
+                raise ValueError("grads must match q, k, v in shape, dtype and device")
+    else:
+        dq, dk, dv = torch.empty_like(q, memory_format=torch.contiguous_format), \
+            torch.empty_like(k, memory_format=torch.contiguous_format), torch.empty_like(v, memory_format=torch.contiguous_format)
+    use_static = static_scratch and not validate_only
+    delta = None if use_static else torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
     b = FlAttnBwdParams()
     b.fwd = fwd
-    b.dout, b.dq, b.dk, b.dv, b.delta = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr()
+    b.dout, b.dq, b.dk, b.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    b.delta = None if delta is None else delta.data_ptr()
     b.dout_strides[:] = _strides4(dout)
     b.dq_strides[:] = _strides4(dq)
     b.dk_strides[:] = _strides4(dk)
@@ -392,7 +400,8 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
         _check(lib.fl_attn_bwd_validate(C.byref(b)))
         return dq, dk, dv
     with torch.cuda.device(q.device):
-        _check(lib.fl_attn_bwd(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        entry = lib.fl_attn_bwd_static if use_static else lib.fl_attn_bwd
+        _check(entry(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     del keep, delta
     return dq, dk, dv
 

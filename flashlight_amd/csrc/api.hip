@@ -18,52 +18,111 @@ static __global__ void doc_table_kernel(const int64_t* ids, int64_t ids_stride, 
   int b = i / nblocks, blk = i % nblocks;
   const int64_t* p = ids + (int64_t)b * ids_stride;
   int p0 = blk * kDocBlock, p1 = min(L, p0 + kDocBlock);
-  int64_t mn = p[p0], mx = mn;
-  for (int j = p0 + 1; j < p1; ++j) {
-    int64_t x = p[j];
-    mn = x < mn ? x : mn;
-    mx = x > mx ? x : mx;
+  // (the loads are independent of one another: unrolled, they are all in flight together instead of one round trip
+  // to memory each; positions past the end repeat the last one)
+  int64_t x[kDocBlock];
+#pragma unroll
+  for (int j = 0; j < kDocBlock; ++j) x[j] = p[min(p0 + j, p1 - 1)];
+  int64_t mn = x[0], mx = x[0];
+#pragma unroll
+  for (int j = 1; j < kDocBlock; ++j) {
+    mn = x[j] < mn ? x[j] : mn;
+    mx = x[j] > mx ? x[j] : mx;
   }
   table[2 * (int64_t)i] = mn;
   table[2 * (int64_t)i + 1] = mx;
 }
 
-// Forward pre-pass for document masks, one workgroup of 256 threads per (batch, query tile of `bm` rows): lists the key
-// tiles (of `bn` keys) that some row of the query tile attends, with the class of each for every wave (`rw` rows per
-// wave), from the (min, max) table; the lists are the same for every head.  Output per workgroup: word 0 = number of
-// entries, then the entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).  Also writes
-// the workgroup's share of the padded copy of the ids ([B][nk * bn], positions past L repeat the last id).
-static __global__ __launch_bounds__(256) void doc_lists_kernel(const int64_t* ids, int64_t ids_stride, const int64_t* table,
-                                                               int blocks, int L, int mask_kind, int bm, int rw, int bn,
-                                                               int n_qtiles, int nk, int list_stride, uint32_t* lists,
-                                                               int64_t* ids_padded) {
-  extern __shared__ uint32_t tl[];  // nk words
-  const int tid = threadIdx.x, lane = tid % 64;
+// (min, max) over a wave of one int64 per lane, wave-uniform.  Nearly every 32- or 64-position run lies inside one
+// document, so "all equal to the first lane's" is tested with one ballot before the reduction.
+static __device__ __forceinline__ void wave_id_range(int64_t x, int64_t& mn, int64_t& mx) {
+  const int64_t first = uniform_i64(x);
+  mn = mx = first;
+  if (__builtin_amdgcn_ballot_w64(x != first) != 0) {
+    int64_t a = x, b = x;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const int64_t a2 = __shfl_xor(a, d, 64), b2 = __shfl_xor(b, d, 64);
+      a = a2 < a ? a2 : a;
+      b = b2 > b ? b2 : b;
+    }
+    mn = uniform_i64(a);
+    mx = uniform_i64(b);
+  }
+}
+
+// Forward pre-pass for document masks, one workgroup of 1024 threads per (batch, query tile of `bm` rows), straight from
+// the ids: lists the key tiles (of `bn` keys) that some row of the query tile attends, with the class of each for every
+// wave of the forward (`rw` rows per wave): EMPTY when the id ranges of the tile's keys and the wave's rows do not meet,
+// FULL when both are the same single id and the positional part of the mask agrees, PARTIAL otherwise.  Valid for
+// arbitrary (unsorted, negative) ids.  The lists are the same for every head.  Output per workgroup: word 0 = number of
+// entries, then the entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).
+// Three phases: a wave per key tile reads its ids with one coalesced load and leaves their (min, max) in LDS (every
+// load of a wave is in flight before the first is looked at: the kernel is a chain of round trips to memory with little
+// to do in between); a thread per key tile classifies it for every wave; one wave compacts the non-empty entries.
+static __global__ __launch_bounds__(1024) void doc_lists_kernel(const int64_t* ids, int64_t ids_stride, int L, int mask_kind,
+                                                                int bm, int rw, int bn, int n_qtiles, int nk, int list_stride,
+                                                                uint32_t* lists) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  int64_t* krange = reinterpret_cast<int64_t*>(lds_raw);                // [nk][2] = (min, max) id of a key tile
+  uint32_t* tl = reinterpret_cast<uint32_t*>(lds_raw + (size_t)nk * 16);  // [nk] uncompacted entries
+  __shared__ int64_t qrange[16];  // (min, max) id of the rows of each of up to 8 waves of the forward
+  constexpr int kWaves = 16, kBatch = 16;
+  const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int b = blockIdx.x / n_qtiles, qt = blockIdx.x % n_qtiles;
   const int nw = bm / rw, q0 = qt * bm;
-  const int64_t* dtab = table + (int64_t)b * blocks * 2;
-  for (int i = tid; i < bm; i += 256) {
-    const int pos = q0 + i;
-    if (pos < nk * bn) ids_padded[(int64_t)b * nk * bn + pos] = ids[(int64_t)b * ids_stride + min(pos, L - 1)];
+  const int64_t* idb = ids + (int64_t)b * ids_stride;
+  // rows past L repeat the last row (a wave without valid rows is EMPTY for every tile whatever its range)
+  const int64_t qid = idb[min(q0 + min(wave, nw - 1) * rw + lane % rw, L - 1)];
+  // key tiles some row may attend under the positional part of the mask: all of them, or those up to the diagonal
+  const int t_end = mask_kind == MASK_DOC_CAUSAL ? min(nk, (min(q0 + bm, L) - 1) / bn + 1) : nk;
+  const int nj = (bn + 63) / 64;  // loads per lane that cover one tile's ids
+  for (int t0 = wave; t0 < t_end || t0 == wave; t0 += kWaves * kBatch) {
+    int64_t lo[kBatch], hi[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int k0 = min(t0 + kWaves * u, t_end - 1) * bn;
+      lo[u] = hi[u] = idb[min(k0 + lane % bn, L - 1)];
+      for (int j = 1; j < nj; ++j) {
+        const int64_t x = idb[min(k0 + j * 64 + lane, L - 1)];
+        lo[u] = x < lo[u] ? x : lo[u];
+        hi[u] = x > hi[u] ? x : hi[u];
+      }
+    }
+    if (t0 == wave) {  // (every wave passes here exactly once)
+      int64_t mn, mx;
+      wave_id_range(qid, mn, mx);
+      if (lane == 0 && wave < nw) {
+        qrange[2 * wave] = mn;
+        qrange[2 * wave + 1] = mx;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int t = t0 + kWaves * u;
+      if (t >= t_end) break;
+      int64_t kmn, kmx, unused;
+      wave_id_range(lo[u], kmn, unused);
+      if (nj > 1) wave_id_range(hi[u], unused, kmx); else kmx = unused;
+      if (lane == 0) {
+        krange[2 * t] = kmn;
+        krange[2 * t + 1] = kmx;
+      }
+    }
   }
-  int64_t qmn[8], qmx[8];
-  for (int w = 0; w < 8; ++w) {
-    qmn[w] = qmx[w] = 0;
-    const int a = q0 + w * rw, e = min(a + rw, L);
-    if (w < nw && a < e) doc_range(dtab, a, e, qmn[w], qmx[w]);
-  }
-  for (int t = tid; t < nk; t += 256) {
+  __syncthreads();
+  for (int t = tid; t < t_end; t += 1024) {
     const int k0 = t * bn, k1 = min(k0 + bn, L);
-    int64_t kmn, kmx;
-    doc_range(dtab, k0, k1, kmn, kmx);
+    const int64_t kmn = krange[2 * t], kmx = krange[2 * t + 1];
     unsigned c = 0;
     for (int w = 0; w < nw; ++w) {
       const int a = q0 + w * rw, e = min(a + rw, L);
+      const int64_t qmn = qrange[2 * w], qmx = qrange[2 * w + 1];
       int cw = TILE_EMPTY;
       if (a < e) {
         cw = classify_positional(mask_kind, a, e, k0, k1, 0, 0);
-        if (kmx < qmn[w] || kmn > qmx[w]) cw = TILE_EMPTY;
-        else if (!(kmn == kmx && qmn[w] == qmx[w] && kmn == qmn[w]) && cw == TILE_FULL) cw = TILE_PARTIAL;
+        if (kmx < qmn || kmn > qmx) cw = TILE_EMPTY;
+        else if (!(kmn == kmx && qmn == qmx && kmn == qmn) && cw == TILE_FULL) cw = TILE_PARTIAL;
         if (cw == TILE_FULL && k0 + bn > L) cw = TILE_PARTIAL;  // ragged tail: keys >= L are masked
       }
       c |= (unsigned)cw << (2 * w);
@@ -71,12 +130,12 @@ static __global__ __launch_bounds__(256) void doc_lists_kernel(const int64_t* id
     tl[t] = (c << 16) | (unsigned)t;
   }
   __syncthreads();
-  if (tid < 64) {
+  if (wave == 0) {
     uint32_t* out = lists + (int64_t)blockIdx.x * list_stride;
     int count = 0;
-    for (int base = 0; base < nk; base += 64) {
+    for (int base = 0; base < t_end; base += 64) {
       const int t = base + lane;
-      const uint32_t e = t < nk ? tl[t] : 0u;
+      const uint32_t e = t < t_end ? tl[t] : 0u;
       const bool keep = (e >> 16) != 0;
       const uint64_t m = __builtin_amdgcn_ballot_w64(keep);
       const int pos = count + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
@@ -89,7 +148,7 @@ static __global__ __launch_bounds__(256) void doc_lists_kernel(const int64_t* id
 
 }  // namespace fl
 
-// Scratch of the entry point that allocates nothing (fl_attn_fwd_static): one copy per GPU the library runs on, held
+// Scratch of the entry point that allocates nothing (fl_attn_bwd_static): one copy per GPU the library runs on, held
 // until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels and memory calls
 // take the device address that call returns (static_scratch_ptr below).
 constexpr size_t kStaticScratchBytes = (size_t)FL_STATIC_SCRATCH_BYTES;
@@ -182,14 +241,12 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
 }
 
 // Device scratch of a document-mask call, in this order (every part a multiple of 16 bytes):
-//   table   [B][ceil(L / 32)][2] int64   (min, max) id per 32 positions (forward pre-pass and backward)
-//   lists   [B][query tiles][stride] u32 the key tiles each query tile visits (forward)
-//   ids     [B][key tiles * bn] int64    the ids padded to whole key tiles (forward)
-// bm / bn: query rows per workgroup and keys per tile of the forward instance.
+//   table   [B][ceil(L / 32)][2] int64   (min, max) id per 32 positions (backward)
+//   lists   [B][query tiles][stride] u32 the key tiles each query tile visits (forward; bm / bn = query rows per
+//                                        workgroup and keys per tile of the forward instance)
 struct DocScratch {
   int64_t blocks, n_qtiles, nk, list_stride;
-  uint64_t table_bytes, lists_bytes, ids_bytes;
-  uint64_t total() const { return table_bytes + lists_bytes + ids_bytes; }
+  uint64_t table_bytes, lists_bytes;
 };
 DocScratch doc_scratch(int64_t B, int64_t L, int64_t bm, int64_t bn) {
   DocScratch d;
@@ -199,7 +256,6 @@ DocScratch doc_scratch(int64_t B, int64_t L, int64_t bm, int64_t bn) {
   d.list_stride = (d.nk + 1 + 3) / 4 * 4;
   d.table_bytes = (uint64_t)B * d.blocks * 2 * sizeof(int64_t);
   d.lists_bytes = (uint64_t)B * d.n_qtiles * d.list_stride * sizeof(uint32_t);
-  d.ids_bytes = (uint64_t)B * d.nk * bn * sizeof(int64_t);
   return d;
 }
 
@@ -344,9 +400,11 @@ uint64_t fl_params_sizeof(void) { return sizeof(fl_attn_params); }
 
 uint64_t fl_workspace_bytes(const fl_attn_params* p) {
   if (!p || !is_doc(p->mask_kind) || p->B <= 0 || p->Lk <= 0) return 0;
-  // tile shape of the instance the forward would run (the largest shapes compiled, if the call names no valid one)
+  // tile shape of the instance the forward would run (the largest lists any compiled shape needs, if the call names no
+  // valid one)
   const fl::Instance* in = select_instance(p);
-  return doc_scratch(p->B, p->Lk, in ? (int64_t)in->rw * in->nw : 128, in ? in->bn : 32).total();
+  const DocScratch d = doc_scratch(p->B, p->Lk, in ? (int64_t)in->rw * in->nw : 64, in ? in->bn : 32);
+  return d.table_bytes + d.lists_bytes;
 }
 
 int fl_attn_validate(const fl_attn_params* p) { return validate(p, nullptr); }
@@ -460,49 +518,18 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
 
   if (is_doc(p->mask_kind)) {
     const DocScratch d = doc_scratch(p->B, p->Lk, bm, in->bn);
-    const int total = p->B * (int)d.blocks;
-    unsigned char* ws = static_cast<unsigned char*>(p->workspace);
-    int64_t* table = reinterpret_cast<int64_t*>(ws);
-    uint32_t* lists = reinterpret_cast<uint32_t*>(ws + d.table_bytes);
-    int64_t* ids_padded = reinterpret_cast<int64_t*>(ws + d.table_bytes + d.lists_bytes);
-    hipLaunchKernelGGL(fl::doc_table_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, p->doc_ids, p->doc_stride,
-                       p->Lk, (int)d.blocks, total, table);
+    uint32_t* lists = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(p->workspace) + d.table_bytes);
+    hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(1024), (size_t)kp.n_ktiles * 20, stream,
+                       p->doc_ids, p->doc_stride, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles, kp.n_ktiles,
+                       (int)d.list_stride, lists);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail((int)e, "doc_table_kernel launch failed: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(256), (size_t)kp.n_ktiles * 4, stream,
-                       p->doc_ids, p->doc_stride, table, (int)d.blocks, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles,
-                       kp.n_ktiles, (int)d.list_stride, lists, ids_padded);
-    e = hipGetLastError();
     if (e != hipSuccess) return fail((int)e, "doc_lists_kernel launch failed: %s", hipGetErrorString(e));
     kp.doc_lists = lists;
     kp.doc_list_stride = (int)d.list_stride;
-    kp.doc_ids_padded = ids_padded;
   }
   hipError_t e = in->launch(kp, grid, (int)lds_bytes_for(in, p), stream);
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));
   return 0;
-}
-
-int fl_attn_fwd_static(const fl_attn_params* p, void* stream) {
-  if (!p) return fail(FL_ERR_NULL, "params is null");
-  fl_attn_params q = *p;
-  const uint64_t need = fl_workspace_bytes(&q);
-  if (need > kStaticScratchBytes)
-    return fail(FL_ERR_WORKSPACE,
-                "fl_attn_fwd_static: this call needs %llu bytes of scratch, the library's static scratch holds %llu "
-                "(document masks up to B * ceil(Lk / 32) = %llu blocks); use fl_attn_fwd with a caller workspace",
-                (unsigned long long)need, (unsigned long long)kStaticScratchBytes,
-                (unsigned long long)(kStaticScratchBytes / 16));
-  q.workspace = nullptr;
-  q.workspace_bytes = 0;
-  if (need) {
-    void* ptr = nullptr;
-    int rc = static_scratch_ptr(&ptr);
-    if (rc) return rc;
-    q.workspace = ptr;
-    q.workspace_bytes = kStaticScratchBytes;
-  }
-  return fl_attn_fwd(&q, stream);
 }
 
 uint64_t fl_static_scratch_bytes(void) { return kStaticScratchBytes; }
@@ -626,6 +653,29 @@ int fl_attn_bwd(const fl_attn_bwd_params* b, void* stream_) {
   e = in->launch_dkv(bp, stream);
   if (e != hipSuccess) return fail((int)e, "backward: launch of the dK/dV kernel failed: %s", hipGetErrorString(e));
   return 0;
+}
+
+int fl_attn_bwd_static(const fl_attn_bwd_params* b, void* stream) {
+  if (!b) return fail(FL_ERR_NULL, "params is null");
+  fl_attn_bwd_params c = *b;
+  const fl_attn_params* p = &b->fwd;
+  if (p->B <= 0 || p->Hq <= 0 || p->Lq <= 0) return fail(FL_ERR_SHAPE, "sizes must be positive");
+  // layout of the static scratch: the row sums (B * Hq * Lq floats, rounded up to 256 bytes), then the document table
+  const uint64_t delta_bytes = ((uint64_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256;
+  const uint64_t table_bytes = fl_workspace_bytes(p);  // (the forward's lists, part of this figure, stay unused here)
+  if (delta_bytes + table_bytes > kStaticScratchBytes)
+    return fail(FL_ERR_WORKSPACE,
+                "fl_attn_bwd_static: this call needs %llu bytes of scratch (4 per query row of every head, plus 16 per 32 "
+                "positions under a document mask), the library's static scratch holds %llu; use fl_attn_bwd with "
+                "caller-provided delta and workspace",
+                (unsigned long long)(delta_bytes + table_bytes), (unsigned long long)kStaticScratchBytes);
+  void* ptr = nullptr;
+  int rc = static_scratch_ptr(&ptr);
+  if (rc) return rc;
+  c.delta = static_cast<float*>(ptr);
+  c.fwd.workspace = table_bytes ? static_cast<unsigned char*>(ptr) + delta_bytes : nullptr;
+  c.fwd.workspace_bytes = table_bytes;
+  return fl_attn_bwd(&c, stream);
 }
 
 }  // extern "C"

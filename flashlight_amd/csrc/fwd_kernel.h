@@ -68,9 +68,6 @@ struct KParams {
   // entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).
   const uint32_t* doc_lists;
   int32_t doc_list_stride;  // words per (batch, query tile): a multiple of 4, at least n_ktiles + 1
-  // the ids again, written by the same pre-pass as [B][n_ktiles * BN] (positions past Lk repeat the last id), so that
-  // a tile's ids are one aligned run whatever Lk is
-  const int64_t* doc_ids_padded;
   int32_t alibi_heads;
   float softcap;
   const bf16_t* bias[2];
@@ -167,6 +164,10 @@ __device__ __forceinline__ uint64_t uniform_ptr(const void* ptr) {
   const uint64_t b = reinterpret_cast<uint64_t>(ptr);
   return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
          ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+}
+__device__ __forceinline__ int64_t uniform_i64(int64_t x) {
+  return (int64_t)((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)x) |
+                   ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)x >> 32)) << 32));
 }
 __device__ __forceinline__ void dma16(uint64_t gbase_uniform, unsigned voff, unsigned lds_base) {
   const unsigned lds_base_uniform = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_base);
@@ -358,11 +359,11 @@ struct FwdTraits {
   // and slot; the transfer is a whole 1 KiB wave transfer whose lanes repeat the row.
   static constexpr int RBYTES = (FEAT & F_BIAS) ? NW * 1024 : 0;
   static constexpr int R_PER_T = (FEAT & F_BIAS) ? 1 : 0;
-  // Document ids of a tile's keys ride with its V tile: per ring slot and wave a private 1 KiB image (one wave
-  // transfer: BN int64 ids, repeated to fill it).
-  static constexpr int IBYTES = (FEAT & F_DOC) ? NW * 1024 : 0;
-  static constexpr int I_PER_T = (FEAT & F_DOC) ? 1 : 0;
-  static_assert(!(FEAT & F_DOC) || BN * 8 <= 1024, "the ids of one tile fit one wave transfer");
+  // Document ids of a tile's keys ride with its V tile: per ring slot and wave a private image of the BN int64 ids,
+  // brought by transfers of 4 bytes per lane (any alignment, exact clamping at the ragged end).
+  static constexpr int I_PER_T = (FEAT & F_DOC) ? BN * 8 / 256 : 0;  // transfers per tile
+  static constexpr int IBYTES = (FEAT & F_DOC) ? NW * BN * 8 : 0;
+  static_assert(!(FEAT & F_DOC) || (BN * 8) % 256 == 0, "whole transfers of 64 dwords");
   static constexpr int K_OFF = 0, V_OFF = NS * KBYTES, B_OFF = NS * (KBYTES + VBYTES), R_OFF = B_OFF + NS * BBYTES,
                        I_OFF = R_OFF + NS * RBYTES, LIST_OFF = I_OFF + NS * IBYTES;
   static constexpr int LDS_FIXED_BYTES = LIST_OFF;
@@ -586,7 +587,7 @@ void fwd_kernel(const KParams p) {
     // LDS byte addresses this wave's transfers of slot 0, first transfer, land at
     const unsigned lds_k = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::K_OFF + wave * 1024);
     const unsigned lds_v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::V_OFF + wave * 1024);
-    const unsigned lds_i = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::I_OFF + wave * 1024);
+    const unsigned lds_i = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::I_OFF + wave * (BN * 8));
     unsigned koff[T::K_PER_T], voff[T::V_PER_T];
 #pragma unroll
     for (int it = 0; it < T::K_PER_T; ++it) {
@@ -619,9 +620,14 @@ void fwd_kernel(const KParams p) {
     };
     auto load_v = [&](int t, int slot) FL_INLINE  {
       if constexpr (kDoc) {
-        // this wave's copy of the tile's key ids: lane l brings ids 2l, 2l + 1 (mod BN)
-        dma16(uniform_ptr(p.doc_ids_padded + ((int64_t)batch * nk + t) * BN), (unsigned)((2 * lane) % BN) * 8u,
-              lds_i + slot * T::IBYTES);
+        // this wave's copy of the tile's key ids, one dword per lane and transfer; keys past Lk repeat the last id
+        const uint64_t ibase = uniform_ptr(p.doc_ids + (int64_t)batch * p.doc_stride + (int64_t)t * BN);
+        const int last = p.Lk - 1 - t * BN;
+#pragma unroll
+        for (int it = 0; it < T::I_PER_T; ++it) {
+          const int d = 64 * it + lane;
+          dma4(ibase, (unsigned)(min(d / 2, last) * 8 + (d % 2) * 4), lds_i + slot * T::IBYTES + it * 256);
+        }
       }
       const uint64_t base = vbase + (uint64_t)(uint32_t)t * v_tile_bytes;
       if (t * BN + BN <= p.Lk) {
@@ -866,7 +872,7 @@ void fwd_kernel(const KParams p) {
         int64_t kdoc[16];
         if constexpr (kDoc) {
           typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
-          const unsigned char* il = smem + T::I_OFF + vslot * T::IBYTES + wave * 1024 + (32 * kb + 4 * h) * 8;
+          const unsigned char* il = smem + T::I_OFF + vslot * T::IBYTES + wave * (BN * 8) + (32 * kb + 4 * h) * 8;
 #pragma unroll
           for (int g = 0; g < 4; ++g)
 #pragma unroll

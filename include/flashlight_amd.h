@@ -100,7 +100,8 @@ typedef struct fl_attn_params {
   int32_t dtype; /* element type of q, k, v, o and gate: FL_BF16 or FL_F16 (the reference's typing admits both,
                   * monkeypatch/fusion/_reduction.py:55-57) */
 
-  /* Scratch for the document-mask tile table; size from fl_workspace_bytes(); may be NULL otherwise. */
+  /* Scratch of document-mask calls (the forward's lists of key tiles per query tile, the backward's table of id
+   * ranges); size from fl_workspace_bytes(), 16-byte aligned; may be NULL otherwise. */
   void* workspace;
   uint64_t workspace_bytes;
 
@@ -139,26 +140,12 @@ const char* fl_last_error(void);
 /* Host-only argument check: the same validation fl_attn_fwd runs before it launches.  Touches no GPU. */
 int fl_attn_validate(const fl_attn_params* p);
 
-/* Bytes of device scratch fl_attn_fwd needs for *p (0 unless a document mask is used). */
+/* Bytes of device scratch fl_attn_fwd and fl_attn_bwd need in `workspace` for *p (0 unless a document mask is used). */
 uint64_t fl_workspace_bytes(const fl_attn_params* p);
 
 /* Runs the fused forward on hipStream_t `stream` (NULL = default stream).
  * Replaces torch.compile(fn)(q, k, v, ...) for the functions of attention_variants/. */
 int fl_attn_fwd(const fl_attn_params* p, void* stream);
-
-/* fl_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as fl_attn_fwd,
- * except that p->workspace / p->workspace_bytes are ignored: the scratch a document mask needs lives in a static
- * device array inside the library (FL_STATIC_SCRATCH_BYTES per GPU, held until the process ends), looked up once per
- * device on the first call made with that device current.  A call whose fl_workspace_bytes() exceeds that size returns
- * FL_ERR_WORKSPACE and launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine.  All calls
- * on one GPU share the array: two such calls that may overlap on that GPU (different streams, or different threads)
- * race; calls queued on one stream are ordered and safe.  Nothing in the array needs clearing between calls: each call
- * rewrites the part it reads. */
-#define FL_STATIC_SCRATCH_BYTES (4u << 20)
-int fl_attn_fwd_static(const fl_attn_params* p, void* stream);
-/* FL_STATIC_SCRATCH_BYTES of the loaded library. */
-uint64_t fl_static_scratch_bytes(void);
 
 /* Describes the kernel instance fl_attn_fwd would pick for *p: tile sizes and launch shape.
  * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
@@ -174,7 +161,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
  * receive the gradients (element type fwd.dtype like dout; strides in elements, last stride 1, others multiples of 8).
  * delta: caller-provided scratch of B * Hq * Lq floats; delta and fwd.lse must be 16-byte aligned.
- * fwd.workspace as for the forward (document masks). */
+ * fwd.workspace: fl_workspace_bytes(&fwd) bytes of scratch under a document mask. */
 typedef struct fl_attn_bwd_params {
   fl_attn_params fwd;
   const void* dout;
@@ -195,6 +182,21 @@ int fl_attn_bwd_validate(const fl_attn_bwd_params* p);
 
 /* Launches the three backward kernels (row sums of dO o O, then dQ, then dK and dV) on `stream`. */
 int fl_attn_bwd(const fl_attn_bwd_params* p, void* stream);
+
+/* fl_attn_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight training loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as fl_attn_bwd,
+ * except that p->delta and p->fwd.workspace / workspace_bytes are ignored: the row sums and the document table live in
+ * a static device array inside the library (FL_STATIC_SCRATCH_BYTES per GPU, held until the process ends), whose
+ * address is looked up once per device on the first call made with that device current.  A call that needs more
+ * (4 bytes per query row of every head, rounded up to 256, plus fl_workspace_bytes()) returns FL_ERR_WORKSPACE and
+ * launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine.  All calls on one GPU share the
+ * array: two such calls that may overlap on that GPU (different streams, or different threads) race; calls queued on
+ * one stream are ordered and safe.  Nothing in the array needs clearing between calls: each call rewrites what it
+ * reads. */
+#define FL_STATIC_SCRATCH_BYTES (8u << 20)
+int fl_attn_bwd_static(const fl_attn_bwd_params* p, void* stream);
+/* FL_STATIC_SCRATCH_BYTES of the loaded library. */
+uint64_t fl_static_scratch_bytes(void);
 
 /* Operand packing for invariant point attention (tests/test_ipa.py:57-125, a test-only function of the reference):
  * builds the concatenated operands with which the function becomes one fl_attn_fwd call.  All tensors are bf16,

@@ -130,12 +130,12 @@ def test_workspace_size_for_document_masks(lib):
     p = good_params(B=3, L=1000)
     assert lib.fl_workspace_bytes(C.byref(p)) == 0
     p.mask_kind = _ffi.MASK_DOCUMENT_CAUSAL
-    # (min, max) table per 32 positions + per (batch, query tile) the list of key tiles (count + entries, rounded up to
-    # 4 words) + the ids padded to whole key tiles, for the tile shape the library reports for this call
+    # the backward's (min, max) table per 32 positions, then per (batch, query tile) the forward's list of key tiles
+    # (count + entries, rounded up to 4 words), for the tile shape the library reports for this call
     shape = _ffi.plan(good_params(B=3, L=1000))
     bm, bn = shape["rows_per_workgroup"], shape["keys_per_tile"]
     nq, nk = -(-1000 // bm), -(-1000 // bn)
-    need = 3 * ((1000 + 31) // 32) * 16 + 3 * nq * ((nk + 1 + 3) // 4 * 4) * 4 + 3 * nk * bn * 8
+    need = 3 * ((1000 + 31) // 32) * 16 + 3 * nq * ((nk + 1 + 3) // 4 * 4) * 4
     assert lib.fl_workspace_bytes(C.byref(p)) == need
     p.doc_ids, p.workspace, p.workspace_bytes = 0x50000, 0x80000, need
     assert rc(lib, p) == 0, _ffi.last_error()

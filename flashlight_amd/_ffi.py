@@ -444,7 +444,7 @@ def plan(p: FlAttnParams) -> dict:
     out = (C.c_int64 * 8)()
     _check(lib.fl_attn_plan(C.byref(p), out))
     return {"rows_per_workgroup": out[0], "keys_per_tile": out[1], "threads": out[2], "workgroups": out[3],
-            "lds_bytes": out[4], "features": out[5]}
+            "lds_bytes": out[4], "features": out[5], "streaming": out[6]}
 
 
 def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink: torch.Tensor) -> float:

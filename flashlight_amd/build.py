@@ -120,6 +120,12 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
             if not o.exists():
                 tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_BWD_D={d}", f"-DFL_BWD_FEAT={feat}", f"-DFL_INST_F16={f16}", "-c",
                                str(CSRC / "bwd_unit.hip"), "-o", str(o)], o))
+    # the shared-bias streaming forward: one unit per element type
+    for f16 in (0, 1):
+        o = objdir / f"pairbias{'_f16' if f16 else ''}.o"
+        objs.append(o)
+        if not o.exists():
+            tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_F16={f16}", "-c", str(CSRC / "pairbias_unit.hip"), "-o", str(o)], o))
     # the instance tables are host data only: compiling them for the device would reference the host launchers
     for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("bwd_table.hip", ["--cuda-host-only"]),
                        ("api.hip", []), ("probe.hip", [])):

@@ -9,6 +9,7 @@
 #include "flashlight_amd.h"
 #include "bwd_instances.h"
 #include "instances.h"
+#include "pairbias_instances.h"
 
 namespace fl {
 // Builds (min, max) of the document ids of every block of kDocBlock positions.
@@ -388,6 +389,71 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   return 0;
 }
 
+// Whether *p (already validated) is a call the shared-bias streaming forward covers: head dim 32, no mask or other
+// score modification, exactly one dense 16-bit bias operand that several consecutive batch entries share, 256 / 320 /
+// 384 keys.  Fills the kernel's parameters and launch shape.
+bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
+  static const bool disabled = std::getenv("FL_NO_PAIRBIAS") != nullptr;  // A/B knob: the general kernel instead
+  if (disabled) return false;
+  if (p->Dqk != 32 || p->Dv != 32 || p->mask_kind != FL_MASK_NONE || p->alibi_heads > 0 || p->softcap > 0.f ||
+      p->diff || p->attended_dump || p->dropout_threshold || p->lse)
+    return false;
+  if (!p->bias[0] || p->bias[1] || p->bias_dtype[0] != p->dtype) return false;
+  const int64_t* bst = p->bias_strides[0];
+  const int div = p->bias_batch_div[0];
+  if (div < 2 || p->B % div != 0 || bst[3] != 1 || bst[2] == 0 || bst[1] == 0) return false;
+  if (p->Lk % 32 != 0 || !fl::pairbias_has_shape(p->Lk / 32)) return false;
+  if (reinterpret_cast<uintptr_t>(p->bias[0]) % 16 != 0 || bst[0] % 8 || bst[1] % 8 || bst[2] % 8) return false;
+  if (reinterpret_cast<uintptr_t>(p->o) % 8 != 0 || (p->gate && reinterpret_cast<uintptr_t>(p->gate) % 8 != 0)) return false;
+  // per-lane byte offsets inside one (batch entry, head) slice are 32-bit
+  const int64_t worst = std::max(std::max(p->q_strides[2], p->o_strides[2]), p->gate ? p->gate_strides[2] : 0);
+  if (((int64_t)p->Lq * worst + 64) * 2 >= ((int64_t)1 << 31)) return false;
+  fl::PParams k;
+  std::memset(&k, 0, sizeof(k));
+  k.q = static_cast<const fl::bf16_t*>(p->q);
+  k.k = static_cast<const fl::bf16_t*>(p->k);
+  k.v = static_cast<const fl::bf16_t*>(p->v);
+  k.o = static_cast<fl::bf16_t*>(p->o);
+  for (int i = 0; i < 3; ++i) {
+    k.qs[i] = p->q_strides[i];
+    k.ks[i] = p->k_strides[i];
+    k.vs[i] = p->v_strides[i];
+    k.os[i] = p->o_strides[i];
+    k.gs[i] = p->gate_strides[i];
+    k.bs[i] = bst[i];
+  }
+  k.B = p->B;
+  k.H = p->Hq;
+  if (p->Hq != p->Hkv) return false;
+  k.Lq = p->Lq;
+  k.Lk = p->Lk;
+  k.scale = p->scale;
+  k.bias = static_cast<const fl::bf16_t*>(p->bias[0]);
+  k.bdiv = div;
+  k.gate = static_cast<const fl::bf16_t*>(p->gate);
+  k.n_qtiles = (p->Lq + 127) / 128;
+  // Launch shape: every workgroup should be resident at once (two per compute unit, 32 compute units per XCD), and a
+  // unit = (chunk of batch entries, pair of heads) with all its query tiles stays on one XCD.  The batch entries of a
+  // bias group are cut into as many chunks as that allows; more chunks than entries make no sense, fewer than one
+  // means several rounds of workgroups.
+  const int64_t groups = p->B / div;
+  k.hgroup = p->Hq % 2 == 0 ? 2 : 1;
+  const int64_t per_unit = (int64_t)k.hgroup * k.n_qtiles;
+  const int64_t units_per_xcd = std::max<int64_t>(1, 64 / per_unit);
+  const int64_t head_groups = p->Hq / k.hgroup;
+  int64_t chunks = (8 * units_per_xcd) / (groups * head_groups);
+  chunks = std::max<int64_t>(1, std::min<int64_t>(chunks, div));
+  k.chunk_len = (int)((div + chunks - 1) / chunks);
+  k.chunks = (div + k.chunk_len - 1) / k.chunk_len;
+  const int64_t n_units = groups * k.chunks * head_groups;
+  const int64_t g = (n_units + 7) / 8 * 8 * per_unit;
+  if (n_units > 0x7fffffff || g > 0x7fffffff) return false;
+  k.n_units = (int)n_units;
+  *grid = (int)g;
+  *out = k;
+  return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -422,6 +488,19 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]) {
   out[4] = lds_bytes_for(in, p);
   out[5] = in->feat;
   out[6] = 0;
+  {
+    // calls the shared-bias streaming forward takes: its fixed shape, and out[6] = 1
+    fl::PParams pb;
+    int pb_grid = 0;
+    if (plan_pairbias(p, &pb, &pb_grid)) {
+      out[0] = 128;
+      out[1] = 64;
+      out[2] = 256;
+      out[3] = pb_grid;
+      out[4] = 32768;
+      out[6] = 1;
+    }
+  }
   out[7] = 0;
   return 0;
 }
@@ -431,6 +510,17 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   int rc = validate(p, &in);
   if (rc) return rc;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+  {
+    fl::PParams pb;
+    int pb_grid = 0;
+    if (plan_pairbias(p, &pb, &pb_grid)) {
+      const hipError_t e = (p->dtype == FL_F16 ? fl::launch_pairbias_f16 : fl::launch_pairbias_bf16)(
+          p->Lk / 32, p->gate != nullptr, pb, pb_grid, stream);
+      if (e != hipSuccess) return fail((int)e, "launch of the shared-bias forward failed: %s", hipGetErrorString(e));
+      return 0;
+    }
+  }
 
   fl::KParams kp;
   std::memset(&kp, 0, sizeof(kp));

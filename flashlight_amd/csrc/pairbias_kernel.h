@@ -1,0 +1,395 @@
+// Attention with one dense bias that many batch entries share (the Evoformer's row attention: N_seq rows of an MSA
+// attend over N_res residues, and every row adds the same pair bias [H, N_res, N_res]; reference
+// attention_variants/evoformer.py:8-36), head dim 32, a few hundred keys.
+//
+// The general forward (fwd_kernel.h) gives such a call one short-lived workgroup per (row, head, 128 queries): six key
+// tiles, a bias tile staged next to every K/V tile, and eight or nine vector instructions per score against eight
+// MFMAs per tile.  This kernel turns the loops inside out:
+//   * a workgroup owns (head, 128 queries) and streams over the batch entries (MSA rows) of its chunk; the K/V tile
+//     ring runs on across entries, the next entry's queries are fetched while this one is computed, so the latencies
+//     that bound a six-tile workgroup are paid once per chunk;
+//   * the bias of the workgroup's queries against ALL keys stays in registers for the whole chunk, already laid out as
+//     MFMA B operands (8 consecutive keys of one query per lane and 16-key group);
+//   * the matrix pipe, which idles at head dim 32, adds it: S^T += Sel . Bias^T with Sel the 32 x 16 selector that puts
+//     key 16m + j on row j of the group, weighted 1/scale (split in two bf16 terms, relative error 2^-17), so the
+//     accumulators hold qk + bias/scale and the weights are exp2(scale * log2(e) * acc - ref): per score one
+//     multiply-add, one exponential, half a pack and half a row-sum instruction.
+// Infinite bias entries are clamped to the largest finite value when the fragments are loaded (0 * inf inside the
+// selector product would poison the 15 other keys of the group); as an additive term that is the same mask.
+#pragma once
+#include "fwd_kernel.h"
+
+namespace fl {
+
+struct PParams {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  bf16_t* o;
+  int64_t qs[3], ks[3], vs[3], os[3];  // element strides: batch, head, seq
+  int32_t B, H, Lq, Lk;
+  float scale;
+  const bf16_t* bias;  // [B / bdiv][H][Lq][Lk], unit key stride
+  int64_t bs[3];       // element strides: group, head, query
+  int32_t bdiv;        // batch entries that share one bias slice
+  const bf16_t* gate;  // optional, addressed like o
+  int64_t gs[3];
+  int32_t n_qtiles;   // ceil(Lq / 128)
+  int32_t chunks;     // chunks per bias group
+  int32_t chunk_len;  // batch entries per chunk (the last chunk of a group may be shorter)
+  int32_t hgroup;     // heads whose workgroups are kept on one XCD (they share cache lines when heads are adjacent)
+  int32_t n_units;    // (bias groups * chunks) * (H / hgroup)
+};
+
+// 16 / 8 bytes per lane from global memory into registers, and 8 bytes back, as asm: inside the streaming loop every
+// vector-memory operation is issued by hand in a fixed order, because the waits there count operations
+// (s_waitcnt vmcnt(N): at most N still outstanding, completion in issue order) and a compiler-issued access would not
+// be in the count.  The loaded registers may be read only after the wait that covers them and a pin_loaded() on them.
+__device__ __forceinline__ u32x4 load16_counted(uint64_t sbase, unsigned voff) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
+  return v;
+}
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x2 load8_counted(uint64_t sbase, unsigned voff) {
+  u32x2 v;
+  asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
+  return v;
+}
+__device__ __forceinline__ void store8_counted(uint64_t sbase, unsigned voff, u32x2 data) {
+  asm volatile("global_store_dwordx2 %0, %1, %2" ::"v"(voff), "v"(data), "s"(sbase));
+}
+template <class V>
+__device__ __forceinline__ void pin_loaded(V& v) {
+  asm volatile("" : "+v"(v));
+}
+
+template <int NKB_, bool GATE_, class Elem_>
+struct PairBiasTraits {
+  using Elem = Elem_;
+  static constexpr int NKB = NKB_;       // 32-key blocks per row: Lk = 32 * NKB
+  static constexpr bool GATE = GATE_;
+  static constexpr int D = 32, BN = 64, NW = 4, NT = 256, BM = 128;
+  static constexpr int NTI = NKB / 2;    // key tiles per batch entry
+  static constexpr int NS = 4;           // K/V tiles resident in LDS; transfers run three tiles ahead
+  static_assert(NKB % 2 == 0 && NTI >= 4, "whole tiles; the wait bookkeeping needs four tiles per entry");
+  static constexpr int TILE_BYTES = BN * D * 2;
+  static constexpr int K_OFF = 0, V_OFF = NS * TILE_BYTES, LDS_BYTES = 2 * NS * TILE_BYTES;
+};
+
+template <class T>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void pairbias_kernel(const PParams p) {
+  using E = typename T::Elem;
+  typedef E ex8 __attribute__((ext_vector_type(8)));
+  typedef E ex4 __attribute__((ext_vector_type(4)));
+  typedef E ex2 __attribute__((ext_vector_type(2)));
+  constexpr int NKB = T::NKB, NTI = T::NTI, NS = T::NS, D = T::D, BN = T::BN;
+  constexpr bool kGate = T::GATE;
+  constexpr float kLog2e = 1.4426950408889634f;
+  using LK = TileLayout<D>;
+  using LV = TileLayout<D>;
+
+  __shared__ __attribute__((aligned(16))) unsigned char smem[T::LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int r = lane % 32, h = lane / 32;
+
+  // ---- workgroup -> (bias group, chunk of batch entries, head, query tile).  Consecutive workgroup ids land on
+  // different XCDs; a unit = (chunk, group of adjacent heads) is kept on one XCD, all its query tiles together: they read
+  // the same K/V, and adjacent heads share cache lines when the head axis is the second-fastest in memory.
+  int fb0, n_items, head, qt, grp;
+  {
+    const int per_unit = p.hgroup * p.n_qtiles;
+    const int x = blockIdx.x % 8, rest = blockIdx.x / 8;
+    const int local = rest % per_unit, u = (rest / per_unit) * 8 + x;
+    if (u >= p.n_units) return;  // (before any barrier)
+    const int hg_count = p.H / p.hgroup;
+    const int ct = u / hg_count, hg = u % hg_count;  // chunk over all groups, head group
+    grp = ct / p.chunks;
+    const int c = ct % p.chunks;
+    head = hg * p.hgroup + local / p.n_qtiles;
+    qt = local % p.n_qtiles;
+    fb0 = grp * p.bdiv + c * p.chunk_len;
+    n_items = min(p.chunk_len, p.bdiv - c * p.chunk_len);
+  }
+  const int qrow = min(qt * T::BM + wave * 32 + r, p.Lq - 1);  // rows past Lq repeat the last row (same values stored)
+
+  // ---- the resident bias: B operands of the selector products, lane (r, h) holds bias[qrow][32 kb + 16 m + 8 h .. + 8]
+  ex8 bfrag[NKB][2];
+  {
+    const bf16_t* brow = p.bias + (int64_t)grp * p.bs[0] + (int64_t)head * p.bs[1] + (int64_t)qrow * p.bs[2];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        u32x4 raw = *reinterpret_cast<const u32x4*>(brow + 32 * kb + 16 * m + 8 * h);
+        // +-inf -> +-largest finite, two elements per register: an element is infinite when its low 15 bits are
+        // exactly the exponent mask (bf16 0x7F80, fp16 0x7C00)
+        constexpr uint32_t kInf = std::is_same<E, f16_t>::value ? 0x7C00u : 0x7F80u;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t x = raw[w];
+          const uint32_t lo_inf = ((x & 0x7FFFu) == kInf) ? 1u : 0u;
+          const uint32_t hi_inf = (((x >> 16) & 0x7FFFu) == kInf) ? 0x10000u : 0u;
+          raw[w] = x - lo_inf - hi_inf;
+        }
+        bfrag[kb][m] = __builtin_bit_cast(ex8, raw);
+      }
+  }
+  // selectors: A operand of group m puts key 16 m + j on row j; lane (r, h) holds Sel[key = r][j = 8 h .. 8 h + 7]
+  ex8 sel[2][2];
+  {
+    const float w = 1.0f / p.scale;
+    const E w_hi = (E)w;
+    const E w_lo = (E)(w - (float)w_hi);
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool on = r == 16 * m + 8 * h + j;
+        sel[m][0][j] = on ? w_hi : (E)0.0f;
+        sel[m][1][j] = on ? w_lo : (E)0.0f;
+      }
+  }
+  const float c2 = p.scale * kLog2e;  // acc * c2 = (qk * scale + bias) in log2 units
+
+  // ---- addresses.  Per-lane byte offsets are constant; scalar bases move with the batch entry and the tile.
+  // K/V tile = 64 rows x 64 bytes = 4 wave transfers of 1 KiB: wave w brings transfer w, lane l -> (row, physical chunk)
+  unsigned koff, voff;
+  {
+    const int id = wave * 64 + lane, row = id / LK::CPR, pc = id % LK::CPR;
+    koff = (unsigned)(row * (int)p.ks[2] + LK::swz_k(row, pc) * 8) * 2u;
+    voff = (unsigned)(row * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
+  }
+  const unsigned lds_k = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::K_OFF + wave * 1024);
+  const unsigned lds_v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::V_OFF + wave * 1024);
+  const uint64_t kbase = uniform_ptr(p.k + (int64_t)head * p.ks[1]), vbase = uniform_ptr(p.v + (int64_t)head * p.vs[1]);
+  const uint64_t qbase = uniform_ptr(p.q + (int64_t)head * p.qs[1]);
+  const uint64_t obase = uniform_ptr(p.o + (int64_t)head * p.os[1]);
+  const uint64_t gbase = kGate ? uniform_ptr(p.gate + (int64_t)head * p.gs[1]) : 0;
+  const unsigned qoff = (unsigned)(qrow * (int)p.qs[2] + 8 * h) * 2u;  // + 32 bytes for the second k-step
+  const unsigned ooff = (unsigned)(qrow * (int)p.os[2] + 4 * h) * 2u;  // + 16 bytes per group of 8 value columns
+  const unsigned goff = kGate ? (unsigned)(qrow * (int)p.gs[2] + 4 * h) * 2u : 0u;
+
+  // tile j of the stream (entry j / NTI of the chunk, tile j % NTI of its keys; past the end the last entry again, so
+  // that every step issues the same operations) -> ring slot j % NS
+  auto issue_tile = [&](int item, int t, int slot) FL_INLINE {
+    const int64_t fb = fb0 + min(item, n_items - 1);
+    dma16(kbase + (uint64_t)((fb * p.ks[0] + (int64_t)t * BN * p.ks[2]) * 2), koff, lds_k + slot * T::TILE_BYTES);
+    dma16(vbase + (uint64_t)((fb * p.vs[0] + (int64_t)t * BN * p.vs[2]) * 2), voff, lds_v + slot * T::TILE_BYTES);
+  };
+
+  // ---- K fragments (A operands of S^T = K . Q^T) of block b of the tile in ring slot `slot`
+  auto k_frags = [&](ex8 (&kf)[2], int slot, int b) FL_INLINE {
+    const unsigned char* kt = smem + T::K_OFF + slot * T::TILE_BYTES;
+    const int row = 32 * b + r;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+      kf[ks] = *reinterpret_cast<const ex8*>(kt + row * (D * 2) + LK::swz_k(row, 2 * ks + h) * 16);
+  };
+  // ---- S^T block: K fragments as A operand, Q fragments as B; then the bias through the selectors
+  auto scores = [&](f32x16& s, const ex8 (&kf)[2], const ex8 (&qf)[2], int kb) FL_INLINE {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) s = mfma32(kf[ks], qf[ks], s);
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int part = 0; part < 2; ++part) s = mfma32(sel[m][part], bfrag[kb][m], s);
+  };
+  // A operand of O^T += V^T . P^T for 16-key chunk c of the tile (the transposing LDS read of the general kernel)
+  auto v_frag = [&](int slot, int c) FL_INLINE -> ex8 {
+    const unsigned char* vt = smem + T::V_OFF + slot * T::TILE_BYTES;
+    ex8 vf;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i16 = lane % 16, g = (lane / 16) % 2;
+      const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
+      const int col = g * 16 + 4 * (i16 % 4);
+      const unsigned char* ap = vt + row * (D * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
+      typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+      const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
+      const ex4 b4 = __builtin_bit_cast(ex4, t4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vf[4 * j + e] = b4[e];
+    }
+    return vf;
+  };
+
+  // ---- softmax state of the current entry.  ref is the reference the weights are formed against, in log2 units; it
+  // starts at 0 and moves only when a row sum says it must (a weight overflowed, or a whole block underflowed with
+  // nothing accumulated yet): any reference gives the same O / l.
+  f32x16 oacc;
+  float ref = 0.f, l_run = 0.f;
+  constexpr float kBig = 0x1p24f, kTiny = std::is_same<E, f16_t>::value ? 0x1p-4f : 0x1p-24f;
+  auto weights = [&](const f32x16& s, ex8 (&pf)[2]) FL_INLINE {
+    const ex2 ones = {(E)1.0f, (E)1.0f};
+    auto form = [&]() FL_INLINE -> float {
+      float rs = 0.f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[j][e] = (E)fast_exp2(__builtin_fmaf(s[8 * j + e], c2, -ref));
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const ex2 pr = {pf[j][e], pf[j][e + 1]};
+          rs = dot2acc(pr, ones, rs);
+        }
+      }
+      return rs;
+    };
+    float rs = form();
+    const bool bad = !(rs <= kBig) | ((rs < kTiny) & (l_run < kTiny));
+    if (__builtin_amdgcn_ballot_w64(bad) != 0) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) m = __builtin_fmaxf(m, s[i]);
+      m = xhalf_max(m) * c2;
+      const float ref_new = (m == -INFINITY) ? ref : __builtin_fmaxf(ref, m);
+      // (when nothing has been accumulated yet the old reference carries no weight: take the block's own maximum)
+      const float use = (l_run == 0.f && m != -INFINITY) ? m : ref_new;
+      const float alpha = __builtin_fminf(fast_exp2(ref - use), 0x1p126f);
+      ref = use;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[i] *= alpha;
+      rs = form();
+    }
+    l_run += rs;
+  };
+
+  // ---- prologue: queries of the first entry, the first three tiles, scores of the first block
+  ex8 qf[2];
+  {
+    const uint64_t qb0 = qbase + (uint64_t)((int64_t)fb0 * p.qs[0] * 2);
+    u32x4 a = load16_counted(qb0, qoff), b = load16_counted(qb0, qoff + 32u);
+    issue_tile(0, 0, 0);
+    issue_tile(0, 1, 1);
+    issue_tile(0, 2, 2);
+    dma_wait<0>();
+    pin_loaded(a);
+    pin_loaded(b);
+    qf[0] = __builtin_bit_cast(ex8, a);
+    qf[1] = __builtin_bit_cast(ex8, b);
+  }
+  __syncthreads();
+  f32x16 s_a, s_b;
+  ex8 kf[2];  // K fragments of the block whose scores are formed next, read from LDS one block ahead of their use
+  k_frags(kf, 0, 0);
+  scores(s_a, kf, qf, 0);
+  k_frags(kf, 0, 1);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+
+  // Operations a wave issues, in order, per entry:  at the barrier point of tile t (in the tile's second block): the two
+  // transfers of the tile three ahead, and at t == 0 also the gate loads of this entry (4, if there is a gate) and the
+  // query loads of the next (2); after the entry's last block: 4 stores.  The barrier point of tile t waits for the
+  // transfers of tile t + 1, issued two barrier points earlier; kAllowed(t) counts what was issued after them.
+  constexpr int NI = 2 + (kGate ? 4 : 0);
+  for (int item = 0; item < n_items; ++item) {
+    const int slot0 = (item * NTI) % NS;
+    u32x4 qn_a, qn_b;        // next entry's query fragments, in flight from tile 0 on
+    u32x2 gl[4];             // this entry's gate logits, likewise
+    const int64_t fbn = fb0 + min(item + 1, n_items - 1);
+    const int64_t fbc = fb0 + item;
+    ex8 qnext[2];
+    static_while<0, NTI>([&](auto tt) FL_INLINE {
+      constexpr int t = decltype(tt)::value;
+      const int slot = (slot0 + t) % NS;
+      static_while<0, 2>([&](auto bb) FL_INLINE {
+        constexpr int b = decltype(bb)::value;
+        constexpr int kb = 2 * t + b;
+        constexpr bool last_block = kb == NKB - 1;
+        if constexpr (b == 0) {
+          // barrier point of tile t, before anything of the tile after it is touched
+          constexpr int kAllowed = 2 + (t == 1 || t == 2 ? NI : 0) + (t == 0 || t == 1 ? 4 : 0);
+          dma_wait<kAllowed>();
+          __syncthreads();  // tile t + 1 is visible; everyone is done with tile t - 1, whose slot the new tile takes
+          issue_tile(item + (t + 3) / NTI, (t + 3) % NTI, (slot + 3) % NS);
+          if constexpr (t == 0) {
+            if constexpr (kGate) {
+              const uint64_t gb = gbase + (uint64_t)(fbc * p.gs[0] * 2);
+#pragma unroll
+              for (int g = 0; g < 4; ++g) gl[g] = load8_counted(gb, goff + 16u * g);
+            }
+            const uint64_t qb = qbase + (uint64_t)(fbn * p.qs[0] * 2);
+            qn_a = load16_counted(qb, qoff);
+            qn_b = load16_counted(qb, qoff + 32u);
+          }
+          if constexpr (t == NTI - 1) {
+            // everything issued at tile 0 has landed (the wait above covers later transfers): next entry's queries
+            pin_loaded(qn_a);
+            pin_loaded(qn_b);
+            qnext[0] = __builtin_bit_cast(ex8, qn_a);
+            qnext[1] = __builtin_bit_cast(ex8, qn_b);
+            if constexpr (kGate) {
+#pragma unroll
+              for (int g = 0; g < 4; ++g) pin_loaded(gl[g]);
+            }
+          }
+        }
+        // Scores of the next block (the first block of the next entry after the last one of this) go to the matrix pipe
+        // under this block's exponentials; their K fragments were read from LDS during the previous block, and the
+        // LDS reads issued now (K fragments for the block after next, V fragments for this block's second product) have
+        // the exponentials to land under.
+        f32x16& cur = (kb % 2 == 0) ? s_a : s_b;
+        f32x16& nxt = (kb % 2 == 0) ? s_b : s_a;
+        ex8 kf_ahead[2], vf[2];
+        k_frags(kf_ahead, (slot + 1) % NS, b);  // block kb + 2: same half of the next tile in the ring
+#pragma unroll
+        for (int c = 0; c < 2; ++c) vf[c] = v_frag(slot, 2 * b + c);
+        if constexpr (last_block) scores(nxt, kf, qnext, 0);
+        else scores(nxt, kf, qf, kb + 1);
+        kf[0] = kf_ahead[0];
+        kf[1] = kf_ahead[1];
+        ex8 pf[2];
+        weights(cur, pf);
+        // 6 LDS reads first, then the 6 score MFMAs spread over the exponentials (64 vector instructions per block)
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+          __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, 10, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) oacc = mfma32(vf[c], pf[c], oacc);
+        return true;
+      });
+      return true;
+    });
+    // ---- this entry is complete: normalise, gate, store; then start the next one
+    {
+      const float l = xhalf_sum(l_run);
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      const uint64_t ob = obase + (uint64_t)(fbc * p.os[0] * 2);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        ex4 o4;
+        if constexpr (kGate) {
+          const ex4 g4 = __builtin_bit_cast(ex4, gl[g]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
+            o4[e] = (E)(oacc[4 * g + e] * inv * sg);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o4[e] = (E)(oacc[4 * g + e] * inv);
+        }
+        store8_counted(ob, ooff + 16u * g, __builtin_bit_cast(u32x2, o4));
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+      ref = 0.f;
+      l_run = 0.f;
+      qf[0] = qnext[0];
+      qf[1] = qnext[1];
+    }
+  }
+  dma_wait<0>();  // nothing of this wave may still be on its way into LDS when the workgroup's allocation is released
+}
+
+}  // namespace fl

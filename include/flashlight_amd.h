@@ -148,7 +148,9 @@ uint64_t fl_workspace_bytes(const fl_attn_params* p);
 int fl_attn_fwd(const fl_attn_params* p, void* stream);
 
 /* Describes the kernel instance fl_attn_fwd would pick for *p: tile sizes and launch shape.
- * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes. */
+ * out[0]=rows per workgroup, out[1]=keys per tile, out[2]=threads, out[3]=workgroups, out[4]=LDS bytes,
+ * out[5]=feature bits of the instance, out[6]=1 when the call goes to the shared-bias streaming kernel instead (head
+ * dim 32, one dense bias shared by several batch entries, 256 / 320 / 384 keys: the Evoformer shape). */
 int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
 
 /* Backward of fl_attn_fwd.  No counterpart in the reference, which is forward-only (its FLOP helper models a

@@ -487,3 +487,45 @@ def test_config0_shape_causal():
     out = A.attention_pytorch_causal(*(t.to(torch.bfloat16).to(DEV) for t in (q, k, v)))
     assert out.shape == (2, 8, 512, 64)
     assert_parity(out, O.attention_causal(q, k, v), "config 0")
+
+
+# ---- the shared-bias streaming kernel (head dim 32, one dense bias shared by the rows of an MSA, 256 / 320 / 384 keys) ----
+
+@pytest.mark.parametrize("B,N,S,H,gate,dtype,inf", [
+    (1, 64, 384, 8, True, torch.bfloat16, False),    # the benchmark's shape class
+    (1, 37, 256, 4, False, torch.bfloat16, False),   # no gate; a row count that leaves a short last chunk
+    (2, 19, 320, 3, True, torch.bfloat16, False),    # two bias groups, odd head count
+    (1, 5, 256, 8, True, torch.float16, False),      # fp16 elements
+    (1, 33, 384, 2, True, torch.bfloat16, True),     # -inf entries in the bias (an additive mask)
+    (1, 2, 256, 8, False, torch.bfloat16, False),    # two rows: chunks of one entry
+])
+def test_shared_bias_streaming_kernel(B, N, S, H, gate, dtype, inf):
+    g = torch.Generator().manual_seed(31)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)  # noqa: E731
+    q, k, v = mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32)
+    bias = mk(B, 1, H, S, S)
+    if inf:
+        bias[..., ::7] = float("-inf")
+    gt = mk(B, N, S, H, 32) if gate else None
+    # the call must be one the streaming kernel takes (the plan says so), not the general one
+    p, _keep = _ffi._fill_params(_ffi.load_library(), *(t.reshape(-1, S, H, 32).transpose(1, 2) for t in (q, k, v)),
+                                 torch.empty(B * N, H, S, 32, dtype=dtype, device=DEV), H, H, None, _ffi.MASK_NONE, 0, 0,
+                                 None, 0, 0.0, [(bias.reshape(B, H, S, S), N)], None, False, 0.0, None)
+    assert _ffi.plan(p)["streaming"] == 1
+    out = A.attention_reference(q, k, v, [bias], gate=gt) if gate else A.attention_reference(q, k, v, [bias])
+    ref = O.attention_evoformer(*f32(q, k, v), [bias.float()], gate=None if gt is None else gt.float())
+    assert_parity(out, ref, f"B{B} N{N} S{S} H{H}")
+
+
+def test_shared_bias_streaming_kernel_matches_the_general_kernel():
+    # same call through both kernels: a second bias operand (all zeros) makes the library take the general one
+    g = torch.Generator().manual_seed(32)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)  # noqa: E731
+    B, N, S, H = 1, 24, 384, 4
+    q, k, v, gt = mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32)
+    bias = mk(B, 1, H, S, S)
+    zero = torch.zeros(B, N, 1, 1, S, dtype=torch.bfloat16, device=DEV)
+    fast = A.attention_reference(q, k, v, [bias], gate=gt)
+    general = A.attention_reference(q, k, v, [zero, bias], gate=gt)
+    assert (fast.float() - general.float()).abs().max().item() <= 2e-2
+    assert_parity(fast, O.attention_evoformer(*f32(q, k, v), [bias.float()], gate=gt.float()), "streaming")

@@ -147,6 +147,23 @@ static __global__ __launch_bounds__(1024) void doc_lists_kernel(const int64_t* i
   }
 }
 
+// Second step of the forward pre-pass for document masks, one workgroup per batch row: the query tiles ordered by
+// falling length of their tile lists (ties by falling index), by counting for every tile how many come before it.
+static __global__ __launch_bounds__(1024) void doc_order_kernel(const uint32_t* lists, int list_stride, int n_qtiles,
+                                                               int32_t* order) {
+  extern __shared__ uint32_t cnt[];  // n_qtiles words
+  const int b = blockIdx.x;
+  const uint32_t* lb = lists + (int64_t)b * n_qtiles * list_stride;
+  for (int i = threadIdx.x; i < n_qtiles; i += 1024) cnt[i] = lb[(int64_t)i * list_stride];
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_qtiles; i += 1024) {
+    const uint32_t mine = cnt[i];
+    int rank = 0;
+    for (int j = 0; j < n_qtiles; ++j) rank += (cnt[j] > mine) || (cnt[j] == mine && j > i);
+    order[(int64_t)b * n_qtiles + rank] = i;
+  }
+}
+
 }  // namespace fl
 
 // Scratch of the entry point that allocates nothing (fl_attn_bwd_static): one copy per GPU the library runs on, held
@@ -245,9 +262,10 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
 //   table   [B][ceil(L / 32)][2] int64   (min, max) id per 32 positions (backward)
 //   lists   [B][query tiles][stride] u32 the key tiles each query tile visits (forward; bm / bn = query rows per
 //                                        workgroup and keys per tile of the forward instance)
+//   order   [B][query tiles] i32          the query tiles by falling list length (forward), rounded up to 16 bytes
 struct DocScratch {
   int64_t blocks, n_qtiles, nk, list_stride;
-  uint64_t table_bytes, lists_bytes;
+  uint64_t table_bytes, lists_bytes, order_bytes;
 };
 DocScratch doc_scratch(int64_t B, int64_t L, int64_t bm, int64_t bn) {
   DocScratch d;
@@ -257,6 +275,7 @@ DocScratch doc_scratch(int64_t B, int64_t L, int64_t bm, int64_t bn) {
   d.list_stride = (d.nk + 1 + 3) / 4 * 4;
   d.table_bytes = (uint64_t)B * d.blocks * 2 * sizeof(int64_t);
   d.lists_bytes = (uint64_t)B * d.n_qtiles * d.list_stride * sizeof(uint32_t);
+  d.order_bytes = ((uint64_t)B * d.n_qtiles * sizeof(int32_t) + 15) / 16 * 16;
   return d;
 }
 
@@ -470,7 +489,7 @@ uint64_t fl_workspace_bytes(const fl_attn_params* p) {
   // valid one)
   const fl::Instance* in = select_instance(p);
   const DocScratch d = doc_scratch(p->B, p->Lk, in ? (int64_t)in->rw * in->nw : 64, in ? in->bn : 32);
-  return d.table_bytes + d.lists_bytes;
+  return d.table_bytes + d.lists_bytes + d.order_bytes;
 }
 
 int fl_attn_validate(const fl_attn_params* p) { return validate(p, nullptr); }
@@ -614,8 +633,14 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
                        (int)d.list_stride, lists);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail((int)e, "doc_lists_kernel launch failed: %s", hipGetErrorString(e));
+    int32_t* order = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p->workspace) + d.table_bytes + d.lists_bytes);
+    hipLaunchKernelGGL(fl::doc_order_kernel, dim3(p->B), dim3(1024), (size_t)kp.n_qtiles * 4, stream, lists,
+                       (int)d.list_stride, kp.n_qtiles, order);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "doc_order_kernel launch failed: %s", hipGetErrorString(e));
     kp.doc_lists = lists;
     kp.doc_list_stride = (int)d.list_stride;
+    kp.doc_order = order;
   }
   hipError_t e = in->launch(kp, grid, (int)lds_bytes_for(in, p), stream);
   if (e != hipSuccess) return fail((int)e, "launch of %s failed: %s", in->name, hipGetErrorString(e));

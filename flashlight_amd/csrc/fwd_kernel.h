@@ -68,6 +68,9 @@ struct KParams {
   // entries in key order (bits 0-15 tile index, two class bits per wave from bit 16 on).
   const uint32_t* doc_lists;
   int32_t doc_list_stride;  // words per (batch, query tile): a multiple of 4, at least n_ktiles + 1
+  // per batch row the query tiles ordered by falling list length (doc_order_kernel): workgroups are dealt in that order,
+  // so that the ones still running when the grid drains are the short ones whatever the document layout
+  const int32_t* doc_order;
   int32_t alibi_heads;
   float softcap;
   const bf16_t* bias[2];
@@ -418,11 +421,13 @@ void fwd_kernel(const KParams p) {
       base = (i % 8) * run;
       i /= 8;
     }
-    const int G = (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || p.mask_kind == MASK_DOC_CAUSAL) ? 4 : 1;
+    const int G = (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || kDoc) ? 4 : 1;
     const int g = i / (G * nq), rem = i % (G * nq);
     const int gg = min(G, run - G * g);
     qt = nq - 1 - rem / gg;
     bh = base + G * g + rem % gg;
+    // document masks: the work of a query tile is the length of its tile list, known from the pre-pass
+    if constexpr (kDoc) qt = p.doc_order[(bh / p.Hq) * nq + rem / gg];
   }
   const int head = bh % p.Hq, batch = bh / p.Hq;
   const int kvh = head / p.group;

@@ -135,7 +135,7 @@ def test_workspace_size_for_document_masks(lib):
     shape = _ffi.plan(good_params(B=3, L=1000))
     bm, bn = shape["rows_per_workgroup"], shape["keys_per_tile"]
     nq, nk = -(-1000 // bm), -(-1000 // bn)
-    need = 3 * ((1000 + 31) // 32) * 16 + 3 * nq * ((nk + 1 + 3) // 4 * 4) * 4
+    need = 3 * ((1000 + 31) // 32) * 16 + 3 * nq * ((nk + 1 + 3) // 4 * 4) * 4 + (3 * nq * 4 + 15) // 16 * 16
     assert lib.fl_workspace_bytes(C.byref(p)) == need
     p.doc_ids, p.workspace, p.workspace_bytes = 0x50000, 0x80000, need
     assert rc(lib, p) == 0, _ffi.last_error()

@@ -28,6 +28,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the eager CPU timing (about 20 s)")
     ap.add_argument("--no-other-configs", action="store_true", help="only run the configuration the metric is quoted on")
+    ap.add_argument("--only", metavar="WORKLOAD", default=None,
+                    help="profiling aid: launch just this workload (e.g. cfg3/document_mask_causal) --warmup + --steps times "
+                         "and print its event-timed duration; nothing else runs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one 256 MiB device-to-device copy (known traffic, for scaling rocprofv3 counters)")
     return ap.parse_args()
@@ -170,6 +173,18 @@ def main():
     _ffi.load_library()  # fail loudly if the HIP extension is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.only:
+        w = W.workload_by_name(args.only)
+        t = w.make(dev)
+        ms = time_back_to_back(lambda: w.call(t), iters=args.steps, warmup=args.warmup)
+        if args.calibrate_copy:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            dst.copy_(src)
+            torch.cuda.synchronize()
+        print(json.dumps({"workload": w.name, "ms": ms, "launches": args.steps, "warmup": args.warmup,
+                          "unmasked_flops": w.flops, "min_bytes": w.min_bytes, "roofline": roofline_entry(w, ms, W)}))
+        return
     all_w = W.build_workloads()
     cfg1 = [w for w in all_w if w.config == 1]
     tens = cfg1[0].make(dev)  # the three variants share q, k, v (same seed)

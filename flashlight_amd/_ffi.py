@@ -321,18 +321,21 @@ def attn_fwd(
         out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
     elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != q.dtype or out.device != q.device:
         raise ValueError("out has the wrong shape, dtype or device")
-    if diff and Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None:
-        # Value columns are independent of one another: a differential launch keeps two sets of output accumulators,
-        # so wide values go in slabs of _MAX_DV_DIFF columns, one launch each, through strided views of v and out
-        # (the reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38).
-        if lse is not None or dropout_p > 0.0:
+    if Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None and (diff or Dqk > 128):
+        # Value columns are independent of one another, so wide values go in slabs of _MAX_DV_DIFF columns, one launch
+        # each, through strided views of v and out: a differential launch keeps two sets of output accumulators (the
+        # reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38), and at head dim 256
+        # the query fragments leave room for 128 output columns per launch.
+        if diff and (lse is not None or dropout_p > 0.0):
             # what the single launch refuses for differential attention is refused here too, instead of dropped
             raise NotImplementedError("differential attention produces no lse and takes no dropout")
         for c in range(0, Dv, _MAX_DV_DIFF):
             attn_fwd(q, k, v[..., c:c + _MAX_DV_DIFF], scale=scale, mask_kind=mask_kind, window=window, prefix=prefix,
                      doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases,
-                     gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=True, lambda_full=lambda_full,
-                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only)
+                     gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=diff, lambda_full=lambda_full,
+                     out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only,
+                     lse=lse if c == 0 else None,  # the row statistics depend on q and k only
+                     dropout_p=dropout_p, dropout_seed=dropout_seed)  # so do the dropout decisions
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,

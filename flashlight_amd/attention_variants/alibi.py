@@ -61,13 +61,11 @@ def attention_pytorch_alibi(query: torch.Tensor, key: torch.Tensor, value: torch
         out = run(query, key, value, scale=scale, enable_gqa=enable_gqa, mask_kind=mask_kind,
                   alibi_heads=score_mod.nheads, softcap=float(softcap or 0.0), dropout_p=dropout_p)
         return grouped_view(out, key, enable_gqa)
-    if softcap is not None:
-        raise NotImplementedError("softcap is only fused together with the bias of generate_alibi_bias_pytorch()")
     if not callable(score_mod):
         raise TypeError("score_mod must be callable as score_mod(q_len, kv_len)")
     bias = dense_bias_operand(score_mod(query.size(-2), key.size(-2)), query, key, enable_gqa)
     out = run(query, key, value, scale=scale, enable_gqa=enable_gqa, mask_kind=mask_kind, biases=[bias],
-              dropout_p=dropout_p)
+              softcap=float(softcap or 0.0), dropout_p=dropout_p)
     return grouped_view(out, key, enable_gqa)
 
 

@@ -1,0 +1,168 @@
+"""Head dim 256 and feature combinations beyond the benchmark's (document mask + ALiBi / soft-cap, dense bias +
+soft-cap, score_mod callables of the soft-cap signature), HIP kernels through the C ABI against the CPU oracle.
+Tolerance: bf16 kernel against the fp32 oracle, max-abs 2e-2 and mean-abs 2e-3.
+
+The reference's generated kernel takes any head dim up to 256 in one block (monkeypatch/fusion/_common.py:4) and
+whatever composition of mask and score modification the eager function writes."""
+import math
+
+import pytest
+import torch
+
+import flashlight_amd.attention_variants as A
+import oracle as O
+from flashlight_amd import _ffi, ops
+from oracle.attention import _softmax_attention, alibi_slopes
+from tests.conftest import assert_parity
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def f32(*ts):
+    return tuple(t.float().cpu() for t in ts)
+
+
+def qkv(B, Hq, Hkv, S, D, Dv=None, seed=0, amp=1.0):
+    g = torch.Generator().manual_seed(seed)
+    shapes = [(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, Dv or D)]
+    ts = [torch.randn(s, generator=g) for s in shapes]
+    ts[0] = ts[0] * amp
+    return tuple(t.to(torch.bfloat16).to(DEV) for t in ts)
+
+
+@pytest.mark.parametrize("S", [1, 65, 300, 1024])
+@pytest.mark.parametrize("Dv", [128, 256])
+def test_head_dim_256_masks(S, Dv):
+    q, k, v = qkv(2, 4, 2, S, 256, Dv, seed=S + Dv)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch(q, k, v, enable_gqa=True), O.attention_vanilla(qf, kf, vf, enable_gqa=True), "vanilla")
+    assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(qf, kf, vf, enable_gqa=True),
+                  "causal")
+    assert_parity(A.attention_pytorch_sliding_window(q, k, v, window_size=70, enable_gqa=True),
+                  O.attention_sliding_window(qf, kf, vf, window_size=70, enable_gqa=True), "sliding")
+    assert_parity(A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=100, enable_gqa=True),
+                  O.attention_prefix_lm(qf, kf, vf, prefix_lengths=100, enable_gqa=True), "prefix")
+
+
+def test_head_dim_256_score_mods_and_documents():
+    S = 700
+    q, k, v = qkv(2, 4, 4, S, 256, 256, seed=5, amp=3.0)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(4)),
+                  O.attention_alibi(qf, kf, vf, score_mod=4), "alibi")
+    assert_parity(A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(20.0)),
+                  O.attention_softcapped(qf, kf, vf, score_mod=20.0), "softcap")
+    assert_parity(A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(4), is_causal=True, softcap=15.0),
+                  O.attention_alibi(qf, kf, vf, score_mod=4, is_causal=True, honor_causal=True, softcap=15.0),
+                  "alibi+softcap+causal")
+    g = torch.Generator().manual_seed(6)
+    ids = torch.sort(torch.randint(0, 5, (2, S), generator=g), dim=1).values
+    for causal in (False, True):
+        assert_parity(A.attention_pytorch_document_mask(q, k, v, ids.to(DEV), is_causal=causal),
+                      O.attention_document_mask(qf, kf, vf, ids, is_causal=causal), f"document causal={causal}")
+
+
+def test_head_dim_256_row_statistics_come_from_the_first_slab():
+    """Values wider than 128 columns go in slabs; lse depends on q and k only and is written once."""
+    q, k, v = qkv(1, 2, 2, 200, 256, 256, seed=8)
+    lse = torch.empty(1, 2, 200, dtype=torch.float32, device=DEV)
+    _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, lse=lse)
+    qf, kf, _ = f32(q, k, v)
+    s = torch.matmul(qf, kf.transpose(-1, -2)) / math.sqrt(256)
+    s = s.masked_fill(torch.ones(200, 200, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.logsumexp(s, dim=-1) / math.log(2.0)  # the kernels keep row statistics in log2 units
+    assert (lse.cpu() - ref).abs().max().item() < 2e-2
+
+
+def _doc_alibi_oracle(qf, kf, vf, ids, nheads, cap, causal):
+    """Eager fp32 composition: cap * tanh(q k^T s / cap) + slope_h (k - q), masked where the ids differ (or k > q)."""
+    slopes = alibi_slopes(nheads).float().view(1, nheads, 1, 1)
+
+    def masked(qi, ki):
+        m = ids[:, qi.view(-1)].view(ids.size(0), 1, -1, 1) != ids[:, ki.view(-1)].view(ids.size(0), 1, 1, -1)
+        return (m | (ki > qi)) if causal else m
+
+    return _softmax_attention(qf, kf, vf, 1.0 / math.sqrt(qf.size(-1)), masked=masked, softcap=cap,
+                              bias=lambda qi, ki: slopes * (ki - qi).float())
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("cap", [None, 12.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_document_mask_with_alibi_and_softcap(D, cap, causal):
+    B, H, S = 2, 4, 600
+    q, k, v = qkv(B, H, H, S, D, seed=D + 3, amp=3.0)
+    g = torch.Generator().manual_seed(21)
+    ids = torch.sort(torch.randint(0, 6, (B, S), generator=g), dim=1).values
+    out = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_DOCUMENT_CAUSAL if causal else _ffi.MASK_DOCUMENT, doc_ids=ids.to(DEV),
+                       alibi_heads=H, softcap=cap or 0.0)
+    assert_parity(out, _doc_alibi_oracle(*f32(q, k, v), ids, H, cap, causal), f"D={D} cap={cap} causal={causal}")
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("gqa", [False, True])
+def test_dense_score_mod_with_softcap(D, gqa):
+    """attention_pytorch_alibi(score_mod=<any callable>, softcap=...): cap first, then the dense tensor (alibi.py:26-30)."""
+    B, Hq, Hkv, S = 2, 4, (2 if gqa else 4), 333
+    q, k, v = qkv(B, Hq, Hkv, S, D, seed=D + 9, amp=4.0)
+    g = torch.Generator().manual_seed(31)
+    dense = torch.randn(Hq, S, S, generator=g) * 2.0
+
+    out = A.attention_pytorch_alibi(q, k, v, score_mod=lambda L, S_: dense.to(DEV), enable_gqa=gqa, softcap=9.0, is_causal=True)
+    ref = O.attention_alibi(*f32(q, k, v), score_mod=lambda L, S_: dense, enable_gqa=gqa, softcap=9.0, is_causal=True,
+                            honor_causal=True)
+    assert_parity(out, ref, f"D={D} gqa={gqa}")
+
+
+def _eager_softcapped(qf, kf, vf, fn, causal=False):
+    """softcap.py:40-53 in fp32 on the CPU: the callable is applied to the whole scaled score matrix."""
+    s = torch.matmul(qf, kf.transpose(-1, -2)) / math.sqrt(qf.size(-1))
+    s = fn(s, 0, 0, None, None)
+    if causal:
+        L, S = s.shape[-2:]
+        s = s.masked_fill(torch.ones(L, S, dtype=torch.bool).triu(1), float("-inf"))
+    return torch.matmul(torch.softmax(s, dim=-1), vf)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_score_mod_callables_of_the_softcap_signature(D):
+    """softcap.py:49 calls score_mod(attn_weight, N, Hq, query, key) with any callable; the ones the kernel can apply
+    in registers are recognised by tracing them."""
+    B, H, S = 2, 4, 400
+    q, k, v = qkv(B, H, H, S, D, seed=D + 40, amp=5.0)
+    qf, kf, vf = f32(q, k, v)
+    g = torch.Generator().manual_seed(41)
+    rel = torch.randn(H, S, S, generator=g)
+
+    def gym_softcap(score, b, h, q_idx, kv_idx):  # attn_gym.mods.generate_tanh_softcap(30, approx=False), as published
+        return 30 * torch.tanh(score / 30)
+
+    def other_spelling(score, b, h, q_idx, kv_idx):
+        return torch.tanh(score * 0.125).mul(8.0)
+
+    def temperature(score, b, h, q_idx, kv_idx):
+        return score / 2.5
+
+    def capped_then_shifted(score, b, h, q_idx, kv_idx):
+        return 10.0 * torch.tanh(score / 10.0) + rel_dev - 3.0
+
+    def scaled_cap(score, b, h, q_idx, kv_idx):  # post != 1 / pre
+        return 6.0 * torch.tanh(0.5 * score)
+
+    for fn in (gym_softcap, other_spelling, temperature, scaled_cap):
+        assert_parity(A.attention_softcapped(q, k, v, score_mod=fn), _eager_softcapped(qf, kf, vf, fn), fn.__name__)
+    rel_dev = rel.to(DEV)
+    out = A.attention_softcapped(q, k, v, score_mod=capped_then_shifted, is_causal=True)
+    rel_dev = rel
+    assert_parity(out, _eager_softcapped(qf, kf, vf, capped_then_shifted, causal=True), "capped_then_shifted")
+
+
+def test_score_mod_the_kernel_cannot_apply_is_refused():
+    q, k, v = qkv(1, 2, 2, 64, 64, seed=50)
+    for fn in (lambda s, b, h, qi, ki: torch.relu(s),
+               lambda s, b, h, qi, ki: torch.tanh(torch.tanh(s)),
+               lambda s, b, h, qi, ki: s * s,
+               lambda s, b, h, qi, ki: -s):
+        with pytest.raises(NotImplementedError):
+            A.attention_softcapped(q, k, v, score_mod=fn)

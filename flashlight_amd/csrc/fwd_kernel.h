@@ -1083,7 +1083,8 @@ void fwd_kernel(const KParams p) {
     };
 
     if constexpr (kDoc) dma_wait<0>();  // the tile list (issued first thing) has landed
-    __syncthreads();  // the previous branch (if any) is done with the LDS buffers
+    // (the previous branch is done with the LDS buffers; every wave's share of the tile list is visible to all)
+    if (br > 0 || kDoc) __syncthreads();
     if constexpr (kDoc) n_list = __builtin_amdgcn_readfirstlane((int)tlist[-1]);
     if (n_list > 0) {
       constexpr int NS = T::NS;

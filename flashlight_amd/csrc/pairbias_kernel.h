@@ -71,8 +71,9 @@ struct PairBiasTraits {
   static constexpr bool GATE = GATE_;
   static constexpr int D = 32, BN = 64, NW = 4, NT = 256, BM = 128;
   static constexpr int NTI = NKB / 2;    // key tiles per batch entry
-  static constexpr int NS = 4;           // K/V tiles resident in LDS; transfers run three tiles ahead
-  static_assert(NKB % 2 == 0 && NTI >= 4, "whole tiles; the wait bookkeeping needs four tiles per entry");
+  static constexpr int NS = 6;           // K/V tiles resident in LDS
+  static constexpr int AHEAD = NS - 1;   // transfers run this many tiles ahead of their use
+  static_assert(NKB % 2 == 0 && NTI >= 2, "whole tiles");
   static constexpr int TILE_BYTES = BN * D * 2;
   static constexpr int K_OFF = 0, V_OFF = NS * TILE_BYTES, LDS_BYTES = 2 * NS * TILE_BYTES;
 };
@@ -261,14 +262,13 @@ void pairbias_kernel(const PParams p) {
     l_run += rs;
   };
 
-  // ---- prologue: queries of the first entry, the first three tiles, scores of the first block
+  // ---- prologue: queries of the first entry, the first AHEAD tiles, scores of the first block
   ex8 qf[2];
   {
     const uint64_t qb0 = qbase + (uint64_t)((int64_t)fb0 * p.qs[0] * 2);
     u32x4 a = load16_counted(qb0, qoff), b = load16_counted(qb0, qoff + 32u);
-    issue_tile(0, 0, 0);
-    issue_tile(0, 1, 1);
-    issue_tile(0, 2, 2);
+#pragma unroll
+    for (int j = 0; j < T::AHEAD; ++j) issue_tile(j / NTI, j % NTI, j);
     dma_wait<0>();
     pin_loaded(a);
     pin_loaded(b);
@@ -284,11 +284,21 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
 
-  // Operations a wave issues, in order, per entry:  at the barrier point of tile t (in the tile's second block): the two
-  // transfers of the tile three ahead, and at t == 0 also the gate loads of this entry (4, if there is a gate) and the
-  // query loads of the next (2); after the entry's last block: 4 stores.  The barrier point of tile t waits for the
-  // transfers of tile t + 1, issued two barrier points earlier; kAllowed(t) counts what was issued after them.
+  // Operations a wave issues, in order, per entry:  at the barrier point of tile t: the two transfers of the tile AHEAD
+  // tiles on, and at t == 0 also the gate loads of this entry (4, if there is a gate) and the query loads of the next (2);
+  // after the entry's last block: 4 stores.  The barrier point of tile t waits for the transfers of tile t + 1, issued
+  // AHEAD - 1 barrier points earlier; allowed(t) counts what was issued after them: the extras of that point, and
+  // everything of the points since.  Running far ahead keeps the stores out of the way: a wait completes in issue
+  // order, so a transfer issued after the stores is only known to have landed once the stores are acknowledged, and
+  // with AHEAD = 5 that is first asked four tiles after them.
   constexpr int NI = 2 + (kGate ? 4 : 0);
+  constexpr int AHEAD = T::AHEAD;
+  auto extras = [](int j) constexpr { const int t = ((j % NTI) + NTI) % NTI; return (t == 0 ? NI : 0) + (t == NTI - 1 ? 4 : 0); };
+  auto allowed = [extras](int t) constexpr {
+    int n = extras(t + 1 - AHEAD);
+    for (int j = t + 2 - AHEAD; j < t; ++j) n += 2 + extras(j);
+    return n;
+  };
   for (int item = 0; item < n_items; ++item) {
     const int slot0 = (item * NTI) % NS;
     u32x4 qn_a, qn_b;        // next entry's query fragments, in flight from tile 0 on
@@ -305,10 +315,12 @@ void pairbias_kernel(const PParams p) {
         constexpr bool last_block = kb == NKB - 1;
         if constexpr (b == 0) {
           // barrier point of tile t, before anything of the tile after it is touched
-          constexpr int kAllowed = 2 + (t == 1 || t == 2 ? NI : 0) + (t == 0 || t == 1 ? 4 : 0);
+          // (the last point of an entry also takes the loads of point 0 into use: only the transfers issued since may stay out)
+          constexpr int kAllowed = t == NTI - 1 && 2 * (NTI - 2) < allowed(t) ? 2 * (NTI - 2) : allowed(t);
+          static_assert(kAllowed < 64, "vmcnt is a 6-bit counter");
           dma_wait<kAllowed>();
           __syncthreads();  // tile t + 1 is visible; everyone is done with tile t - 1, whose slot the new tile takes
-          issue_tile(item + (t + 3) / NTI, (t + 3) % NTI, (slot + 3) % NS);
+          issue_tile(item + (t + AHEAD) / NTI, (t + AHEAD) % NTI, (slot + AHEAD) % NS);
           if constexpr (t == 0) {
             if constexpr (kGate) {
               const uint64_t gb = gbase + (uint64_t)(fbc * p.gs[0] * 2);

@@ -58,7 +58,8 @@ class FlAttnBwdParams(C.Structure):
         ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
         ("dq_strides", C.c_int64 * 4), ("dk_strides", C.c_int64 * 4), ("dv_strides", C.c_int64 * 4),
         ("delta", C.c_void_p),
-        ("reserved", C.c_int32 * 8),
+        ("dscores", C.c_void_p),
+        ("reserved", C.c_int32 * 6),
     ]
 
 
@@ -359,12 +360,16 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
              *, scale: Optional[float] = None, mask_kind: int = MASK_NONE, window: int = 0, prefix: int = 0,
              doc_ids: Optional[torch.Tensor] = None, alibi_heads: int = 0, softcap: float = 0.0,
              validate_only: bool = False, dropout_p: float = 0.0, dropout_seed: int = 0, static_scratch: bool = False,
-             grads: Optional[Sequence[torch.Tensor]] = None):
+             grads: Optional[Sequence[torch.Tensor]] = None, biases: Sequence[tuple[torch.Tensor, int]] = (),
+             dscores: Optional[torch.Tensor] = None):
     """Gradients (dq, dk, dv) of `attn_fwd` called with the same arguments (dropout rate and seed included); `out` and `lse` are what that call
     returned and filled, `dout` [B, Hq, Lq, Dv] the gradient of its result.  Three launches on the current stream.
     `grads` = (dq, dk, dv) receives the results when given.  `static_scratch` goes through `fl_attn_bwd_static`: nothing
     is allocated here beyond the results, the library's own static device array serves as scratch (calls that may
-    overlap on one GPU must not both use it)."""
+    overlap on one GPU must not both use it).
+    `biases` are the forward's bias operands (positional masks only); `dscores`, a zero-filled contiguous float32
+    [B, Hq, Lq, Lk] tensor, then receives the gradient with respect to the scores, from which the caller sums the
+    gradient of each operand over the axes it broadcasts over."""
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
         _require_gpu_half(name, t, q if isinstance(q, torch.Tensor) and q.dtype in _HALF_TYPES else None)
@@ -378,9 +383,13 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
         raise ValueError("lse must be the contiguous float32 [B, Hq, Lq] tensor the forward filled")
     fwd, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                             (), None, False, 0.0, None, dropout_p, dropout_seed,
+                             biases, None, False, 0.0, None, dropout_p, dropout_seed,
                              alloc_workspace=validate_only or not static_scratch)
     fwd.lse = lse.data_ptr()
+    if dscores is not None:
+        if dscores.dtype != torch.float32 or tuple(dscores.shape) != (B, Hq, Lq, Lk) or not dscores.is_contiguous() or \
+                dscores.device != q.device:
+            raise ValueError("dscores must be a contiguous float32 [B, Hq, Lq, Lk] tensor on the inputs' device")
     if grads is not None:
         dq, dk, dv = grads
         for g, like in ((dq, q), (dk, k), (dv, v)):
@@ -395,6 +404,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     b.fwd = fwd
     b.dout, b.dq, b.dk, b.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     b.delta = None if delta is None else delta.data_ptr()
+    b.dscores = None if dscores is None else dscores.data_ptr()
     b.dout_strides[:] = _strides4(dout)
     b.dq_strides[:] = _strides4(dq)
     b.dk_strides[:] = _strides4(dk)

@@ -656,8 +656,13 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   const fl_attn_params* p = &b->fwd;
   int rc = validate(p, nullptr);
   if (rc) return rc;
-  if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
-    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands, gate, differential attention and the dump hook are not supported");
+  if (p->gate || p->diff || p->attended_dump)
+    return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
+  const bool has_bias = p->bias[0] || p->bias[1];
+  if (has_bias && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind) || p->dropout_threshold))
+    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands go with positional masks only (no ALiBi, soft-cap, document mask or dropout)");
+  if (b->dscores && !has_bias) return fail(FL_ERR_ARG, "backward: dscores is only written for calls with bias operands");
+  if (b->dscores && reinterpret_cast<uintptr_t>(b->dscores) % 16) return fail(FL_ERR_ALIGN, "backward: dscores must be 16-byte aligned");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
   if ((rc = check_ptr("dout", b->dout, 16)) || (rc = check_ptr("dq", b->dq, 8)) || (rc = check_ptr("dk", b->dk, 8)) ||
       (rc = check_ptr("dv", b->dv, 8)) || (rc = check_ptr("delta", b->delta, 16)) ||
@@ -668,7 +673,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
       (rc = check_strides("o", p->o_strides, 8)))
     return rc;
   if (reinterpret_cast<uintptr_t>(p->o) % 16) return fail(FL_ERR_ALIGN, "backward: o must be 16-byte aligned");
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < 6; ++i)
     if (b->reserved[i] != 0) return fail(FL_ERR_ARG, "reserved[%d] must be 0", i);
   // per-lane byte offsets inside one staged tile (up to 128 rows) are 32-bit
   const int64_t worst = std::max(std::max(p->q_strides[2], p->k_strides[2]), std::max(p->v_strides[2], b->dout_strides[2]));
@@ -683,11 +688,14 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     want = fl::F_DOC;
   }
   if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() has excluded document masks
+  if (has_bias) want = fl::F_BIAS;
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)
       in = &fl::kBwdInstances[i];
-  if (!in) return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d (64 and 128 are compiled)", p->Dqk);
+  if (!in)
+    return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d with features 0x%x (compiled: 64 and 128; 32 "
+                "without score modification or with bias operands)", p->Dqk, want);
   if (out) *out = in;
   g_err[0] = 0;
   return 0;
@@ -750,6 +758,13 @@ int fl_attn_bwd(const fl_attn_bwd_params* b, void* stream_) {
   bp.drop_seed[0] = p->dropout_seed[0];
   bp.drop_seed[1] = p->dropout_seed[1];
   bp.drop_rescale = 65536.0f / (65536.0f - (float)p->dropout_threshold);
+  for (int nb = 0; nb < 2; ++nb) {
+    bp.bias[nb] = p->bias[nb];
+    for (int i = 0; i < 4; ++i) bp.bbs[nb][i] = p->bias_strides[nb][i];
+    bp.bdiv[nb] = p->bias_batch_div[nb] > 0 ? p->bias_batch_div[nb] : 1;
+    bp.bias_f32[nb] = p->bias_dtype[nb] == FL_F32;
+  }
+  bp.dscores = b->dscores;
   if (is_doc(p->mask_kind)) {
     const int blocks = (p->Lk + fl::kDocBlock - 1) / fl::kDocBlock;
     const int total = p->B * blocks;

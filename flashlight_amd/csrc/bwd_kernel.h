@@ -49,6 +49,13 @@ struct BParams {
   uint32_t drop_thr;      // as in KParams: 0 = no dropout
   uint32_t drop_seed[2];
   float drop_rescale;
+  // Bias operands (F_BIAS), addressed as in the forward: element (batch / bdiv, head, query, key) through bbs, 16-bit
+  // elements of the call's type or fp32.  They are read from global memory where they are used.
+  const void* bias[2];
+  int64_t bbs[2][4];
+  int32_t bdiv[2];
+  int32_t bias_f32[2];
+  float* dscores;  // optional [B, Hq, Lq, Lk]: d(loss) / d(score), written by the dQ kernel for the tiles it visits
 };
 
 // delta[b, h, q] = -sum_d dO[b, h, q, d] * O[b, h, q, d]; one row per group of DV / 8 lanes.
@@ -113,8 +120,9 @@ __global__ __launch_bounds__(T::NT) __attribute__((amdgpu_waves_per_eu(T::WAVES_
 void bwd_kernel(const BParams p) {
   constexpr int D = T::D, ROLE = T::ROLE, TB = T::TB, BT = T::BT, KS = T::KS, DB = T::DB, NT = T::NT;
   constexpr uint32_t FEAT = T::FEAT;
-  constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC;
+  constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC, kBias = FEAT & F_BIAS;
   constexpr bool kDQ = ROLE == ROLE_DQ;
+  static_assert(!kBias || !(kAlibi || kSoftcap || kDoc || (FEAT & F_DROPOUT)), "bias operands go with positional masks only");
   using E = typename T::Elem;  // pointers in BParams are typed bf16_t whatever E is: 16 opaque bits
   typedef E ex8 __attribute__((ext_vector_type(8)));
   typedef E ex4 __attribute__((ext_vector_type(4)));
@@ -321,6 +329,20 @@ void bwd_kernel(const BParams p) {
     }
     return skip;
   };
+  // Sum of the bias operands at (query, key) of head `hd` (positions inside the sequences)
+  auto bias_at = [&](int qpos, int kpos, int hd) FL_INLINE -> float {
+    float b = 0.f;
+    if constexpr (kBias) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        if (p.bias[nb] == nullptr) continue;
+        const int64_t off = (int64_t)(batch / p.bdiv[nb]) * p.bbs[nb][0] + (int64_t)hd * p.bbs[nb][1] +
+                            (int64_t)qpos * p.bbs[nb][2] + (int64_t)kpos * p.bbs[nb][3];
+        b += p.bias_f32[nb] ? static_cast<const float*>(p.bias[nb])[off] : (float)static_cast<const E*>(p.bias[nb])[off];
+      }
+    }
+    return b;
+  };
   // One step: the tile in ring slot `slot` against the owner operands.
   auto run_step = [&](int s, int slot, bool full, bool doc_uniform) FL_INLINE {
     const int t0 = step_tile(s) * BT;
@@ -434,6 +456,10 @@ void bwd_kernel(const BParams p) {
                 s2 = __builtin_fmaf(x, p.scale_log2, c0);
               }
               if constexpr (kAlibi) s2 = __builtin_fmaf(slope_off, (float)off, s2);
+              if constexpr (kBias) {
+                const int sp = min(sbase + off, slen - 1), op = min(opos, olen - 1);
+                s2 = __builtin_fmaf(bias_at(kDQ ? op : sp, kDQ ? sp : op, shead), kLog2e, s2);
+              }
               float pw = fast_exp2(s2);
               if (!full) {  // workgroup-uniform
                 bool ok = (off <= hi) & (off >= lo);
@@ -508,6 +534,12 @@ void bwd_kernel(const BParams p) {
                 ds = kDeltaInit ? pd[sb][i] * x2[sb][i] : pd[sb][i] * (x2[sb][i] + (kDQ ? delta_o : dl4[e]));
               }
               dsf[2 * sb + i / 8][i % 8] = (E)ds;
+              if constexpr (kBias && kDQ) {
+                // the gradient with respect to the score (no soft-cap goes with a bias: d(score) / d(qk * scale) = 1)
+                const int key = sbase + 8 * g + e;
+                if (p.dscores != nullptr && opos < p.Lq && key < p.Lk)
+                  p.dscores[(((int64_t)batch * p.Hq + ohead) * p.Lq + opos) * p.Lk + key] = ds;
+              }
             }
           }
         }

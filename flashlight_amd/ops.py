@@ -113,6 +113,79 @@ def _backward(ctx, dout, dlse):
 attn_fwd_lse.register_autograd(_backward, setup_context=_setup_context)
 
 
+class _BiasAttention(torch.autograd.Function):
+    """The forward with bias operands for calls that will be differentiated (the reference's Evoformer function and its
+    dense `score_mod` tensors, attention_variants/evoformer.py:24-27, alibi.py:26-30; the reference itself has no
+    backward).  The backward kernels return, next to dq, dk, dv, the gradient with respect to the scores; the gradient of
+    a bias operand is that array summed over the batch entries and axes the operand broadcasts over."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, mask_kind, window, prefix, div0, div1, bias0, bias1):
+        out = _alloc_out(q, v, False, False)
+        lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
+        biases = [(b, d) for b, d in ((bias0, div0), (bias1, div1)) if b is not None]
+        _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, biases=biases, out=out, lse=lse)
+        ctx.save_for_backward(q, k, v, out, lse, bias0, bias1)
+        ctx.args = (scale, mask_kind, window, prefix, div0, div1)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, bias0, bias1 = ctx.saved_tensors
+        scale, mask_kind, window, prefix, div0, div1 = ctx.args
+        biases = [(b, d) for b, d in ((bias0, div0), (bias1, div1)) if b is not None]
+        want = [b is not None and ctx.needs_input_grad[9 + i] for i, b in enumerate((bias0, bias1))]
+        dscores = None
+        if any(want):
+            dscores = torch.zeros((q.size(0), q.size(1), q.size(2), k.size(2)), dtype=torch.float32, device=q.device)
+        dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout.to(q.dtype), scale=scale, mask_kind=mask_kind, window=window,
+                                   prefix=prefix, biases=biases, dscores=dscores)
+        dbs = []
+        for b, d, w in ((bias0, div0, want[0]), (bias1, div1, want[1])):
+            if not w:
+                dbs.append(None)
+                continue
+            g = dscores.view(dscores.size(0) // d, d, *dscores.shape[1:]).sum(1)
+            axes = [i for i in range(4) if b.size(i) == 1 and g.size(i) != 1]
+            if axes:
+                g = g.sum(axes, keepdim=True)
+            dbs.append(g.to(b.dtype))
+        return dq, dk, dv, None, None, None, None, None, None, dbs[0], dbs[1]
+
+
+def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases, gate, diff,
+                    lambda_full, dropout_p, dropout_seed):
+    """The forward as a composition every part of which has a backward: the sigmoid gate and the difference of the two
+    softmax branches are applied as tensor operations around the fused calls (one call per branch and per slab of as
+    many value columns as the head dim, since the backward kernels take equal head dims)."""
+    if diff:
+        h, hk, d = q.size(1) // 2, k.size(1) // 2, q.size(3)
+        if v.size(3) % d:
+            raise NotImplementedError("gradients of differential attention need a value width that is a multiple of the head dim")
+        parts = []
+        for br in range(2):
+            qb, kb = q[:, br * h:(br + 1) * h], k[:, br * hk:(br + 1) * hk]
+            parts.append(torch.cat([_differentiable(qb, kb, v[..., c:c + d], scale=scale, mask_kind=mask_kind, window=window,
+                                                    prefix=prefix, doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap,
+                                                    biases=biases, gate=None, diff=False, lambda_full=0.0,
+                                                    dropout_p=dropout_p, dropout_seed=dropout_seed).float()
+                                    for c in range(0, v.size(3), d)], dim=-1))
+        out = (parts[0] - lambda_full * parts[1]).to(q.dtype)
+    elif biases:
+        if dropout_p > 0.0 or alibi_heads or softcap or doc_ids is not None:
+            raise NotImplementedError("gradients with bias operands are built for positional masks without ALiBi, soft-cap, "
+                                      "document ids or dropout")
+        bl = list(biases) + [(None, 1)] * (2 - len(biases))
+        out = _BiasAttention.apply(q, k, v, None if scale is None else float(scale), int(mask_kind), int(window), int(prefix),
+                                   int(bl[0][1]), int(bl[1][1]), bl[0][0], bl[1][0])
+    else:
+        out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
+                              int(prefix), doc_ids, int(alibi_heads), float(softcap), dropout_p, int(dropout_seed))
+    if gate is not None:
+        out = (out.float() * torch.sigmoid(gate.float())).to(q.dtype)
+    return out
+
+
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
              dropout_seed=None) -> torch.Tensor:
@@ -135,15 +208,16 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
             dropout_seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
     else:
         dropout_seed = 0
-    if (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) or \
-            (dropout_p > 0.0 and torch.compiler.is_compiling()):
-        if biases or gate is not None or diff or seq_major_out:
-            raise NotImplementedError(
-                "no backward is implemented for bias operands, the sigmoid gate or differential attention: call under "
-                "torch.no_grad() (or detach the inputs) if only the forward is wanted")
-        out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
-                              int(prefix), doc_ids, int(alibi_heads), float(softcap), dropout_p, int(dropout_seed))
-        return out
+    wants_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (q, k, v, gate, *(b for b, _ in biases)))
+    if wants_grad or (dropout_p > 0.0 and torch.compiler.is_compiling()):
+        if torch.compiler.is_compiling() and (biases or gate is not None or diff):
+            raise NotImplementedError("gradients with bias operands, the gate or differential attention are not traceable "
+                                      "by torch.compile: differentiate the eager call")
+        # (the result comes back in [B, H, L, Dv] memory order whatever seq_major_out asks for)
+        return _differentiable(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
+                               alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
+                               lambda_full=lambda_full, dropout_p=dropout_p, dropout_seed=dropout_seed)
     if torch.compiler.is_compiling():
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),

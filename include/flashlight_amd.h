@@ -158,8 +158,11 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * softmax attention, recomputing the weights from the forward's row statistics.
  * `fwd` describes the forward call whose gradients are wanted: same q, k, v, sizes, scale, mask and score
  * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
- * kind, grouped-query heads, ALiBi, the tanh soft-cap; Dqk == Dv in {64, 128}.  Not supported (FL_ERR_UNSUPPORTED):
- * bias operands, gate, differential attention, the attended_dump hook.
+ * kind, grouped-query heads, ALiBi, the tanh soft-cap; Dqk == Dv in {64, 128}, and {32, 64, 128} without a score
+ * modification or with bias operands.  Bias operands (fwd.bias, as in the forward) go with positional masks only, not
+ * with ALiBi, a soft-cap, a document mask or dropout.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
+ * (both are compositions of calls that are supported: out * sigmoid(gate); one call per branch and half of the value
+ * columns), the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
  * receive the gradients (element type fwd.dtype like dout; strides in elements, last stride 1, others multiples of 8).
  * delta: caller-provided scratch of B * Hq * Lq floats; delta and fwd.lse must be 16-byte aligned.
@@ -173,7 +176,13 @@ typedef struct fl_attn_bwd_params {
   void* dv;
   int64_t dq_strides[4], dk_strides[4], dv_strides[4];
   float* delta;
-  int32_t reserved[8]; /* must be 0 */
+  /* Optional, with bias operands: fp32 [B, Hq, Lq, Lk], contiguous, 16-byte aligned.  Receives the gradient of the
+   * loss with respect to the score of every (query, key) pair, i.e. with respect to whatever was added to q k^T * scale:
+   * the gradient of a bias operand is this array summed over the axes (and batch entries) the operand broadcasts
+   * over.  Only key tiles that some query of the workgroup attends are written (zeros where a pair is masked inside
+   * them): clear the array before the call. */
+  float* dscores;
+  int32_t reserved[6]; /* must be 0 */
 } fl_attn_bwd_params;
 
 /* sizeof(fl_attn_bwd_params) in the loaded library. */

@@ -40,6 +40,26 @@ def test_oracle_gradients_against_finite_differences(name, fn):
     assert torch.autograd.gradcheck(lambda a, b, c: fn(a, b, c), (q, k, v), eps=1e-6, atol=1e-5, rtol=1e-4), name
 
 
+def test_oracle_gradients_of_bias_gate_and_branches_against_finite_differences():
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).requires_grad_(True)  # noqa: E731
+    # Evoformer layout [B, N, S, H, D] with a mask bias, a pair bias and the gate
+    q, k, v, gate = (mk(1, 2, 4, 2, 3) for _ in range(4))
+    b1, b2 = mk(1, 2, 1, 1, 4), mk(1, 1, 2, 4, 4)
+    assert torch.autograd.gradcheck(lambda q, k, v, b1, b2, gate: O.attention_evoformer(q, k, v, [b1, b2], gate=gate),
+                                    (q, k, v, b1, b2, gate), eps=1e-6, atol=1e-5, rtol=1e-4)
+    # dense score_mod tensor (the ALiBi signature), causal
+    q, k, v = _tiny()
+    dense = mk(2, 5, 5)
+    assert torch.autograd.gradcheck(
+        lambda q, k, v, d: O.attention_alibi(q, k, v, score_mod=lambda L, S: d, enable_gqa=True, is_causal=True, honor_causal=True),
+        (q, k, v, dense), eps=1e-6, atol=1e-5, rtol=1e-4)
+    # differential attention: q, k [B, 2H, S, d], v [B, H, S, 2d]
+    q, k, v = mk(1, 4, 5, 3), mk(1, 4, 5, 3), mk(1, 2, 5, 6)
+    assert torch.autograd.gradcheck(lambda q, k, v: O.diff_attention(q, k, v, lambda_full=0.6, is_causal=True), (q, k, v),
+                                    eps=1e-6, atol=1e-5, rtol=1e-4)
+
+
 def test_backward_abi_validation():
     lib = _ffi.load_library()
     assert lib.fl_bwd_params_sizeof() == C.sizeof(_ffi.FlAttnBwdParams)
@@ -66,7 +86,9 @@ def test_backward_abi_validation():
         (lambda b: setattr(b, "delta", 0), -1, "delta"),
         (lambda b: setattr(b, "dout", 0xA0008), -7, "dout"),
         (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),
-        (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1)), -4, "not supported"),
+        (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
+                    setattr(b.fwd, "softcap", 30.0)), -4, "positional masks only"),
+        (lambda b: setattr(b, "dscores", 0xF0000), -5, "dscores"),
         (lambda b: (setattr(b.fwd, "gate", 0x70000), b.fwd.gate_strides.__setitem__(slice(0, 4), list(b.fwd.o_strides))),
          -4, "not supported"),
         (lambda b: b.reserved.__setitem__(3, 1), -5, "reserved"),
@@ -77,21 +99,21 @@ def test_backward_abi_validation():
         mutate(b)
         assert rc(b) == code and word in _ffi.last_error(), (_ffi.last_error(), word)
         assert lib.fl_attn_bwd(C.byref(b), None) == code  # the same check runs before any launch
+    assert rc(params(D=32)) == 0, _ffi.last_error()
     b = params(D=32)
-    assert rc(b) == -4 and "head dim" in _ffi.last_error()
+    b.fwd.alibi_heads = 4  # head dim 32 is compiled without score modifications (or with bias operands) only
+    assert rc(b) == -4 and "kernel" in _ffi.last_error()
+    # bias operands are taken with positional masks, and then dscores may be given
+    b = params()
+    b.fwd.bias[0], b.fwd.bias_batch_div[0] = 0x60000, 1
+    b.fwd.bias_strides[0][:] = (0, 0, b.fwd.Lk, 1)
+    b.dscores = 0xF0000
+    assert rc(b) == 0, _ffi.last_error()
+    b.dscores = 0xF0004
+    assert rc(b) == -7 and "dscores" in _ffi.last_error()
     b = params(D=64, Dv=128)
     b.fwd.diff = 0
     assert rc(b) == -4
-
-
-def test_front_end_refuses_to_differentiate_what_has_no_backward():
-    # checked before anything touches a GPU
-    q = torch.randn(1, 3, 16, 2, 32).bfloat16().requires_grad_(True)
-    with pytest.raises(NotImplementedError, match="no backward"):
-        A.attention_reference(q, q, q, [torch.zeros(1, 1, 2, 16, 16).bfloat16()])
-    qd = torch.randn(1, 4, 16, 64).bfloat16().requires_grad_(True)
-    with pytest.raises(NotImplementedError, match="no backward"):
-        A.diffattn(qd, qd, torch.randn(1, 2, 16, 128).bfloat16())
 
 
 # ---- the kernels ---------------------------------------------------------------------------------------------------------------
@@ -259,3 +281,80 @@ def test_gradients_under_torch_compile_equal_eager():
     torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd_lse.default,
                           (q.detach().requires_grad_(True), k, v, -1.0, 1, 0, 0, None, 0, 0.0),
                           test_utils=("test_schema", "test_faketensor", "test_autograd_registration"))
+
+
+# ---- gradients through bias operands, the gate and the two branches of differential attention ------------------------------
+
+def _compare(name, got, want):
+    for what, g_, w_ in zip(name[1], got, want):
+        assert g_ is not None and tuple(g_.shape) == tuple(w_.shape), f"{name[0]}: {what}"
+        scale = max(1.0, w_.abs().max().item())
+        assert_parity(g_.float() / scale, w_.float() / scale, f"{name[0]}: {what}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("D", [64, 128])
+def test_gradients_dense_score_mod(D, causal):
+    """attention_pytorch_alibi with an arbitrary dense tensor (alibi.py:26-30): gradients reach q, k, v and the tensor."""
+    B, Hq, Hkv, L = 2, 4, 2, 200
+    q, k, v, dout = _inputs(B, Hq, Hkv, L, D, seed=300 + D)
+    g = torch.Generator().manual_seed(9)
+    dense = torch.randn(Hq, L, L, generator=g)
+    outs = []
+    for dev, dtype, mod in ((DEV, torch.bfloat16, A), ("cpu", torch.float32, None)):
+        qq, kk, vv = (t.detach().to(dev).to(dtype).requires_grad_(True) for t in (q, k, v))
+        dd = dense.to(dev).requires_grad_(True)
+        if mod is not None:
+            out = A.attention_pytorch_alibi(qq, kk, vv, score_mod=lambda L_, S_: dd, enable_gqa=True, is_causal=causal)
+        else:
+            out = O.attention_alibi(qq, kk, vv, score_mod=lambda L_, S_: dd, enable_gqa=True, is_causal=causal,
+                                    honor_causal=True)
+        out.backward(dout.to(dev).to(out.dtype).reshape(out.shape))
+        outs.append((out.detach().reshape(B, Hq, L, D), qq.grad, kk.grad, vv.grad, dd.grad))
+    torch.cuda.synchronize()
+    _compare((f"dense score_mod D={D} causal={causal}", ("out", "dq", "dk", "dv", "dbias")), outs[0], outs[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,N,S,H,D", [(1, 6, 96, 2, 32), (2, 3, 70, 3, 64)])
+def test_gradients_evoformer_biases_and_gate(B, N, S, H, D):
+    """attention_reference with the benchmark's two biases (evoformer.py:46-47) and the gate: gradients of every operand."""
+    g = torch.Generator().manual_seed(B + S)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)  # noqa: E731
+    q, k, v, gate, dout = (mk(B, N, S, H, D) for _ in range(5))
+    b1, b2 = mk(B, N, 1, 1, S), mk(B, 1, H, S, S)
+    res = []
+    for dev, dtype in ((DEV, torch.bfloat16), ("cpu", torch.float32)):
+        ts = [t.detach().to(dev).to(dtype).requires_grad_(True) for t in (q, k, v, b1, b2, gate)]
+        fn = A.attention_reference if dev == DEV else O.attention_evoformer
+        out = fn(ts[0], ts[1], ts[2], [ts[3], ts[4]], gate=ts[5])
+        out.backward(dout.to(dev).to(out.dtype))
+        res.append([out.detach()] + [t.grad for t in ts])
+    torch.cuda.synchronize()
+    _compare((f"evoformer {B, N, S, H, D}", ("out", "dq", "dk", "dv", "dbias1", "dbias2", "dgate")), res[0], res[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("causal", [False, True])
+def test_gradients_differential_attention(causal):
+    B, H, S, d = 2, 2, 200, 64
+    g = torch.Generator().manual_seed(17)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)  # noqa: E731
+    q, k, v, dout = mk(B, 2 * H, S, d), mk(B, 2 * H, S, d), mk(B, H, S, 2 * d), mk(B, H, S, 2 * d)
+    res = []
+    for dev, dtype in ((DEV, torch.bfloat16), ("cpu", torch.float32)):
+        ts = [t.detach().to(dev).to(dtype).requires_grad_(True) for t in (q, k, v)]
+        fn = A.diffattn if dev == DEV else O.diff_attention
+        out = fn(ts[0], ts[1], ts[2], lambda_full=0.8, is_causal=causal)
+        out.backward(dout.to(dev).to(out.dtype))
+        res.append([out.detach()] + [t.grad for t in ts])
+    torch.cuda.synchronize()
+    _compare((f"diffattn causal={causal}", ("out", "dq", "dk", "dv")), res[0], res[1])
+
+
+@pytest.mark.gpu
+def test_plain_gradients_at_head_dim_32():
+    q, k, v, dout = _inputs(2, 4, 2, 300, 32, seed=32)
+    _check("causal D=32", *VARIANTS["causal"], q, k, v, dout)
+    _check("sliding D=32", *VARIANTS["sliding"], q, k, v, dout)

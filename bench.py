@@ -37,8 +37,8 @@ def parse_args():
 
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 256 MiB copy's readings);
-# commands and raw values: profiles/fwd_kernel_d128_cfg1_counters.md
-MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 410.6e6, "cfg1/sliding_window": 311.4e6}
+# commands and raw values: profiles/fwd_kernel_d128_cfg1_{vanilla,causal,sliding_window}.md
+MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 407.1e6, "cfg1/sliding_window": 326.4e6}
 
 FLUSH_BYTES = 512 << 20  # twice the 256 MB memory-side cache: zeroing it evicts the operands of the previous launch
 CPU_CAP_S = 12.0         # wall-clock cap per configuration for the eager CPU timing
@@ -48,17 +48,22 @@ def event_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def time_launches(fn, iters: int, warmup: int = 20, flush=None):
+def time_launches(fn, iters: int, warmup: int = 20, flush=None, flush_by: str = "zero"):
     """Trimmed mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
     current stream (the stream the kernels are launched on).  With `flush` (a device buffer larger than the caches)
     the buffer is zeroed before every bracketed launch, like the reference's harness does (benchmarks/_utils.py:145-151
-    there): the launch then reads its operands from HBM."""
+    there): the launch then reads its operands from HBM.  Zeroing leaves the memory-side cache full of modified lines,
+    whose write-back shares the HBM with the launch that follows (a plain copy of 268 MB takes 0.072 ms after it, 0.049
+    ms after a flush that only reads); `flush_by="read"` sums the buffer instead: cold operands, clean cache."""
     for _ in range(warmup):
         fn()
     pairs = [event_pair() for _ in range(iters)]
     for a, b in pairs:
         if flush is not None:
-            flush.zero_()
+            if flush_by == "zero":
+                flush.zero_()
+            else:
+                flush.view(torch.int32).sum()
         a.record()
         fn()
         b.record()
@@ -216,12 +221,14 @@ def main():
     for w in cfg1:
         mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(50, args.steps))
         cold_ms, cold_med = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush)
+        clean_ms, _ = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush, flush_by="read")
         tf = w.flops / mean_ms / 1e9
         variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
                             "ms_back_to_back": time_back_to_back(lambda w=w: w.call(tens), iters=max(50, args.steps), warmup=20),
                             "ms_flushed": cold_ms, "ms_flushed_median": cold_med, "tflops_flushed": w.flops / cold_ms / 1e9,
-                            "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
-                            "roofline": roofline_entry(w, mean_ms, W), "roofline_flushed": roofline_entry(w, cold_ms, W)}
+                            "ms_cold": clean_ms, "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
+                            "roofline": roofline_entry(w, mean_ms, W), "roofline_flushed": roofline_entry(w, cold_ms, W),
+                            "roofline_cold": roofline_entry(w, clean_ms, W)}
     dom = max(cfg1, key=lambda w: variants[w.name]["ms"])  # the launch that dominates the step
     dv = variants[dom.name]
     roofline = {"bound": "mfma", "kernel": f"fl::fwd_kernel ({dom.name})", "achieved": dv["tflops"],
@@ -240,16 +247,30 @@ def main():
             t = w.make(dev)
             mean_ms = time_back_to_back(lambda: w.call(t), iters=100, warmup=50)
             cold_ms, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush)
+            clean_ms, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush, flush_by="read")
             tf = w.flops / mean_ms / 1e9
             others[w.name] = {"ms": mean_ms, "timing": "warm: 100 launches back to back after 50 warm-up launches; "
                                                        "flushed: 50 launches, 512 MB zeroed before each",
                               "ms_flushed": cold_ms, "tflops": tf, "tflops_flushed": w.flops / cold_ms / 1e9,
                               "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS, "unmasked_flops": w.flops,
-                              "min_bytes": w.min_bytes, "roofline": roofline_entry(w, mean_ms, W),
-                              "roofline_flushed": roofline_entry(w, cold_ms, W)}
+                              "ms_cold": clean_ms, "min_bytes": w.min_bytes, "roofline": roofline_entry(w, mean_ms, W),
+                              "roofline_flushed": roofline_entry(w, cold_ms, W), "roofline_cold": roofline_entry(w, clean_ms, W)}
             del t
             torch.cuda.empty_cache()
-    del flush
+    # What a plain device-to-device copy with the headline configuration's traffic (268 MB read + written) takes under the
+    # same three cache states: the practical HBM roofline of this part for the launches that are bound by it.
+    src = torch.empty(128 << 20, dtype=torch.uint8, device=dev).random_()
+    dst = torch.empty_like(src)
+    copy_bytes = 2 * src.numel()
+    hbm_cal = {"bytes": copy_bytes,
+               "ms_warm": time_launches(lambda: dst.copy_(src), iters=50)[1],
+               "ms_flushed": time_launches(lambda: dst.copy_(src), iters=50, warmup=5, flush=flush)[1],
+               "ms_cold": time_launches(lambda: dst.copy_(src), iters=50, warmup=5, flush=flush, flush_by="read")[1]}
+    for entry, w in [(variants[w.name], w) for w in cfg1] + [(others[w.name], w) for w in all_w if w.name in others]:
+        if w.bound == "hbm":  # fraction of the plain copy's rate on the same number of bytes in the same cache state
+            entry["vs_copy"] = {st: hbm_cal["ms_" + st] * w.min_bytes / copy_bytes / entry[key]
+                                for st, key in (("warm", "ms"), ("flushed", "ms_flushed"), ("cold", "ms_cold"))}
+    del flush, src, dst
 
     # What the matrix pipe alone sustains on this part (same MFMA instruction, operands in registers, nothing else
     # running), on N(0,1) operands like the benchmark's and on zeros, and the forward itself on all-zero inputs: the
@@ -291,7 +312,9 @@ def main():
                    "seed": cfg1[0].seed, "unmasked_flops_per_step": step_flops},
         "pct_mfma_peak": 100 * step_flops / wall_ms / 1e9 / W.PEAK_BF16_TFLOPS,
         "cache_state": "value and ms_per_step: warm (steps back to back on the same operands); *_flushed: 512 MB zeroed "
-                       "before each launch",
+                       "before each launch (the reference harness's recipe; the cache is then full of modified lines); "
+                       "*_cold: 512 MB read before each launch (cold operands, clean cache)",
+        "hbm_calibration": hbm_cal,
         "ms_per_step_flushed": step_flushed_ms, "value_flushed": step_flops / step_flushed_ms / 1e9,
         "peak_used_TFLOPs": W.PEAK_BF16_TFLOPS,
         "variants": variants, "roofline": roofline, "other_configs": others, "power_context": context,

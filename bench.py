@@ -296,6 +296,22 @@ def main():
         # the dominant launch against what the matrix pipe alone sustains on the same kind of data in this run
         context["roofline_frac_vs_mfma_only_randn"] = roofline["achieved"] / context["mfma_only_randn_operands_TFLOPs"]
         del tens, zeros, ops
+        # The forward's step as a register-only probe (zero operands): nominal-clock cycles per 32 x 32 block of scores
+        # and SIMD for the MFMAs alone, for the step as the forward has it (softmax vector work, data dependences), and
+        # with the K / V fragments read from LDS; last, the forward itself on zero inputs.
+        sink2 = torch.empty(2 * n_cu * 256, dtype=torch.float32, device=dev)
+        ladder = {}
+        for D in (64, 128):
+            for level, tag in ((0, "mfma_only"), (2, "step_in_registers"), (3, "plus_lds_operand_reads")):
+                blocks = [0]
+
+                def run(D=D, level=level):
+                    blocks[0] = _ffi.probe_step(D, level, 1000, 2 * n_cu, sink2)
+                ms = time_back_to_back(run, iters=20, warmup=5)
+                # two workgroups of four waves per compute unit: every SIMD hosts two waves
+                ladder[f"d{D}_{tag}"] = ms * 1e-3 * 2.4e9 / (2 * blocks[0])
+        ladder["d128_forward_zero_inputs"] = 16 * 32 / (context["vanilla_on_zero_inputs_TFLOPs"] / W.PEAK_BF16_TFLOPS)
+        context["cycles_per_block_at_2p4GHz"] = ladder
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)

@@ -125,6 +125,8 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_ipa_pack.argtypes = [C.POINTER(FlIpaPackParams), C.c_void_p]
     lib.fl_probe_mfma_rate.restype = C.c_int
     lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.fl_probe_step.restype = C.c_int
+    lib.fl_probe_step.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
         raise RuntimeError(f"{p}: ABI version {lib.fl_version()} != expected {ABI_VERSION}")
     if lib.fl_params_sizeof() != C.sizeof(FlAttnParams):
@@ -474,3 +476,17 @@ def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink:
     if rc != 0:
         raise FlashlightError(rc, "fl_probe_mfma_rate rejected its arguments" if rc < 0 else "probe launch failed")
     return float(n_workgroups) * 8 * iters * 32 * 32768.0
+
+
+def probe_step(head_dim: int, level: int, iters: int, n_workgroups: int, sink: torch.Tensor) -> int:
+    """Launches the step-structure probe on the current stream (measurement aid, include/flashlight_amd.h) and returns
+    the number of 32 x 32 score blocks every wave works through; `sink`: float32 device tensor of n_workgroups * 256
+    elements."""
+    if sink.dtype != torch.float32 or not sink.is_cuda or sink.numel() < n_workgroups * 256:
+        raise ValueError("sink must be a float32 device tensor of n_workgroups * 256 elements")
+    stream = torch.cuda.current_stream(sink.device).cuda_stream
+    rc = load_library().fl_probe_step(int(head_dim), int(level), int(iters), int(n_workgroups), sink.data_ptr(),
+                                      C.c_void_p(stream))
+    if rc != 0:
+        raise FlashlightError(rc, "fl_probe_step rejected its arguments" if rc < 0 else "probe launch failed")
+    return 2 * int(iters)

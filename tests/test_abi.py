@@ -189,3 +189,6 @@ def test_probe_rejects_bad_arguments_without_a_gpu(lib):
     aligned = (addr + 15) // 16 * 16
     assert lib.fl_probe_mfma_rate(C.c_void_p(aligned), 0, 1, 1, C.c_void_p(aligned), None) == -5
     assert lib.fl_probe_mfma_rate(C.c_void_p(aligned + 2), 1, 1, 1, C.c_void_p(aligned), None) == -7
+    assert lib.fl_probe_step(64, 2, 1, 1, None, None) == -5
+    assert lib.fl_probe_step(64, 4, 1, 1, C.c_void_p(aligned), None) == -5
+    assert lib.fl_probe_step(96, 2, 1, 1, C.c_void_p(aligned), None) == -4

@@ -1107,11 +1107,63 @@ void fwd_kernel(const KParams p) {
         if (j < n_list) load_v(entry_tile(ent[j]), j);
       dma_wait<0>();
       __syncthreads();
+      // The list positions whose tiles are not EMPTY for this wave's rows form one run [a_live, b_live) (an EMPTY tile
+      // between two others, possible under unsorted document ids, counts as live: it is computed and masked).  Before
+      // and after its run the wave takes part in the transfers and barriers of the steps and computes nothing: the far
+      // side of the diagonal, the keys outside a window, other documents.
+      int a_live = 0, b_live = n_list;
+      if constexpr (kDoc) {
+        int a = n_list, b = 0;
+        for (int base = 0; base < n_list; base += 64) {
+          const int i = base + lane;
+          const bool live = i < n_list && ((tlist[min(i, n_list - 1)] >> (16 + 2 * wave)) & 3u) != (unsigned)TILE_EMPTY;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+          if (m != 0) {
+            a = min(a, base + (int)__builtin_ctzll(m));
+            b = max(b, base + 64 - (int)__builtin_clzll(m));
+          }
+        }
+        a_live = __builtin_amdgcn_readfirstlane(a);
+        b_live = __builtin_amdgcn_readfirstlane(b);
+      } else if constexpr (FEAT & F_ALIBI) {  // positions run from the last tile down
+        a_live = max(0, t_lo + n_list - 1 - e_hi);
+        b_live = min(n_list, t_lo + n_list - e_lo);
+      } else {
+        a_live = max(0, e_lo - t_lo);
+        b_live = min(n_list, e_hi - t_lo + 1);
+      }
+      if (a_live >= b_live) a_live = b_live = n_list;  // nothing for this wave
+      // A run starts at ring slot 0 (the unrolled loop below enters there, and a second way in would cost registers: the
+      // compiler then keeps both score buffers alive through both steps): up to NS - 1 EMPTY tiles ahead of it are taken
+      // into the run and computed and masked like any other.
+      else a_live -= a_live % NS;
       f32x16 s_a[KB][QB], s_b[KB][QB];
-      qk(s_a, 0);
-      score_mods(s_a, entry_tile(ent[0]), 0);
+      if (a_live == 0 && b_live > 0) {
+        qk(s_a, 0);
+        score_mods(s_a, entry_tile(ent[0]), 0);
+      }
       __syncthreads();  // K slot 0 may be overwritten from here on
 
+      // What every wave does in every step but the workgroup's last, whatever it computes: at the top, the transfers of K
+      // NS tiles on into the slot whose tile was consumed in the previous step, and of V NS - 1 tiles on; at the end,
+      // the wait for the transfers the next step reads (later ones may stay in flight) and the barrier.
+      auto issue_loads = [&](int slot) FL_INLINE -> bool {
+        const bool steady = pos + NS < n_list;
+        if (steady) {
+          load_k(entry_tile(ent[NS]), slot);
+          load_b(entry_tile(ent[NS]), slot);  // the bias of this step's tile was consumed at the end of the previous step
+        }
+        if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
+        return steady;
+      };
+      auto end_step = [&](bool steady) FL_INLINE {
+        if (steady) dma_wait<(NS - 2) * LPS>(); else dma_wait<0>();
+        __syncthreads();
+        ++pos;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) ent[j] = ent[j + 1];
+        ent[NS] = list_entry(pos + NS);
+      };
       // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
       // maxima, and the (rare) rescale.
       auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e, int vslot) FL_INLINE {
@@ -1134,12 +1186,7 @@ void fwd_kernel(const KParams p) {
         constexpr int slot = decltype(slot_tag)::value;
         // K slot `slot` held this tile's K and V slot `slot - 1` the previous tile's V: both were last read before the
         // barrier that ended the previous step
-        const bool steady = pos + NS < n_list;
-        if (steady) {
-          load_k(entry_tile(ent[NS]), slot);
-          load_b(entry_tile(ent[NS]), slot);  // the bias of this step's tile was consumed at the end of the previous step
-        }
-        if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
+        const bool steady = issue_loads(slot);
         settle(sc, ent[0], slot);
         ex8 pf[QB][2 * KB];
         // Raised issue priority while this wave has matrix work: of the two waves sharing a SIMD, the one that is in
@@ -1159,20 +1206,25 @@ void fwd_kernel(const KParams p) {
           sched_second_product<NB, (16 * KB * QB * mod_ops + NB - 1) / NB>();
         }
         __builtin_amdgcn_s_setprio(0);
-        // the next step reads K and V transfers issued NS - 2 steps ago: later ones may stay in flight
-        if (steady) dma_wait<(NS - 2) * LPS>(); else dma_wait<0>();
-        __syncthreads();
-        ++pos;
-#pragma unroll
-        for (int j = 0; j < NS; ++j) ent[j] = ent[j + 1];
-        ent[NS] = list_entry(pos + NS);
+        end_step(steady);
       };
-      int last_slot = 0;  // ring slot of the final tile; its scores are in s_a when the slot is even
+      // steps before this wave's run: transfers and barriers only, except that the step before the run forms the scores
+      // of the run's first tile, as every step does for the tile after it
+      while (pos < a_live && pos + 1 < n_list) {
+        const bool steady = issue_loads(pos % NS);
+        if (pos + 1 == a_live) {
+          qk(s_a, 0);
+          score_mods(s_a, entry_tile(ent[1]), 0);
+        }
+        end_step(steady);
+      }
+      if (pos >= a_live && pos < b_live) {
+      int last_slot = 0;  // ring slot of the run's final tile; its scores are in s_a when the slot is even
       bool more = true;
       while (more) {
         more = static_while<0, NS>([&](auto idx) FL_INLINE  {
           constexpr int slot = decltype(idx)::value;
-          if (!(pos + 1 < n_list)) {
+          if (!(pos + 1 < b_live)) {
             last_slot = slot;
             return false;
           }
@@ -1180,7 +1232,11 @@ void fwd_kernel(const KParams p) {
           return true;
         });
       }
-      // last tile: nothing left to prefetch
+      // the run's last tile: no scores of a next tile to form; the step's transfers and barrier only if the workgroup
+      // has further steps
+      const bool more_steps = pos + 1 < n_list;
+      bool steady_tail = false;
+      if (more_steps) steady_tail = issue_loads(last_slot);
       static_while<0, NS>([&](auto idx) FL_INLINE  {
         constexpr int slot = decltype(idx)::value;
         if (last_slot != slot) return true;
@@ -1198,6 +1254,13 @@ void fwd_kernel(const KParams p) {
         pv_mma(pf, slot, vfirst, std::false_type{});
         return false;
       });
+      if (more_steps) end_step(steady_tail);
+      }
+      // steps after the run
+      while (pos + 1 < n_list) {
+        const bool steady = issue_loads(pos % NS);
+        end_step(steady);
+      }
     }
 
     // ---- normalise this branch ---------------------------------------------------------------------------------

@@ -220,3 +220,21 @@ def test_rewritten_dense_document_differential_and_msa_on_gpu():
     Q, K, V = (torch.randn(1, 3, 104, 2, 32, generator=g).to(BF).to(dev) for _ in range(3))
     mask, pair = torch.randn(1, 3, 1, 1, 104, generator=g).to(BF).to(dev), torch.randn(1, 1, 2, 104, 104, generator=g).to(BF).to(dev)
     _check_on_gpu(lambda Q, K, V, m, p: E.msa_row(Q, K, V, [m, p]), (Q, K, V, mask, pair), "msa row")
+
+
+@pytest.mark.gpu
+def test_a_fully_masked_row_comes_out_as_zeros():
+    """A row whose keys a run-time mask all removes: eager PyTorch averages the values uniformly under a finite fill
+    (every score equals the fill) and returns NaN under -inf; the rewritten graph treats any fill <= -1e9 as "not
+    attended" and returns zeros for such a row, like every entry of the package.  Rows with a key left are unaffected."""
+    dev = "cuda"
+    q, k, v = _qkv(N=1, Hq=2, Hkv=2, L=72, E=64, dev=dev, seed=21)
+    bias = torch.zeros(1, 2, 72, 72, device=dev)
+    pad = torch.ones(1, 72, dtype=torch.bool, device=dev)   # every key padded away: all rows fully masked
+    torch._dynamo.reset()
+    got = torch.compile(E.learned_bias, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, bias, pad)
+    assert torch.count_nonzero(got).item() == 0
+    pad[0, :5] = False                                         # five keys left: ordinary attention over them
+    torch._dynamo.reset()
+    got = torch.compile(E.learned_bias, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, bias, pad)
+    assert_parity(got, E.learned_bias(q.float(), k.float(), v.float(), bias, pad), "five keys left")

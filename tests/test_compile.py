@@ -5,6 +5,8 @@ import torch
 
 import flashlight_amd.attention_variants as A
 import flashlight_amd.ops  # noqa: F401  (registers the operator)
+import oracle as O
+from tests.conftest import assert_parity
 
 BF = torch.bfloat16
 
@@ -37,6 +39,14 @@ def _qkv(B=1, Hq=4, Hkv=2, S=64, D=64):
             torch.randn(B, Hkv, S, D, generator=g).to(BF))
 
 
+ORACLE = {
+    "vanilla": lambda q, k, v: O.attention_vanilla(q, k, v, enable_gqa=True),
+    "causal": lambda q, k, v: O.attention_causal(q, k, v, enable_gqa=True),
+    "sliding": lambda q, k, v: O.attention_sliding_window(q, k, v, window_size=16, enable_gqa=True),
+    "prefix": lambda q, k, v: O.attention_prefix_lm(q, k, v, prefix_lengths=8, enable_gqa=True),
+    "alibi": lambda q, k, v: O.attention_alibi(q, k, v, score_mod=q.size(-3), enable_gqa=True),
+    "softcap": lambda q, k, v: O.attention_softcapped(q, k, v, score_mod=30.0, enable_gqa=True),
+}
 CASES = {
     "vanilla": lambda q, k, v: A.attention_pytorch(q, k, v, enable_gqa=True),
     "causal": lambda q, k, v: A.attention_pytorch_causal(q, k, v, enable_gqa=True),
@@ -94,6 +104,9 @@ def test_compiled_equals_eager_on_gpu():
         torch._dynamo.reset()
         got = torch.compile(fn, backend="aot_eager", fullgraph=True)(q, k, v)
         assert torch.equal(got, fn(q, k, v)), name
+        # and against the CPU oracle: the compiled graph computes the right thing, not merely the same thing
+        want = ORACLE[name](q.float().cpu(), k.float().cpu(), v.float().cpu())
+        assert_parity(got.reshape(want.shape), want, f"compiled {name}")
     Q, K, V, G = (torch.randn(1, 3, 104, 2, 32, device=dev).to(BF) for _ in range(4))
     pair, mask = torch.randn(1, 1, 2, 104, 104, device=dev).to(BF), torch.randn(1, 3, 1, 1, 104, device=dev).to(BF)
     fn = lambda Q, K, V, m, p, G: A.attention_reference(Q, K, V, [m, p], gate=G)

@@ -101,7 +101,7 @@ def test_backward_abi_validation():
         assert lib.fl_attn_bwd(C.byref(b), None) == code  # the same check runs before any launch
     assert rc(params(D=32)) == 0, _ffi.last_error()
     b = params(D=32)
-    b.fwd.alibi_heads = 4  # head dim 32 is compiled without score modifications (or with bias operands) only
+    b.fwd.dropout_threshold = 1000  # no dropout kernels at head dim 32
     assert rc(b) == -4 and "kernel" in _ffi.last_error()
     # bias operands are taken with positional masks, and then dscores may be given
     b = params()

@@ -358,3 +358,8 @@ def test_plain_gradients_at_head_dim_32():
     q, k, v, dout = _inputs(2, 4, 2, 300, 32, seed=32)
     _check("causal D=32", *VARIANTS["causal"], q, k, v, dout)
     _check("sliding D=32", *VARIANTS["sliding"], q, k, v, dout)
+    _check("alibi+softcap+causal D=32", *VARIANTS["alibi+softcap+causal"], q, k, v, dout)
+    ids = torch.randint(0, 4, (2, 300), generator=torch.Generator().manual_seed(6)).sort(dim=1).values.to(DEV)
+    _check("document causal D=32",
+           lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids, enable_gqa=True, is_causal=True),
+           lambda q, k, v: O.attention_document_mask(q, k, v, ids, enable_gqa=True, is_causal=True), q, k, v, dout)

@@ -324,7 +324,7 @@ def attn_fwd(
         out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
     elif tuple(out.shape) != (B, Hq, Lq, Dv) or out.dtype != q.dtype or out.device != q.device:
         raise ValueError("out has the wrong shape, dtype or device")
-    if Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None and (diff or Dqk > 128):
+    if Dv > _MAX_DV_DIFF and Dv % _MAX_DV_DIFF == 0 and attended_dump is None and (diff or Dqk >= 128):
         # Value columns are independent of one another, so wide values go in slabs of _MAX_DV_DIFF columns, one launch
         # each, through strided views of v and out: a differential launch keeps two sets of output accumulators (the
         # reference's benchmark shape: q, k [B, 16, S, 128], v [B, 8, S, 256], diff_attn.py:33-38), and at head dim 256

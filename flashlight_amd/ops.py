@@ -8,6 +8,7 @@ Outside of tracing the front-ends call the C ABI directly (no dispatcher overhea
 """
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
@@ -186,6 +187,36 @@ def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi
     return out
 
 
+_HEAD_DIMS = (32, 64, 128)
+
+
+def _pad_head_dims(q, k, v, gate, diff):
+    """(q, k, v, gate) with zero columns appended up to a compiled head dim, or None when the head dims are compiled as
+    they are (32, 64, 128 for q, k and v alike; 256 for q and k with values in slabs of 128 columns; the 64/128 and
+    128/256 pairs of differential attention) or when no padding would help."""
+    dqk, dv = q.size(-1), v.size(-1)
+    if dqk != k.size(-1) or q.dim() != 4 or v.dim() != 4:
+        return None  # left to the binding's own checks
+    if diff:
+        if dv != 2 * dqk or dqk > 128:
+            return None
+        pq = next(p for p in (64, 128) if p >= dqk)
+        pv = 2 * pq
+    elif (dqk, dv) in ((32, 64), (64, 128)):
+        return None  # compiled pairs (invariant point attention's channel counts land on them)
+    elif dqk > 128 or dv > 128:
+        if dqk > 256:
+            return None
+        pq, pv = (256 if dqk > 128 else 128), -(-dv // 128) * 128
+    else:
+        pq = pv = next(p for p in _HEAD_DIMS if p >= max(dqk, dv))
+    if (pq, pv) == (dqk, dv):
+        return None
+    pad = torch.nn.functional.pad
+    return (pad(q, (0, pq - dqk)), pad(k, (0, pq - dqk)), pad(v, (0, pv - dv)),
+            None if gate is None else pad(gate, (0, pv - dv)))
+
+
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
              dropout_seed=None) -> torch.Tensor:
@@ -197,6 +228,17 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     generator, so `torch.manual_seed` reproduces a run; the same seed gives the same decisions in forward and backward."""
     dropout_p = float(dropout_p)
     _ffi.dropout_threshold(dropout_p)  # range check
+    padded = _pad_head_dims(q, k, v, gate, diff)
+    if padded is not None:
+        # head dims between the compiled ones: zero columns change neither q.k nor the columns of the result that are
+        # kept (the reference's generated kernel takes any head dim up to 256, monkeypatch/fusion/_common.py:4)
+        qp, kp, vp, gp = padded
+        if scale is None:
+            scale = 1.0 / math.sqrt(q.size(-1))
+        out = dispatch(qp, kp, vp, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
+                       alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gp, diff=diff, lambda_full=lambda_full,
+                       seq_major_out=seq_major_out, dropout_p=dropout_p, dropout_seed=dropout_seed)
+        return out[..., :v.size(-1)]
     if dropout_p > 0.0:
         if biases or gate is not None or diff or seq_major_out:
             raise NotImplementedError("dropout is built for positional masks, the in-kernel ALiBi term and the soft-cap; not "

@@ -166,3 +166,42 @@ def test_score_mod_the_kernel_cannot_apply_is_refused():
                lambda s, b, h, qi, ki: -s):
         with pytest.raises(NotImplementedError):
             A.attention_softcapped(q, k, v, score_mod=fn)
+
+
+@pytest.mark.parametrize("D,Dv", [(16, 16), (48, 48), (80, 80), (96, 96), (112, 64), (40, 100), (192, 192), (128, 256), (72, 160)])
+def test_head_dims_between_the_compiled_ones(D, Dv):
+    """Any head dim up to 256 (the reference's generated kernel takes them in one block, monkeypatch/fusion/_common.py:4):
+    q, k and v are zero-padded to a compiled head dim and the result is cut back; the default scale is that of the
+    unpadded head dim."""
+    q, k, v = qkv(2, 4, 2, 260, D, Dv, seed=D + Dv)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch(q, k, v, enable_gqa=True), O.attention_vanilla(qf, kf, vf, enable_gqa=True), "vanilla")
+    assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(qf, kf, vf, enable_gqa=True),
+                  "causal")
+    assert_parity(A.attention_pytorch_sliding_window(q, k, v, window_size=50, enable_gqa=True),
+                  O.attention_sliding_window(qf, kf, vf, window_size=50, enable_gqa=True), "sliding")
+
+
+def test_gradients_at_a_head_dim_between_the_compiled_ones():
+    D = 96
+    g = torch.Generator().manual_seed(96)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)  # noqa: E731
+    q, k, v, dout = mk(2, 4, 150, D), mk(2, 2, 150, D), mk(2, 2, 150, D), mk(2, 4, 150, D)
+    res = []
+    for dev, dtype in ((DEV, torch.bfloat16), ("cpu", torch.float32)):
+        ts = [t.detach().to(dev).to(dtype).requires_grad_(True) for t in (q, k, v)]
+        fn = A.attention_pytorch_causal if dev == DEV else O.attention_causal
+        out = fn(ts[0], ts[1], ts[2], enable_gqa=True)
+        out.backward(dout.to(dev).to(out.dtype).reshape(out.shape))
+        res.append([out.detach().reshape(2, 4, 150, D)] + [t.grad for t in ts])
+    for what, got, want in zip(("out", "dq", "dk", "dv"), res[0], res[1]):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, what)
+
+
+def test_differential_attention_at_head_dim_48():
+    g = torch.Generator().manual_seed(48)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)  # noqa: E731
+    q, k, v = mk(2, 4, 200, 48), mk(2, 4, 200, 48), mk(2, 2, 200, 96)
+    out = A.diffattn(q.to(DEV), k.to(DEV), v.to(DEV), lambda_full=0.5, is_causal=True)
+    assert_parity(out, O.diff_attention(q.float(), k.float(), v.float(), lambda_full=0.5, is_causal=True), "diff d=48")

@@ -269,7 +269,10 @@ def test_front_end_errors_on_gpu_tensors():
         A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(8), enable_gqa=True)
     q48 = torch.randn(1, 2, 64, 48, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
-        A.attention_pytorch(q48, q48, q48)
+        _ffi.attn_fwd(q48, q48, q48)  # the C ABI takes compiled head dims only (the front-ends pad others)
+    q320 = torch.randn(1, 2, 64, 320, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
+        A.attention_pytorch(q320, q320, q320)  # beyond 256
 
 
 def test_mfma_rate_probe_runs_and_sums_products():

@@ -101,6 +101,33 @@ def test_document_mask_with_alibi_and_softcap(D, cap, causal):
 
 
 @pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("cap", [None, 12.0])
+@pytest.mark.parametrize("causal", [False, True])
+def test_document_mask_with_dense_bias_and_gate(D, cap, causal):
+    """Documents + a dense additive term per head (bf16, shared by the batch) + a row-broadcast fp32 term + the gate."""
+    B, H, S = 2, 4, 520
+    q, k, v = qkv(B, H, H, S, D, seed=D + 11, amp=2.0)
+    g = torch.Generator().manual_seed(23)
+    ids = torch.sort(torch.randint(0, 5, (B, S), generator=g), dim=1).values
+    if causal:
+        ids = ids[:, torch.randperm(S, generator=g)]  # ids in no order: the tile lists have holes
+    dense = (torch.randn(1, H, S, S, generator=g) * 1.5).to(torch.bfloat16)
+    row = torch.randn(B, 1, 1, S, generator=g)
+    gate = torch.randn(B, H, S, D, generator=g).to(torch.bfloat16)
+    out = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_DOCUMENT_CAUSAL if causal else _ffi.MASK_DOCUMENT, doc_ids=ids.to(DEV),
+                       softcap=cap or 0.0, biases=[(dense.to(DEV), B), (row.to(DEV), 1)], gate=gate.to(DEV))
+
+    def masked(qi, ki):
+        m = ids[:, qi.view(-1)].view(B, 1, -1, 1) != ids[:, ki.view(-1)].view(B, 1, 1, -1)
+        return (m | (ki > qi)) if causal else m
+
+    qf, kf, vf = f32(q, k, v)
+    ref = _softmax_attention(qf, kf, vf, 1.0 / math.sqrt(D), masked=masked, softcap=cap,
+                             bias=lambda qi, ki: (dense.float()[..., qi.view(-1), :], row))
+    assert_parity(out, ref * torch.sigmoid(gate.float()), f"D={D} cap={cap} causal={causal}")
+
+
+@pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("gqa", [False, True])
 def test_dense_score_mod_with_softcap(D, gqa):
     """attention_pytorch_alibi(score_mod=<any callable>, softcap=...): cap first, then the dense tensor (alibi.py:26-30)."""

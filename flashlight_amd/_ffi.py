@@ -148,7 +148,7 @@ def _check(rc: int) -> None:
 
 
 def _strides4(t: torch.Tensor) -> Sequence[int]:
-    return tuple(int(s) for s in t.stride())
+    return t.stride()
 
 
 _HALF_TYPES = {torch.bfloat16: FL_BF16, torch.float16: FL_F16}
@@ -175,9 +175,24 @@ def _require_gpu_bf16(name: str, t: torch.Tensor) -> None:
 
 def _dim_contiguous(t: torch.Tensor) -> torch.Tensor:
     """The kernels address [batch, head, seq, dim] through strides but need dim contiguous and 16-byte rows."""
+    if t.is_contiguous():  # (copying would change nothing; decided first because it is the common case)
+        return t
     if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
         return t.contiguous()
     return t
+
+
+def _launch_on(device: torch.device, entry, params) -> None:
+    """Calls `entry(&params, stream)` with `device` current and torch's current stream of that device."""
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
+        # (the raw-stream getter skips the Stream object; it is what torch's own generated code calls)
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        stream = raw(torch.cuda.current_device()) if raw is not None else torch.cuda.current_stream().cuda_stream
+        _check(entry(C.byref(params), C.c_void_p(stream)))
+        return
+    with torch.cuda.device(device):
+        _check(entry(C.byref(params), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
 
 
 def dropout_threshold(p: float) -> int:
@@ -350,9 +365,7 @@ def attn_fwd(
     if validate_only:
         _check(lib.fl_attn_validate(C.byref(p)))
         return out
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        _check(lib.fl_attn_fwd(C.byref(p), C.c_void_p(stream)))
+    _launch_on(q.device, lib.fl_attn_fwd, p)
     # tensors in `keep` were last used on the current stream; the caching allocator orders their reuse after it
     del keep
     return out
@@ -414,9 +427,7 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     if validate_only:
         _check(lib.fl_attn_bwd_validate(C.byref(b)))
         return dq, dk, dv
-    with torch.cuda.device(q.device):
-        entry = lib.fl_attn_bwd_static if use_static else lib.fl_attn_bwd
-        _check(entry(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    _launch_on(q.device, lib.fl_attn_bwd_static if use_static else lib.fl_attn_bwd, b)
     del keep, delta
     return dq, dk, dv
 

@@ -9,12 +9,13 @@ from .. import _ffi, ops
 
 
 def check_heads(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, enable_gqa: bool) -> None:
-    for name, t in (("query", query), ("key", key), ("value", value)):
-        if t.dim() != 4:
-            raise ValueError(f"{name} must be [N, H, L, E], got shape {tuple(t.shape)}")
-    hq, hkv = query.size(1), key.size(1)
-    if value.size(1) != hkv:
-        raise ValueError(f"key has {hkv} heads but value has {value.size(1)}")
+    if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+        for name, t in (("query", query), ("key", key), ("value", value)):
+            if t.dim() != 4:
+                raise ValueError(f"{name} must be [N, H, L, E], got shape {tuple(t.shape)}")
+    hq, hkv = query.shape[1], key.shape[1]
+    if value.shape[1] != hkv:
+        raise ValueError(f"key has {hkv} heads but value has {value.shape[1]}")
     if enable_gqa:
         if hq % hkv:
             raise ValueError(f"enable_gqa: {hq} query heads are not a multiple of {hkv} key/value heads")

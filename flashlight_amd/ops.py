@@ -194,7 +194,9 @@ def _pad_head_dims(q, k, v, gate, diff):
     """(q, k, v, gate) with zero columns appended up to a compiled head dim, or None when the head dims are compiled as
     they are (32, 64, 128 for q, k and v alike; 256 for q and k with values in slabs of 128 columns; the 64/128 and
     128/256 pairs of differential attention) or when no padding would help."""
-    dqk, dv = q.size(-1), v.size(-1)
+    dqk, dv = q.shape[-1], v.shape[-1]
+    if not diff and dqk == dv and dqk in _HEAD_DIMS:
+        return None  # the common case, decided first: this runs on every call
     if dqk != k.size(-1) or q.dim() != 4 or v.dim() != 4:
         return None  # left to the binding's own checks
     if diff:

@@ -1,0 +1,94 @@
+"""The library launches on the caller's current stream, allocates nothing and never synchronises, so a call can sit on a
+side stream or inside a captured HIP graph.  Every replay of a graph is compared with the eager call on the same
+operands (bit-exact: the same kernels on the same data), with eager work and synchronisations between the replays."""
+import pytest
+import torch
+
+import flashlight_amd.attention_variants as A
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _qkv(B, H, S, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    return tuple(torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(3))
+
+
+def test_launches_on_the_callers_stream():
+    q_old, k, v = _qkv(2, 4, 300, 64, 1)
+    q_new = _qkv(2, 4, 300, 64, 2)[0]
+    want = A.attention_pytorch_causal(q_new, k, v)
+    torch.cuda.synchronize()
+    q = q_old.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(40_000_000)  # the side stream is busy for a while; the default stream is idle
+        q.copy_(q_new)                 # queued behind the sleep
+        out = A.attention_pytorch_causal(q, k, v)  # on the side stream it sees the new q; on any other, the old one
+    side.synchronize()
+    assert torch.equal(out, want)
+
+
+def _replay_against_eager(make_call, operands, fresh):
+    """Captures make_call(*operands) once, then replays it on three fresh sets of operand values."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture, as torch.cuda.graph asks
+        make_call(*operands)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = make_call(*operands)
+    for i in range(3):
+        for dst, src in zip(operands, fresh(i)):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = make_call(*operands)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i}"
+
+
+def test_forward_in_a_captured_graph_causal_gqa():
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(2, 8, 257, 128, generator=g).to(torch.bfloat16).to(DEV)
+    k, v = (torch.randn(2, 2, 257, 128, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+
+    def fresh(i):
+        gi = torch.Generator().manual_seed(100 + i)
+        return (torch.randn(q.shape, generator=gi).to(torch.bfloat16).to(DEV),
+                torch.randn(k.shape, generator=gi).to(torch.bfloat16).to(DEV),
+                torch.randn(v.shape, generator=gi).to(torch.bfloat16).to(DEV))
+
+    _replay_against_eager(lambda a, b, c: A.attention_pytorch_causal(a, b, c, enable_gqa=True), (q, k, v), fresh)
+
+
+def test_forward_in_a_captured_graph_document_mask():
+    """Three kernels per call (the two pre-pass kernels and the forward) and a workspace from torch's allocator."""
+    q, k, v = _qkv(2, 4, 700, 64, 5)
+    ids = torch.sort(torch.randint(0, 6, (2, 700), generator=torch.Generator().manual_seed(6)), dim=1).values.to(DEV)
+
+    def fresh(i):
+        gi = torch.Generator().manual_seed(200 + i)
+        new_ids = torch.sort(torch.randint(0, 3 + 4 * i, (2, 700), generator=gi), dim=1).values.to(DEV)
+        return (*_qkv(2, 4, 700, 64, 300 + i), new_ids)
+
+    _replay_against_eager(lambda a, b, c, d: A.attention_pytorch_document_mask(a, b, c, d, is_causal=True),
+                          (q, k, v, ids), fresh)
+
+
+def test_forward_in_a_captured_graph_shared_bias_kernel():
+    g = torch.Generator().manual_seed(7)
+    shape = (1, 16, 256, 4, 32)
+    q, k, v, gate = (torch.randn(shape, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    bias = torch.randn(1, 1, 4, 256, 256, generator=g).to(torch.bfloat16).to(DEV)
+
+    def fresh(i):
+        gi = torch.Generator().manual_seed(400 + i)
+        return (*(torch.randn(shape, generator=gi).to(torch.bfloat16).to(DEV) for _ in range(4)),
+                torch.randn(bias.shape, generator=gi).to(torch.bfloat16).to(DEV))
+
+    _replay_against_eager(lambda a, b, c, d, e: A.attention_reference(a, b, c, [e], gate=d), (q, k, v, gate, bias), fresh)

@@ -92,3 +92,46 @@ def test_forward_in_a_captured_graph_shared_bias_kernel():
                 torch.randn(bias.shape, generator=gi).to(torch.bfloat16).to(DEV))
 
     _replay_against_eager(lambda a, b, c, d, e: A.attention_reference(a, b, c, [e], gate=d), (q, k, v, gate, bias), fresh)
+
+
+def test_training_step_in_a_captured_graph_with_the_static_scratch_backward():
+    """Forward with row statistics, then the backward that allocates nothing (`static_scratch`: the library's own
+    device array is its scratch), results into tensors made beforehand: the whole step is captured and replayed."""
+    from flashlight_amd import _ffi
+    B, Hq, Hkv, L, D = 2, 4, 2, 333, 64
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, Hq, L, D, generator=g).to(torch.bfloat16).to(DEV)
+    k, v = (torch.randn(B, Hkv, L, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    dout = torch.randn(B, Hq, L, D, generator=g).to(torch.bfloat16).to(DEV)
+    out, lse = torch.empty_like(q), torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+
+    def step(q_, k_, v_, dout_):
+        _ffi.attn_fwd(q_, k_, v_, mask_kind=_ffi.MASK_CAUSAL, out=out, lse=lse)
+        _ffi.attn_bwd(q_, k_, v_, out, lse, dout_, mask_kind=_ffi.MASK_CAUSAL, static_scratch=True, grads=grads)
+        return torch.cat([t.reshape(-1) for t in (out, *grads)])
+
+    def eager(q_, k_, v_, dout_):
+        o = torch.empty_like(q_)
+        s = torch.empty_like(lse)
+        _ffi.attn_fwd(q_, k_, v_, mask_kind=_ffi.MASK_CAUSAL, out=o, lse=s)
+        return torch.cat([t.reshape(-1) for t in (o, *_ffi.attn_bwd(q_, k_, v_, o, s, dout_, mask_kind=_ffi.MASK_CAUSAL))])
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(q, k, v, dout)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        flat = step(q, k, v, dout)
+    for i in range(3):
+        gi = torch.Generator().manual_seed(500 + i)
+        for t in (q, k, v, dout):
+            t.copy_(torch.randn(t.shape, generator=gi).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager(q, k, v, dout)
+        torch.cuda.synchronize()
+        assert torch.equal(flat, want), f"replay {i}"

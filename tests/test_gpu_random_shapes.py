@@ -32,12 +32,22 @@ def _case(seed):
 
 @pytest.mark.parametrize("seed", range(96))
 def test_random_shape(seed):
+    _run_case(seed, torch.bfloat16)
+
+
+@pytest.mark.parametrize("seed", range(200, 248))
+def test_random_shape_fp16(seed):
+    """The same draw with fp16 elements (every instance is compiled once per element type)."""
+    _run_case(seed, torch.float16)
+
+
+def _run_case(seed, dtype):
     c = _case(seed)
     g = torch.Generator().manual_seed(1000 + seed)
     B, Hq, Hkv, L, D = c["B"], c["Hkv"] * c["G"], c["Hkv"], c["L"], c["D"]
-    q = (torch.randn(B, Hq, L, D, generator=g) * c["amp"]).to(torch.bfloat16)
-    k = torch.randn(B, Hkv, L, D, generator=g).to(torch.bfloat16)
-    v = torch.randn(B, Hkv, L, D, generator=g).to(torch.bfloat16)
+    q = (torch.randn(B, Hq, L, D, generator=g) * c["amp"]).to(dtype)
+    k = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
     qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
     qf, kf, vf = q.float(), k.float(), v.float()
     kind = c["kind"]

@@ -41,42 +41,76 @@ def test_random_shape_fp16(seed):
     _run_case(seed, torch.float16)
 
 
-def _run_case(seed, dtype):
+def _functions(c, seed, g):
+    """(HIP front-end, oracle) as functions of (q, k, v) for the drawn case; `g` supplies the document ids."""
+    B, Hq, L = c["B"], c["Hkv"] * c["G"], c["L"]
+    kind = c["kind"]
+    if kind == "vanilla":
+        return (lambda q, k, v: A.attention_pytorch(q, k, v, enable_gqa=True),
+                lambda q, k, v: O.attention_vanilla(q, k, v, enable_gqa=True))
+    if kind == "causal":
+        return (lambda q, k, v: A.attention_pytorch_causal(q, k, v, enable_gqa=True),
+                lambda q, k, v: O.attention_causal(q, k, v, enable_gqa=True))
+    if kind == "sliding":
+        return (lambda q, k, v: A.attention_pytorch_sliding_window(q, k, v, window_size=c["window"], enable_gqa=True),
+                lambda q, k, v: O.attention_sliding_window(q, k, v, window_size=c["window"], enable_gqa=True))
+    if kind == "prefix":
+        return (lambda q, k, v: A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=c["prefix"], enable_gqa=True),
+                lambda q, k, v: O.attention_prefix_lm(q, k, v, prefix_lengths=c["prefix"], enable_gqa=True))
+    if kind in ("document", "document_causal"):
+        ids = torch.sort(torch.randint(0, c["ndocs"], (B, L), generator=g), dim=1).values
+        if seed % 3 == 0:
+            ids = ids[:, torch.randperm(L, generator=g)]  # ids in no order: tiles of one document lie scattered
+        causal = kind == "document_causal"
+        return (lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids.to(q.device), enable_gqa=True, is_causal=causal),
+                lambda q, k, v: O.attention_document_mask(q, k, v, ids.to(q.device), enable_gqa=True, is_causal=causal))
+    if kind == "alibi":
+        return (lambda q, k, v: A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(Hq), enable_gqa=True),
+                lambda q, k, v: O.attention_alibi(q, k, v, score_mod=Hq, enable_gqa=True))
+    if kind == "softcap_causal":
+        return (lambda q, k, v: A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(c["cap"]), enable_gqa=True,
+                                                       is_causal=True),
+                lambda q, k, v: O.attention_softcapped(q, k, v, score_mod=c["cap"], enable_gqa=True, is_causal=True,
+                                                       honor_causal=True))
+    return (lambda q, k, v: A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(Hq), enable_gqa=True,
+                                                      is_causal=True, softcap=c["cap"]),
+            lambda q, k, v: O.attention_alibi(q, k, v, score_mod=Hq, enable_gqa=True, is_causal=True, honor_causal=True,
+                                              softcap=c["cap"]))
+
+
+def _draw(seed, dtype):
     c = _case(seed)
     g = torch.Generator().manual_seed(1000 + seed)
     B, Hq, Hkv, L, D = c["B"], c["Hkv"] * c["G"], c["Hkv"], c["L"], c["D"]
     q = (torch.randn(B, Hq, L, D, generator=g) * c["amp"]).to(dtype)
     k = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
     v = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
-    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
-    qf, kf, vf = q.float(), k.float(), v.float()
-    kind = c["kind"]
-    if kind == "vanilla":
-        got, want = A.attention_pytorch(qd, kd, vd, enable_gqa=True), O.attention_vanilla(qf, kf, vf, enable_gqa=True)
-    elif kind == "causal":
-        got, want = A.attention_pytorch_causal(qd, kd, vd, enable_gqa=True), O.attention_causal(qf, kf, vf, enable_gqa=True)
-    elif kind == "sliding":
-        got = A.attention_pytorch_sliding_window(qd, kd, vd, window_size=c["window"], enable_gqa=True)
-        want = O.attention_sliding_window(qf, kf, vf, window_size=c["window"], enable_gqa=True)
-    elif kind == "prefix":
-        got = A.attention_pytorch_prefix_lm(qd, kd, vd, prefix_lengths=c["prefix"], enable_gqa=True)
-        want = O.attention_prefix_lm(qf, kf, vf, prefix_lengths=c["prefix"], enable_gqa=True)
-    elif kind in ("document", "document_causal"):
-        ids = torch.sort(torch.randint(0, c["ndocs"], (B, L), generator=g), dim=1).values
-        if seed % 3 == 0:
-            ids = ids[:, torch.randperm(L, generator=g)]  # ids in no order: tiles of one document lie scattered
-        causal = kind == "document_causal"
-        got = A.attention_pytorch_document_mask(qd, kd, vd, ids.to(DEV), enable_gqa=True, is_causal=causal)
-        want = O.attention_document_mask(qf, kf, vf, ids, enable_gqa=True, is_causal=causal)
-    elif kind == "alibi":
-        got = A.attention_pytorch_alibi(qd, kd, vd, score_mod=A.generate_alibi_bias_pytorch(Hq), enable_gqa=True)
-        want = O.attention_alibi(qf, kf, vf, score_mod=Hq, enable_gqa=True)
-    elif kind == "softcap_causal":
-        got = A.attention_softcapped(qd, kd, vd, score_mod=A.generate_tanh_softcap(c["cap"]), enable_gqa=True, is_causal=True)
-        want = O.attention_softcapped(qf, kf, vf, score_mod=c["cap"], enable_gqa=True, is_causal=True, honor_causal=True)
-    else:
-        got = A.attention_pytorch_alibi(qd, kd, vd, score_mod=A.generate_alibi_bias_pytorch(Hq), enable_gqa=True,
-                                        is_causal=True, softcap=c["cap"])
-        want = O.attention_alibi(qf, kf, vf, score_mod=Hq, enable_gqa=True, is_causal=True, honor_causal=True,
-                                 softcap=c["cap"])
+    return c, g, q, k, v
+
+
+def _run_case(seed, dtype):
+    c, g, q, k, v = _draw(seed, dtype)
+    hip_fn, oracle_fn = _functions(c, seed, g)
+    got, want = hip_fn(q.to(DEV), k.to(DEV), v.to(DEV)), oracle_fn(q.float(), k.float(), v.float())
     assert_parity(got.reshape(want.shape), want, str(c))
+
+
+@pytest.mark.parametrize("seed", range(300, 348))
+def test_random_shape_gradients(seed):
+    """dq, dk, dv of the same draws from the HIP backward kernels (the reference has no backward) against autograd through
+    the fp32 oracle, each scaled by its largest reference entry so that the forward's tolerance applies."""
+    c, g, q, k, v = _draw(seed, torch.bfloat16)
+    hip_fn, oracle_fn = _functions(c, seed, g)
+    dout = torch.randn(q.shape, generator=g).to(torch.bfloat16)
+
+    def grads(fn, dtype, device):
+        a, b, w = (t.to(device=device, dtype=dtype).requires_grad_(True) for t in (q, k, v))
+        out = fn(a, b, w)
+        out.backward(dout.to(device=device, dtype=out.dtype).reshape(out.shape))
+        return a.grad, b.grad, w.grad
+
+    got = grads(hip_fn, torch.bfloat16, DEV)
+    want = grads(oracle_fn, torch.float32, "cpu")
+    for name, x, y in zip(("dq", "dk", "dv"), got, want):
+        scale = max(1.0, y.abs().max().item())
+        assert_parity(x.float() / scale, y / scale, f"{name} {c}")

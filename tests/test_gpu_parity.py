@@ -501,6 +501,8 @@ def test_config0_shape_causal():
     (1, 5, 256, 8, True, torch.float16, False),      # fp16 elements
     (1, 33, 384, 2, True, torch.bfloat16, True),     # -inf entries in the bias (an additive mask)
     (1, 2, 256, 8, False, torch.bfloat16, False),    # two rows: chunks of one entry
+    (1, 21, 320, 2, False, torch.bfloat16, False),   # five tiles per entry without a gate
+    (1, 40, 384, 4, False, torch.float16, False),    # six tiles per entry without a gate, fp16
 ])
 def test_shared_bias_streaming_kernel(B, N, S, H, gate, dtype, inf):
     g = torch.Generator().manual_seed(31)

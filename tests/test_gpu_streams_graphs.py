@@ -135,3 +135,28 @@ def test_training_step_in_a_captured_graph_with_the_static_scratch_backward():
         want = eager(q, k, v, dout)
         torch.cuda.synchronize()
         assert torch.equal(flat, want), f"replay {i}"
+
+
+def test_results_repeat_bit_for_bit():
+    """No atomics and a fixed order of accumulation: the same call twice gives the same bits, forward and backward,
+    whatever else ran in between (here: the other call's launches, queued on the same stream)."""
+    from flashlight_amd import _ffi
+    g = torch.Generator().manual_seed(13)
+    q = torch.randn(2, 8, 700, 64, generator=g).to(torch.bfloat16).to(DEV)
+    k, v = (torch.randn(2, 2, 700, 64, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    dout = torch.randn(2, 8, 700, 64, generator=g).to(torch.bfloat16).to(DEV)
+    ids = torch.sort(torch.randint(0, 7, (2, 700), generator=g), dim=1).values.to(DEV)
+
+    def once():
+        outs = []
+        for kw in (dict(mask_kind=_ffi.MASK_CAUSAL), dict(mask_kind=_ffi.MASK_DOCUMENT_CAUSAL, doc_ids=ids),
+                   dict(mask_kind=_ffi.MASK_SLIDING, window=100, alibi_heads=8, softcap=20.0)):
+            lse = torch.empty(2, 8, 700, dtype=torch.float32, device=DEV)
+            out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+            outs += [out, lse, *_ffi.attn_bwd(q, k, v, out, lse, dout, **kw)]
+        return outs
+
+    first, second = once(), once()
+    torch.cuda.synchronize()
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)

@@ -36,9 +36,16 @@ def parse_args():
     return ap.parse_args()
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a 256 MiB copy's readings);
-# commands and raw values: profiles/fwd_kernel_d128_cfg1_{vanilla,causal,sliding_window}.md
-MEASURED_HBM_BYTES = {"cfg1/vanilla": 268.7e6, "cfg1/causal": 407.1e6, "cfg1/sliding_window": 326.4e6}
+def measured_hbm_bytes() -> dict:
+    """HBM bytes per launch of each workload as rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measured them (scaled by a
+    256 MiB copy's readings): profiles/hbm_traffic.json, written from the same profiler runs as the per-workload
+    summaries beside it (which give the commands and raw values).  Empty if the file is missing."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return {k: float(v) for k, v in json.load(f)["bytes_per_launch"].items()}
+    except (OSError, KeyError, ValueError):
+        return {}
 
 FLUSH_BYTES = 512 << 20  # twice the 256 MB memory-side cache: zeroing it evicts the operands of the previous launch
 CPU_CAP_S = 12.0         # wall-clock cap per configuration for the eager CPU timing
@@ -49,7 +56,7 @@ def event_pair():
 
 
 def time_launches(fn, iters: int, warmup: int = 20, flush=None, flush_by: str = "zero"):
-    """Trimmed mean / median duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
+    """Trimmed mean / median / plain mean duration (ms) of single launches of `fn`, each bracketed by its own pair of events on the
     current stream (the stream the kernels are launched on).  With `flush` (a device buffer larger than the caches)
     the buffer is zeroed before every bracketed launch, like the reference's harness does (benchmarks/_utils.py:145-151
     there): the launch then reads its operands from HBM.  Zeroing leaves the memory-side cache full of modified lines,
@@ -70,7 +77,7 @@ def time_launches(fn, iters: int, warmup: int = 20, flush=None, flush_by: str = 
     torch.cuda.synchronize()
     ts = sorted(a.elapsed_time(b) for a, b in pairs)
     keep = ts[: max(1, int(len(ts) * 0.9))]  # drop the slowest tenth: one-off host hiccups land inside an event pair
-    return statistics.fmean(keep), statistics.median(ts)
+    return statistics.fmean(keep), statistics.median(ts), statistics.fmean(ts)
 
 
 def time_back_to_back(fn, iters: int, warmup: int = 10) -> float:
@@ -219,11 +226,14 @@ def main():
     flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
     variants = {}
     for w in cfg1:
-        mean_ms, med_ms = time_launches(lambda w=w: w.call(tens), iters=max(50, args.steps))
-        cold_ms, cold_med = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush)
-        clean_ms, _ = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush, flush_by="read")
+        mean_ms, med_ms, all_ms = time_launches(lambda w=w: w.call(tens), iters=max(50, args.steps))
+        cold_ms, cold_med, _ = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush)
+        clean_ms, _, _ = time_launches(lambda w=w: w.call(tens), iters=50, warmup=5, flush=flush, flush_by="read")
         tf = w.flops / mean_ms / 1e9
-        variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
+        variants[w.name] = {"ms": mean_ms, "ms_median": med_ms, "ms_mean_untrimmed": all_ms,
+                            "timing": "ms: mean of single event-bracketed launches without the slowest tenth; "
+                                      "ms_mean_untrimmed: all of them; ms_back_to_back: launches queued between one pair of events",
+                            "tflops": tf, "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS,
                             "ms_back_to_back": time_back_to_back(lambda w=w: w.call(tens), iters=max(50, args.steps), warmup=20),
                             "ms_flushed": cold_ms, "ms_flushed_median": cold_med, "tflops_flushed": w.flops / cold_ms / 1e9,
                             "ms_cold": clean_ms, "unmasked_flops": w.flops, "min_bytes": w.min_bytes,
@@ -234,7 +244,7 @@ def main():
     roofline = {"bound": "mfma", "kernel": f"fl::fwd_kernel ({dom.name})", "achieved": dv["tflops"],
                 "peak": W.PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dv["tflops"] / W.PEAK_BF16_TFLOPS,
                 "frac_flushed": dv["tflops_flushed"] / W.PEAK_BF16_TFLOPS,
-                "traffic": MEASURED_HBM_BYTES.get(dom.name), "traffic_unit": "bytes/launch (rocprofv3, see profiles/)",
+                "traffic": measured_hbm_bytes().get(dom.name), "traffic_unit": "bytes/launch (rocprofv3, see profiles/)",
                 "launch_ms": dv["ms"], "flops_per_launch": dom.flops}
     step_flushed_ms = sum(v["ms_flushed"] for v in variants.values())
 
@@ -249,12 +259,14 @@ def main():
             while time.perf_counter() - t_ramp < PREWARM_S / 2:
                 w.call(t)
                 torch.cuda.synchronize()
-            mean_ms = min(time_back_to_back(lambda: w.call(t), iters=100, warmup=50) for _ in range(3))
-            cold_ms, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush)
-            clean_ms, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush, flush_by="read")
+            runs = [time_back_to_back(lambda: w.call(t), iters=100, warmup=50) for _ in range(3)]
+            mean_ms = min(runs)
+            cold_ms, _, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush)
+            clean_ms, _, _ = time_launches(lambda: w.call(t), iters=50, warmup=5, flush=flush, flush_by="read")
             tf = w.flops / mean_ms / 1e9
-            others[w.name] = {"ms": mean_ms, "timing": "warm: best of three runs of 100 launches back to back, each after 50 warm-up launches; "
-                                                       "flushed: 50 launches, 512 MB zeroed before each",
+            others[w.name] = {"ms": mean_ms, "ms_mean_of_runs": statistics.fmean(runs),
+                              "timing": "ms: BEST of three runs of 100 launches back to back, each after 50 warm-up launches "
+                                        "(ms_mean_of_runs: their mean); flushed: 50 launches, 512 MB zeroed before each",
                               "ms_flushed": cold_ms, "tflops": tf, "tflops_flushed": w.flops / cold_ms / 1e9,
                               "pct_mfma_peak": 100 * tf / W.PEAK_BF16_TFLOPS, "unmasked_flops": w.flops,
                               "ms_cold": clean_ms, "min_bytes": w.min_bytes, "roofline": roofline_entry(w, mean_ms, W),

@@ -107,6 +107,8 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_params_sizeof.restype = C.c_uint64
     lib.fl_workspace_bytes.restype = C.c_uint64
     lib.fl_workspace_bytes.argtypes = [C.POINTER(FlAttnParams)]
+    lib.fl_bwd_workspace_bytes.restype = C.c_uint64
+    lib.fl_bwd_workspace_bytes.argtypes = [C.POINTER(FlAttnParams)]
     lib.fl_attn_validate.restype = C.c_int
     lib.fl_attn_validate.argtypes = [C.POINTER(FlAttnParams)]
     lib.fl_attn_plan.restype = C.c_int
@@ -123,10 +125,6 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_bwd_static.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
     lib.fl_ipa_pack.restype = C.c_int
     lib.fl_ipa_pack.argtypes = [C.POINTER(FlIpaPackParams), C.c_void_p]
-    lib.fl_probe_mfma_rate.restype = C.c_int
-    lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
-    lib.fl_probe_step.restype = C.c_int
-    lib.fl_probe_step.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
         raise RuntimeError(f"{p}: ABI version {lib.fl_version()} != expected {ABI_VERSION}")
     if lib.fl_params_sizeof() != C.sizeof(FlAttnParams):
@@ -473,8 +471,28 @@ def plan(p: FlAttnParams) -> dict:
             "lds_bytes": out[4], "features": out[5], "streaming": out[6]}
 
 
+_probe_lib = None
+
+
+def load_probe_library() -> C.CDLL:
+    """Loads the bench-only library of measurement probes (include/flashlight_amd_probe.h), built next to the product
+    library; the product library exports none of them."""
+    global _probe_lib
+    if _probe_lib is None:
+        p = LIB_PATH.with_name("libflashlight_amd_probe.so")
+        if not p.exists():
+            raise FileNotFoundError(f"{p} is missing: build it with `python -m flashlight_amd.build` (needs hipcc)")
+        lib = C.CDLL(str(p))
+        lib.fl_probe_mfma_rate.restype = C.c_int
+        lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        lib.fl_probe_step.restype = C.c_int
+        lib.fl_probe_step.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        _probe_lib = lib
+    return _probe_lib
+
+
 def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink: torch.Tensor) -> float:
-    """Launches the MFMA-only rate probe on the current stream (measurement aid, include/flashlight_amd.h) and returns
+    """Launches the MFMA-only rate probe on the current stream (measurement aid, include/flashlight_amd_probe.h) and returns
     the FLOPs of the launch.  `operands`: bf16 device tensor (multiple of 8 elements, 16-byte aligned) the per-lane
     fragments are read from; `sink`: float32 device tensor of n_workgroups * 512 elements."""
     if operands.dtype != torch.bfloat16 or not operands.is_cuda or not operands.is_contiguous() or operands.numel() % 8:
@@ -482,7 +500,7 @@ def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink:
     if sink.dtype != torch.float32 or sink.numel() < n_workgroups * 512 or sink.device != operands.device:
         raise ValueError("sink must be a float32 tensor of n_workgroups * 512 elements on the operands' device")
     stream = torch.cuda.current_stream(operands.device).cuda_stream
-    rc = load_library().fl_probe_mfma_rate(operands.data_ptr(), operands.numel() // 8, int(iters), int(n_workgroups),
+    rc = load_probe_library().fl_probe_mfma_rate(operands.data_ptr(), operands.numel() // 8, int(iters), int(n_workgroups),
                                            sink.data_ptr(), C.c_void_p(stream))
     if rc != 0:
         raise FlashlightError(rc, "fl_probe_mfma_rate rejected its arguments" if rc < 0 else "probe launch failed")
@@ -490,13 +508,13 @@ def probe_mfma_rate(operands: torch.Tensor, iters: int, n_workgroups: int, sink:
 
 
 def probe_step(head_dim: int, level: int, iters: int, n_workgroups: int, sink: torch.Tensor) -> int:
-    """Launches the step-structure probe on the current stream (measurement aid, include/flashlight_amd.h) and returns
+    """Launches the step-structure probe on the current stream (measurement aid, include/flashlight_amd_probe.h) and returns
     the number of 32 x 32 score blocks every wave works through; `sink`: float32 device tensor of n_workgroups * 256
     elements."""
     if sink.dtype != torch.float32 or not sink.is_cuda or sink.numel() < n_workgroups * 256:
         raise ValueError("sink must be a float32 device tensor of n_workgroups * 256 elements")
     stream = torch.cuda.current_stream(sink.device).cuda_stream
-    rc = load_library().fl_probe_step(int(head_dim), int(level), int(iters), int(n_workgroups), sink.data_ptr(),
+    rc = load_probe_library().fl_probe_step(int(head_dim), int(level), int(iters), int(n_workgroups), sink.data_ptr(),
                                       C.c_void_p(stream))
     if rc != 0:
         raise FlashlightError(rc, "fl_probe_step rejected its arguments" if rc < 0 else "probe launch failed")

@@ -34,6 +34,7 @@ HIPCC_FLAGS = [
 # Development knobs: extra hipcc flags (e.g. -DFL_SCHED=2) and an alternative output path for side-by-side builds.
 HIPCC_FLAGS += os.environ.get("FL_HIPCC_EXTRA", "").split()
 LIB_PATH = Path(os.environ.get("FL_LIB", str(LIB_PATH)))
+PROBE_LIB_PATH = LIB_PATH.with_name("libflashlight_amd_probe.so")
 
 
 def hipcc() -> str:
@@ -128,11 +129,15 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
             tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_F16={f16}", "-c", str(CSRC / "pairbias_unit.hip"), "-o", str(o)], o))
     # the instance tables are host data only: compiling them for the device would reference the host launchers
     for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("bwd_table.hip", ["--cuda-host-only"]),
-                       ("api.hip", []), ("probe.hip", [])):
+                       ("api.hip", []), ("ipa_pack.hip", [])):
         o = objdir / (Path(src).stem + ".o")
         objs.append(o)
         if not o.exists():
             tasks.append(([cc, *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(o)], o))
+    # the measurement probes go into a library of their own, which only the benchmark loads
+    probe_obj = objdir / "probe.o"
+    if not probe_obj.exists():
+        tasks.append(([cc, *HIPCC_FLAGS, "-c", str(CSRC / "probe.hip"), "-o", str(probe_obj)], probe_obj))
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
         for log in ex.map(_compile, tasks):
             if verbose and log.strip():
@@ -140,6 +145,9 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
     tmp = LIB_PATH.with_suffix(".so.tmp")
     _compile(([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", *map(str, objs), "-o", str(tmp)], tmp))
     os.replace(tmp, LIB_PATH)
+    tmp = PROBE_LIB_PATH.with_suffix(".so.tmp")
+    _compile(([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", str(probe_obj), "-o", str(tmp)], tmp))
+    os.replace(tmp, PROBE_LIB_PATH)
     return LIB_PATH
 
 

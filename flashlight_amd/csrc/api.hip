@@ -172,6 +172,8 @@ static __global__ __launch_bounds__(1024) void doc_order_kernel(const uint32_t* 
 constexpr size_t kStaticScratchBytes = (size_t)FL_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
+extern "C" uint64_t fl_bwd_workspace_bytes(const fl_attn_params* p);
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -288,7 +290,10 @@ int64_t lds_bytes_for(const fl::Instance* in, const fl_attn_params* p) {
 }
 int64_t max_keys_for(const fl::Instance* in) {
   int64_t tiles = fl::kMaxKeyTiles;
-  if (in->feat & fl::F_DOC) tiles = std::min<int64_t>(tiles, (fl::kMaxLdsBytes - in->lds_fixed_bytes) / 1024 * 256 - 4);
+  if (in->feat & fl::F_DOC) {
+    tiles = std::min<int64_t>(tiles, (fl::kMaxLdsBytes - in->lds_fixed_bytes) / 1024 * 256 - 4);
+    tiles = std::min<int64_t>(tiles, (fl::kMaxLdsBytes - 128) / 20);  // the pre-pass: 20 bytes of LDS per key tile
+  }
   return tiles * in->bn;
 }
 
@@ -309,7 +314,7 @@ int check_ptr(const char* what, const void* ptr, int align) {
   return 0;
 }
 
-int validate(const fl_attn_params* p, const fl::Instance** out) {
+int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = false) {
   if (!p) return fail(FL_ERR_NULL, "params is null");
   int rc;
   if ((rc = check_ptr("q", p->q, 16)) || (rc = check_ptr("k", p->k, 16)) || (rc = check_ptr("v", p->v, 16)) ||
@@ -397,7 +402,12 @@ int validate(const fl_attn_params* p, const fl::Instance** out) {
   const int64_t grid = (int64_t)p->B * p->Hq * (((int64_t)p->Lq + bm - 1) / bm);
   if (grid > 0x7fffffff) return fail(FL_ERR_SHAPE, "too many workgroups (%lld)", (long long)grid);
   if (is_doc(p->mask_kind)) {
-    const uint64_t need = fl_workspace_bytes(p);
+    // the forward's pre-pass keeps 20 bytes per key tile (and 128 more) in LDS
+    if (!for_bwd && (int64_t)nkt * 20 + 128 > fl::kMaxLdsBytes)
+      return fail(FL_ERR_SHAPE, "Lk=%d exceeds the supported maximum of %lld keys for a document mask with this kernel", p->Lk,
+                  (long long)max_keys_for(in));
+    // (a backward call needs the table of id ranges only, not the forward's lists)
+    const uint64_t need = for_bwd ? fl_bwd_workspace_bytes(p) : fl_workspace_bytes(p);
     if (!p->workspace || p->workspace_bytes < need)
       return fail(FL_ERR_WORKSPACE, "document mask needs a %llu-byte workspace (got %llu)", (unsigned long long)need,
                   (unsigned long long)(p->workspace ? p->workspace_bytes : 0));
@@ -427,6 +437,15 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   // per-lane byte offsets inside one (batch entry, head) slice are 32-bit
   const int64_t worst = std::max(std::max(p->q_strides[2], p->o_strides[2]), p->gate ? p->gate_strides[2] : 0);
   if (((int64_t)p->Lq * worst + 64) * 2 >= ((int64_t)1 << 31)) return false;
+  // ... and so are those inside one key tile of 64 rows
+  if ((64 * std::max(p->k_strides[2], p->v_strides[2]) + 32) * 2 >= ((int64_t)1 << 31)) return false;
+  // the selector weight 1 / scale must be an ordinary number in the element type (bf16 shares fp32's range; fp16 ends at
+  // 65504 and loses precision below 2^-14)
+  {
+    const float w = 1.0f / p->scale;
+    const float w_max = p->dtype == FL_F16 ? 32768.0f : 0x1p100f, w_min = p->dtype == FL_F16 ? 0x1p-10f : 0x1p-100f;
+    if (!(w <= w_max) || !(w >= w_min)) return false;
+  }
   fl::PParams k;
   std::memset(&k, 0, sizeof(k));
   k.q = static_cast<const fl::bf16_t*>(p->q);
@@ -490,6 +509,11 @@ uint64_t fl_workspace_bytes(const fl_attn_params* p) {
   const fl::Instance* in = select_instance(p);
   const DocScratch d = doc_scratch(p->B, p->Lk, in ? (int64_t)in->rw * in->nw : 64, in ? in->bn : 32);
   return d.table_bytes + d.lists_bytes + d.order_bytes;
+}
+
+uint64_t fl_bwd_workspace_bytes(const fl_attn_params* p) {
+  if (!p || !is_doc(p->mask_kind) || p->B <= 0 || p->Lk <= 0) return 0;
+  return doc_scratch(p->B, p->Lk, 128, 64).table_bytes;
 }
 
 int fl_attn_validate(const fl_attn_params* p) { return validate(p, nullptr); }
@@ -628,6 +652,9 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   if (is_doc(p->mask_kind)) {
     const DocScratch d = doc_scratch(p->B, p->Lk, bm, in->bn);
     uint32_t* lists = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(p->workspace) + d.table_bytes);
+    static const hipError_t lists_attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&fl::doc_lists_kernel),
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, fl::kMaxLdsBytes - 128);
+    if (lists_attr != hipSuccess) return fail((int)lists_attr, "doc_lists_kernel: %s", hipGetErrorString(lists_attr));
     hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(1024), (size_t)kp.n_ktiles * 20, stream,
                        p->doc_ids, p->doc_stride, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles, kp.n_ktiles,
                        (int)d.list_stride, lists);
@@ -654,7 +681,7 @@ uint64_t fl_bwd_params_sizeof(void) { return sizeof(fl_attn_bwd_params); }
 static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out) {
   if (!b) return fail(FL_ERR_NULL, "params is null");
   const fl_attn_params* p = &b->fwd;
-  int rc = validate(p, nullptr);
+  int rc = validate(p, nullptr, true);
   if (rc) return rc;
   if (p->gate || p->diff || p->attended_dump)
     return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
@@ -792,12 +819,12 @@ int fl_attn_bwd_static(const fl_attn_bwd_params* b, void* stream) {
   if (p->B <= 0 || p->Hq <= 0 || p->Lq <= 0) return fail(FL_ERR_SHAPE, "sizes must be positive");
   // layout of the static scratch: the row sums (B * Hq * Lq floats, rounded up to 256 bytes), then the document table
   const uint64_t delta_bytes = ((uint64_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256;
-  const uint64_t table_bytes = fl_workspace_bytes(p);  // (the forward's lists, part of this figure, stay unused here)
+  const uint64_t table_bytes = fl_bwd_workspace_bytes(p);
   if (delta_bytes + table_bytes > kStaticScratchBytes)
     return fail(FL_ERR_WORKSPACE,
                 "fl_attn_bwd_static: this call needs %llu bytes of scratch (4 per query row of every head, plus 16 per 32 "
-                "positions under a document mask), the library's static scratch holds %llu; use fl_attn_bwd with "
-                "caller-provided delta and workspace",
+                "positions of every batch row under a document mask), the library's static scratch holds %llu; use "
+                "fl_attn_bwd with caller-provided delta and workspace",
                 (unsigned long long)(delta_bytes + table_bytes), (unsigned long long)kStaticScratchBytes);
   void* ptr = nullptr;
   int rc = static_scratch_ptr(&ptr);

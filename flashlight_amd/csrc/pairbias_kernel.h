@@ -250,8 +250,10 @@ void pairbias_kernel(const PParams p) {
       for (int i = 0; i < 16; ++i) m = __builtin_fmaxf(m, s[i]);
       m = xhalf_max(m) * c2;
       const float ref_new = (m == -INFINITY) ? ref : __builtin_fmaxf(ref, m);
-      // (when nothing has been accumulated yet the old reference carries no weight: take the block's own maximum)
-      const float use = (l_run == 0.f && m != -INFINITY) ? m : ref_new;
+      // (when nothing has been accumulated yet the old reference carries no weight: take the block's own maximum.  The
+      // two lanes of a query hold different keys and so different partial sums; the decision takes their total, so
+      // that both form their weights against the same reference and scale the shared accumulators alike)
+      const float use = (xhalf_sum(l_run) == 0.f && m != -INFINITY) ? m : ref_new;
       const float alpha = __builtin_fminf(fast_exp2(ref - use), 0x1p126f);
       ref = use;
       l_run *= alpha;

@@ -140,8 +140,14 @@ const char* fl_last_error(void);
 /* Host-only argument check: the same validation fl_attn_fwd runs before it launches.  Touches no GPU. */
 int fl_attn_validate(const fl_attn_params* p);
 
-/* Bytes of device scratch fl_attn_fwd and fl_attn_bwd need in `workspace` for *p (0 unless a document mask is used). */
+/* Bytes of device scratch fl_attn_fwd needs in `workspace` for *p (0 unless a document mask is used): the key tiles
+ * every query tile visits, so the figure grows with Lq * Lk / (rows per workgroup * keys per tile).  Enough for
+ * fl_attn_bwd as well. */
 uint64_t fl_workspace_bytes(const fl_attn_params* p);
+
+/* Bytes of device scratch fl_attn_bwd alone needs in fwd.workspace (0 unless a document mask is used): 16 bytes per 32
+ * positions of every batch row.  No counterpart in the reference. */
+uint64_t fl_bwd_workspace_bytes(const fl_attn_params* p);
 
 /* Runs the fused forward on hipStream_t `stream` (NULL = default stream).
  * Replaces torch.compile(fn)(q, k, v, ...) for the functions of attention_variants/. */
@@ -165,7 +171,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
  * receive the gradients (element type fwd.dtype like dout; strides in elements, last stride 1, others multiples of 8).
  * delta: caller-provided scratch of B * Hq * Lq floats; delta and fwd.lse must be 16-byte aligned.
- * fwd.workspace: fl_workspace_bytes(&fwd) bytes of scratch under a document mask. */
+ * fwd.workspace: fl_bwd_workspace_bytes(&fwd) bytes of scratch under a document mask. */
 typedef struct fl_attn_bwd_params {
   fl_attn_params fwd;
   const void* dout;
@@ -198,7 +204,7 @@ int fl_attn_bwd(const fl_attn_bwd_params* p, void* stream);
  * except that p->delta and p->fwd.workspace / workspace_bytes are ignored: the row sums and the document table live in
  * a static device array inside the library (FL_STATIC_SCRATCH_BYTES per GPU, held until the process ends), whose
  * address is looked up once per device on the first call made with that device current.  A call that needs more
- * (4 bytes per query row of every head, rounded up to 256, plus fl_workspace_bytes()) returns FL_ERR_WORKSPACE and
+ * (4 bytes per query row of every head, rounded up to 256, plus fl_bwd_workspace_bytes()) returns FL_ERR_WORKSPACE and
  * launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine.  All calls on one GPU share the
  * array: two such calls that may overlap on that GPU (different streams, or different threads) race; calls queued on
  * one stream are ordered and safe.  Nothing in the array needs clearing between calls: each call rewrites what it
@@ -227,24 +233,6 @@ typedef struct fl_ipa_pack_params {
   float q_scale, point_weight;
 } fl_ipa_pack_params;
 int fl_ipa_pack(const fl_ipa_pack_params* p, void* stream);
-
-/* Measurement aid with no counterpart in the reference: launches a kernel that does nothing but issue
- * v_mfma_f32_32x32x16_bf16 (the instruction both products of the forward are built from) on operand fragments read
- * once from `operands`, so that the matrix-pipe rate this part sustains on given data can be put next to the
- * forward's.  One workgroup of 512 threads per compute unit, two waves per SIMD; every lane reads 12 16-byte
- * fragments (8 A, 4 B) at 16-byte index (thread * 12 + j) % n_fragments and issues iters * 32 MFMAs; one float per
- * thread is written to `sink` (n_workgroups * 512 floats).  Work = n_workgroups * 8 * iters * 32 * 32768 FLOP.
- * Returns 0, or a negative code for bad arguments (see fl_last_error()). */
-int fl_probe_mfma_rate(const void* operands, int64_t n_fragments, int iters, int n_workgroups, float* sink, void* stream);
-
-/* Measurement aid with no counterpart in the reference: the forward's key-tile step reduced to its instruction mix and
- * data dependences, on zero operands held in registers (head_dim 64 or 128; 2 * iters blocks of 32 keys x 32 queries
- * per wave, workgroups of 4 waves).  level 0: the block's MFMAs alone; 1: MFMAs and the softmax's vector work with no
- * dependence between them; 2: the step as the forward has it (scores chained on one accumulator, weights from the
- * scores, P.V from the weights); 3: the same with the K and V fragments read from LDS.  The time per block against the
- * MFMAs' own time says what the instruction mix, its dependences and the operand reads cost before any global memory,
- * transfer or barrier enters.  One float per thread goes to `sink` (n_workgroups * 256 floats). */
-int fl_probe_step(int head_dim, int level, int iters, int n_workgroups, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

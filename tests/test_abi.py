@@ -181,8 +181,16 @@ def test_ipa_pack_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.fl_ipa_pack(C.byref(p), None) == -2                       # no rows
 
 
-def test_probe_rejects_bad_arguments_without_a_gpu(lib):
-    # the measurement aid checks its arguments on the host before it launches anything
+def test_probe_library_is_separate_and_rejects_bad_arguments_without_a_gpu(lib):
+    # the measurement aids live in a bench-only library: the product library exports none of them, the probe library
+    # exports every function its header declares, and each checks its arguments on the host before launching anything
+    assert not hasattr(lib, "fl_probe_mfma_rate") and not hasattr(lib, "fl_probe_step")
+    lib = _ffi.load_probe_library()
+    text = re.sub(r"/\*.*?\*/", "", (HEADER.parent / "flashlight_amd_probe.h").read_text(), flags=re.S)
+    declared = re.findall(r"^\s*(?:const\s+)?[\w\s\*]+?\b(fl_\w+)\s*\(", text, flags=re.M)
+    assert set(declared) == {"fl_probe_mfma_rate", "fl_probe_step"}
+    for n in declared:
+        assert hasattr(lib, n), f"{n} is declared in flashlight_amd_probe.h but not exported"
     assert lib.fl_probe_mfma_rate(None, 1, 1, 1, None, None) == -5
     buf = (C.c_char * 64)()
     addr = C.addressof(buf)

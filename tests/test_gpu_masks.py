@@ -84,6 +84,59 @@ def test_d128_instance_bit_exact():
         assert np.array_equal(got[0, 0], M.attend_matrix(kind, 300, 300, **kw))
 
 
+def _dump_call(q, k, v, S, **kw):
+    """Attended-pair bitmap of one call, after checking that the instance chosen with the dump hook has the tile shape
+    (query rows per workgroup, keys per tile, threads) of the instance the same call runs without it."""
+    Hq = q.shape[1] // (2 if kw.get("diff") else 1)
+    dump = torch.zeros(1, Hq, S, S, dtype=torch.uint8, device=DEV)
+    shapes = []
+    for d in (None, dump):
+        out = torch.empty(1, Hq, S, v.shape[-1], dtype=q.dtype, device=DEV)
+        fk = dict(scale=None, mask_kind=kw.get("mask_kind", _ffi.MASK_NONE), window=kw.get("window", 0), prefix=0,
+                  doc_ids=kw.get("doc_ids"), alibi_heads=0, softcap=0.0, biases=[], gate=None, diff=kw.get("diff", False),
+                  lambda_full=kw.get("lambda_full", 0.0), attended_dump=d)
+        p, _keep = _ffi._fill_params(_ffi.load_library(), q, k, v, out, Hq, k.shape[1] // (2 if kw.get("diff") else 1),
+                                     fk["scale"], fk["mask_kind"], fk["window"], fk["prefix"], fk["doc_ids"], 0, 0.0, [],
+                                     None, fk["diff"], fk["lambda_full"], d)
+        plan = _ffi.plan(p)
+        shapes.append((plan["rows_per_workgroup"], plan["keys_per_tile"], plan["threads"]))
+    assert shapes[0] == shapes[1], f"dump instance {shapes[1]} differs from the production instance {shapes[0]}"
+    _ffi.attn_fwd(q, k, v, attended_dump=dump, **kw)
+    torch.cuda.synchronize()
+    return dump.cpu().numpy().astype(bool), shapes[0]
+
+
+@pytest.mark.parametrize("S", [63, 65, 129, 257, 300, 1000])
+def test_production_tile_shapes_bit_exact(S):
+    # The tile shapes the benchmark configurations launch under a mask, other than the default 128 rows x 64 keys:
+    # head dim 128 with a short sliding window (two-wave workgroups, 64 rows x 32 keys), document masks at head dim 128
+    # (128 rows x 32 keys), causal differential attention (32-key tiles, two softmax branches).
+    g = torch.Generator().manual_seed(7000 + S)
+    mk = lambda h, d: torch.randn(1, h, S, d, generator=g).bfloat16().to(DEV)  # noqa: E731
+    q, k, v = mk(2, 128), mk(2, 128), mk(2, 128)
+    for w in (0, 31, 32, 33, 100, 256):
+        got, shape = _dump_call(q, k, v, S, mask_kind=_ffi.MASK_SLIDING, window=w)
+        assert shape == (64, 32, 128), shape
+        want = M.attend_matrix("sliding", S, S, window=w)
+        assert np.array_equal(got[0, 0], want) and np.array_equal(got[0, 1], want), f"sliding {w} S={S}"
+    rng = np.random.default_rng(S)
+    cuts = np.sort(rng.choice(np.arange(1, S), size=min(4, S - 1), replace=False))
+    for tag, ids in (("sorted", np.searchsorted(cuts, np.arange(S), side="right")),
+                     ("unsorted", rng.integers(-1, 2, size=S) * (2 ** 35)), ("edges at 32", np.arange(S) // 32)):
+        for kind in ("document", "document_causal"):
+            got, shape = _dump_call(q, k, v, S, mask_kind=KIND[kind],
+                                    doc_ids=torch.as_tensor(ids, dtype=torch.int64, device=DEV)[None])
+            assert shape == (128, 32, 256), shape
+            want = M.attend_matrix(kind, S, S, doc_ids=ids)
+            assert np.array_equal(got[0, 0], want) and np.array_equal(got[0, 1], want), f"{kind}/{tag} S={S}"
+    q2, k2, v2 = mk(4, 64), mk(4, 64), mk(2, 128)
+    for kind in ("none", "causal"):
+        got, shape = _dump_call(q2, k2, v2, S, mask_kind=KIND[kind], diff=True, lambda_full=0.8)
+        assert shape == (128, 32, 256), shape
+        want = M.attend_matrix(kind, S, S)
+        assert np.array_equal(got[0, 0], want) and np.array_equal(got[0, 1], want), f"diff {kind} S={S}"
+
+
 # ---- properties that hold at any size: checked at the full benchmark shapes -----------------------------------------------
 
 def test_rows_sum_to_one_and_value_linearity_full_size():

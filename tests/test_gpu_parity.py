@@ -522,6 +522,29 @@ def test_shared_bias_streaming_kernel(B, N, S, H, gate, dtype, inf):
     assert_parity(out, ref, f"B{B} N{N} S{S} H{H}")
 
 
+@pytest.mark.parametrize("dtype,drop", [(torch.bfloat16, float("-inf")), (torch.float16, -21.0)])
+def test_shared_bias_streaming_kernel_half_masked_lanes(dtype, drop):
+    # The two lanes of a query hold alternate runs of 8 keys.  Here one lane's keys of the first 64 positions carry no
+    # weight (-inf in bf16; 30 log2 units down in fp16, whose weights underflow there) while the other lane's do, and
+    # the second 32-key block's maximum lies below the first's: both lanes must still agree on one softmax reference.
+    g = torch.Generator().manual_seed(33)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)  # noqa: E731
+    B, N, S, H = 1, 9, 256, 2
+    q, k, v = mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32)
+    bias = mk(B, 1, H, S, S).float()
+    keys = torch.arange(S, device=DEV)
+    stripe = (keys < 64) & (keys % 16 < 8)
+    bias[..., stripe] = float("-inf") if drop == float("-inf") else bias[..., stripe] + drop
+    bias[..., 8:16] += 6.0
+    bias = bias.to(dtype)
+    p, _keep = _ffi._fill_params(_ffi.load_library(), *(t.reshape(-1, S, H, 32).transpose(1, 2) for t in (q, k, v)),
+                                 torch.empty(B * N, H, S, 32, dtype=dtype, device=DEV), H, H, None, _ffi.MASK_NONE, 0, 0,
+                                 None, 0, 0.0, [(bias.reshape(B, H, S, S), N)], None, False, 0.0, None)
+    assert _ffi.plan(p)["streaming"] == 1
+    out = A.attention_reference(q, k, v, [bias])
+    assert_parity(out, O.attention_evoformer(*f32(q, k, v), [bias.float()]), f"half-masked lanes {dtype}")
+
+
 def test_shared_bias_streaming_kernel_matches_the_general_kernel():
     # same call through both kernels: a second bias operand (all zeros) makes the library take the general one
     g = torch.Generator().manual_seed(32)

@@ -45,7 +45,7 @@ class FlAttnParams(C.Structure):
         ("bias_dtype", C.c_int32 * 2),
         ("lse", C.c_void_p),
         ("dropout_threshold", C.c_uint32), ("dropout_seed", C.c_uint32 * 2),
-        ("reserved", C.c_int32 * 1),
+        ("flags", C.c_uint32),
     ]
 
 
@@ -201,8 +201,25 @@ def dropout_threshold(p: float) -> int:
     return min(int(round(p * 65536.0)), 65535)
 
 
+class DocWorkspace:
+    """Scratch of document-mask forward calls, kept across calls.  The first call made with a handle allocates the
+    buffer and runs the pre-pass that lists, from the ids, the key tiles every query tile visits; later calls with the
+    same handle, the same ids tensor (same memory, not modified in place since) and the same shapes and options skip the
+    pre-pass (FL_FLAG_DOC_PREPARED).  Anything else refills the handle.  The handle keeps the ids tensor alive.  The
+    calls must be ordered on the device like any producer and consumer of one buffer (same stream, or events)."""
+
+    def __init__(self):
+        self.buffer = None
+        self.key = None
+        self.ids = None
+
+
+FLAG_DOC_PREPARED = 1
+
+
 def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases,
-                 gate, diff, lambda_full, attended_dump, dropout_p=0.0, dropout_seed=0, alloc_workspace=True):
+                 gate, diff, lambda_full, attended_dump, dropout_p=0.0, dropout_seed=0, alloc_workspace=True,
+                 doc_workspace=None):
     """Fills an `fl_attn_params` for validated 4-D tensors; returns it with the tensors that must outlive the launch."""
     B, _, Lq, Dqk = q.shape
     Lk, Dv = k.shape[2], v.shape[3]
@@ -276,7 +293,19 @@ def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, d
         p.attended_dump = attended_dump.data_ptr()
     need = lib.fl_workspace_bytes(C.byref(p)) if alloc_workspace else 0
     if need:
-        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        if doc_workspace is not None:
+            d = keep[4]  # the ids as the kernel reads them
+            key = (d.data_ptr(), d._version, tuple(d.shape), tuple(d.stride()), B, Hq, Hkv, Lk, Dqk, Dv, q.dtype, int(mask_kind),
+                   p.alibi_heads > 0, p.softcap > 0.0, len(biases), gate is not None, bool(diff), attended_dump is not None,
+                   int(need), str(q.device))
+            if doc_workspace.key == key and doc_workspace.buffer is not None:
+                p.flags |= FLAG_DOC_PREPARED
+            else:
+                doc_workspace.buffer = torch.empty(need, dtype=torch.uint8, device=q.device)
+                doc_workspace.key, doc_workspace.ids = key, d
+            ws = doc_workspace.buffer
+        else:
+            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
         p.workspace, p.workspace_bytes = ws.data_ptr(), need
         keep.append(ws)
     return p, keep
@@ -304,6 +333,7 @@ def attn_fwd(
     lse: Optional[torch.Tensor] = None,
     dropout_p: float = 0.0,
     dropout_seed: int = 0,
+    doc_workspace: Optional[DocWorkspace] = None,
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
@@ -313,6 +343,7 @@ def attn_fwd(
     `lse` (float32 [B, Hq, Lq]) receives the row statistics that `attn_bwd` needs.
     `dropout_p` > 0 drops softmax weights (torch.nn.functional.dropout semantics) by a hash of (`dropout_seed`, batch,
     head, query, key); positional masks and GQA only.
+    `doc_workspace` (document masks): a `DocWorkspace` handle that keeps the pre-pass's result across calls.
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -351,11 +382,13 @@ def attn_fwd(
                      gate=None if gate is None else gate[..., c:c + _MAX_DV_DIFF], diff=diff, lambda_full=lambda_full,
                      out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only,
                      lse=lse if c == 0 else None,  # the row statistics depend on q and k only
-                     dropout_p=dropout_p, dropout_seed=dropout_seed)  # so do the dropout decisions
+                     dropout_p=dropout_p, dropout_seed=dropout_seed,  # so do the dropout decisions
+                     doc_workspace=doc_workspace)  # (and the key-tile lists: the slabs share one instance)
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
-                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed)
+                           biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed,
+                           doc_workspace=doc_workspace)
     if lse is not None:
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
             raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")

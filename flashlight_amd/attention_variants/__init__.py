@@ -11,7 +11,7 @@ from .alibi import alibi_bias, attention_pytorch_alibi, generate_alibi_bias_pyto
 from .softcap import attention_softcapped, generate_tanh_softcap  # noqa: F401
 from .sliding_window import attention_pytorch_sliding_window, get_sliding_mask  # noqa: F401
 from .prefix_lm import attention_pytorch_prefix_lm, get_prefix_lm_mask  # noqa: F401
-from .document_mask import attention_pytorch_document_mask, create_document_id  # noqa: F401
+from .document_mask import DocumentMaskWorkspace, attention_pytorch_document_mask, create_document_id  # noqa: F401
 from .diff_attn import diffattn  # noqa: F401
 from .evoformer import attention_reference  # noqa: F401
 from .ipa import invariant_point_attention  # noqa: F401

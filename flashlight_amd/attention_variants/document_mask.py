@@ -11,18 +11,26 @@ from ._common import grouped_view, run
 
 def attention_pytorch_document_mask(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                     document_id: torch.Tensor, scale=None, enable_gqa=False, *,
-                                    is_causal: bool = False) -> torch.Tensor:
+                                    is_causal: bool = False, workspace: "_ffi.DocWorkspace | None" = None) -> torch.Tensor:
     """document_mask.py:6-41: `document_id` is an integer tensor [N, L]; q attends k iff document_id[n, q] ==
     document_id[n, k] (both directions inside a document).  The ids may be any integers in any order; sorted ids let
     the kernel skip whole key tiles.
 
     is_causal (not in the reference, default off) additionally requires k <= q: the mask the reference's
-    FlexAttention baseline uses for this variant (benchmarks/run_flex_variants.py:66-90)."""
+    FlexAttention baseline uses for this variant (benchmarks/run_flex_variants.py:66-90).
+
+    workspace (not in the reference): a `DocumentMaskWorkspace()` handle.  Calls that pass the same handle with the
+    same `document_id` tensor and shapes derive the key tiles each query tile visits once instead of on every call, as
+    that baseline builds its block mask once for all layers (run_flex_variants.py:66-90)."""
     if document_id.dim() != 2:
         raise ValueError(f"document_id must be [N, L], got {tuple(document_id.shape)}")
     kind = _ffi.MASK_DOCUMENT_CAUSAL if is_causal else _ffi.MASK_DOCUMENT
-    out = run(query, key, value, scale=scale, enable_gqa=enable_gqa, mask_kind=kind, doc_ids=document_id)
+    out = run(query, key, value, scale=scale, enable_gqa=enable_gqa, mask_kind=kind, doc_ids=document_id,
+              doc_workspace=workspace)
     return grouped_view(out, key, enable_gqa)
+
+
+DocumentMaskWorkspace = _ffi.DocWorkspace
 
 
 def create_document_id(batch_size: int, seq_len: int, num_docs: int = 12,

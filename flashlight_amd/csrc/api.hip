@@ -288,6 +288,8 @@ int64_t lds_bytes_for(const fl::Instance* in, const fl_attn_params* p) {
   const DocScratch d = doc_scratch(p->B, p->Lk, (int64_t)in->rw * in->nw, in->bn);
   return in->lds_fixed_bytes + (d.list_stride * 4 + 1023) / 1024 * 1024;
 }
+// Dynamic LDS bytes of the document-mask pre-pass (doc_lists_kernel): 20 per key tile; it has 128 static bytes besides
+int64_t prepass_lds_bytes(int64_t n_ktiles) { return n_ktiles * 20; }
 int64_t max_keys_for(const fl::Instance* in) {
   int64_t tiles = fl::kMaxKeyTiles;
   if (in->feat & fl::F_DOC) {
@@ -332,7 +334,9 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   if ((rc = check_strides("q", p->q_strides, 8)) || (rc = check_strides("k", p->k_strides, 8)) ||
       (rc = check_strides("v", p->v_strides, 8)) || (rc = check_strides("o", p->o_strides, 4)))
     return rc;
-  if (p->reserved[0] != 0) return fail(FL_ERR_ARG, "reserved[0] must be 0");
+  if (p->flags & ~(uint32_t)FL_FLAG_DOC_PREPARED) return fail(FL_ERR_ARG, "unknown bits in flags: 0x%x", p->flags);
+  if ((p->flags & FL_FLAG_DOC_PREPARED) && !is_doc(p->mask_kind))
+    return fail(FL_ERR_ARG, "FL_FLAG_DOC_PREPARED goes with a document mask only");
   if (p->dropout_threshold) {
     if (p->dropout_threshold > 65535u)
       return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
@@ -403,7 +407,7 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   if (grid > 0x7fffffff) return fail(FL_ERR_SHAPE, "too many workgroups (%lld)", (long long)grid);
   if (is_doc(p->mask_kind)) {
     // the forward's pre-pass keeps 20 bytes per key tile (and 128 more) in LDS
-    if (!for_bwd && (int64_t)nkt * 20 + 128 > fl::kMaxLdsBytes)
+    if (!for_bwd && prepass_lds_bytes(nkt) + 128 > fl::kMaxLdsBytes)
       return fail(FL_ERR_SHAPE, "Lk=%d exceeds the supported maximum of %lld keys for a document mask with this kernel", p->Lk,
                   (long long)max_keys_for(in));
     // (a backward call needs the table of id ranges only, not the forward's lists)
@@ -647,24 +651,34 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   const int bm = in->rw * in->nw;
   kp.n_qtiles = (p->Lq + bm - 1) / bm;
   kp.n_ktiles = (p->Lk + in->bn - 1) / in->bn;
+  {
+    // Masks whose work grows with the query position: (batch, head) pairs are taken four at a time (measured: one at a
+    // time costs the document-mask configuration 20 %, whose two heads per XCD then drain one after the other; two, eight
+    // or sixteen instead of four change the causal launch by 1-4 %)
+    const bool growing = p->mask_kind == FL_MASK_CAUSAL || p->mask_kind == FL_MASK_PREFIX_LM || is_doc(p->mask_kind);
+    static const int knob = std::getenv("FL_HEAD_GROUP") ? std::atoi(std::getenv("FL_HEAD_GROUP")) : 0;  // tuning knob
+    kp.head_group = !growing ? 1 : (knob > 0 ? knob : 4);
+  }
   const int grid = p->B * p->Hq * kp.n_qtiles;
 
   if (is_doc(p->mask_kind)) {
     const DocScratch d = doc_scratch(p->B, p->Lk, bm, in->bn);
     uint32_t* lists = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(p->workspace) + d.table_bytes);
-    static const hipError_t lists_attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&fl::doc_lists_kernel),
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, fl::kMaxLdsBytes - 128);
-    if (lists_attr != hipSuccess) return fail((int)lists_attr, "doc_lists_kernel: %s", hipGetErrorString(lists_attr));
-    hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(1024), (size_t)kp.n_ktiles * 20, stream,
-                       p->doc_ids, p->doc_stride, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles, kp.n_ktiles,
-                       (int)d.list_stride, lists);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail((int)e, "doc_lists_kernel launch failed: %s", hipGetErrorString(e));
     int32_t* order = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(p->workspace) + d.table_bytes + d.lists_bytes);
-    hipLaunchKernelGGL(fl::doc_order_kernel, dim3(p->B), dim3(1024), (size_t)kp.n_qtiles * 4, stream, lists,
-                       (int)d.list_stride, kp.n_qtiles, order);
-    e = hipGetLastError();
-    if (e != hipSuccess) return fail((int)e, "doc_order_kernel launch failed: %s", hipGetErrorString(e));
+    if (!(p->flags & FL_FLAG_DOC_PREPARED)) {
+      static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&fl::doc_lists_kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, fl::kMaxLdsBytes - 128);
+      if (attr != hipSuccess) return fail((int)attr, "doc_lists_kernel: %s", hipGetErrorString(attr));
+      hipLaunchKernelGGL(fl::doc_lists_kernel, dim3(p->B * kp.n_qtiles), dim3(1024), (size_t)prepass_lds_bytes(kp.n_ktiles), stream,
+                         p->doc_ids, p->doc_stride, p->Lk, p->mask_kind, bm, in->rw, in->bn, kp.n_qtiles, kp.n_ktiles,
+                         (int)d.list_stride, lists);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail((int)e, "doc_lists_kernel launch failed: %s", hipGetErrorString(e));
+      hipLaunchKernelGGL(fl::doc_order_kernel, dim3(p->B), dim3(1024), (size_t)kp.n_qtiles * 4, stream, lists,
+                         (int)d.list_stride, kp.n_qtiles, order);
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail((int)e, "doc_order_kernel launch failed: %s", hipGetErrorString(e));
+    }
     kp.doc_lists = lists;
     kp.doc_list_stride = (int)d.list_stride;
     kp.doc_order = order;

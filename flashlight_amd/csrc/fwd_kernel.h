@@ -89,6 +89,7 @@ struct KParams {
   uint32_t drop_thr;      // a weight is dropped when its 16 hash bits are < drop_thr (1 .. 65535; 0: no dropout)
   uint32_t drop_seed[2];  // low and high half of the 64-bit seed
   float drop_rescale;     // 65536 / (65536 - drop_thr), applied to the kept weights
+  int32_t head_group;  // (batch, head) pairs whose query tiles are dealt together, longest first (1: head by head)
   int32_t n_qtiles;  // ceil(Lq / BM)
   int32_t n_ktiles;  // ceil(Lk / BN)
 };
@@ -408,10 +409,11 @@ void fwd_kernel(const KParams p) {
 
   // ---- workgroup -> (batch, head, query tile).  Consecutive workgroup ids land on different XCDs, so ids are
   // regrouped to give every XCD a contiguous run of (batch, head) pairs: their K/V stay in that XCD's L2.
-  // Under masks whose work grows with the query position (causal, prefix-LM, causal documents) heads are taken four
-  // at a time and their query tiles dealt from the last (longest) to the first, round-robin over the four heads: the
-  // workgroups still running when the grid drains are the short ones.  Under the other masks every query tile costs
-  // the same, and heads are taken one at a time (HBM then sees each K/V tile once).
+  // Under masks whose work grows with the query position (causal, prefix-LM, causal documents) heads are taken
+  // p.head_group at a time (enough of them to fill the XCD's workgroup slots about twice over) and their query tiles
+  // dealt from the last (longest) to the first, round-robin over those heads: the workgroups still running when the grid
+  // drains are the short ones.  Under the other masks every query tile costs the same, and heads are taken one at a
+  // time (HBM then sees each K/V tile once).
   int bh, qt;
   {
     const int nbh = p.B * p.Hq, nq = p.n_qtiles;
@@ -421,7 +423,7 @@ void fwd_kernel(const KParams p) {
       base = (i % 8) * run;
       i /= 8;
     }
-    const int G = (p.mask_kind == MASK_CAUSAL || p.mask_kind == MASK_PREFIX || kDoc) ? 4 : 1;
+    const int G = p.head_group;
     const int g = i / (G * nq), rem = i % (G * nq);
     const int gg = min(G, run - G * g);
     qt = nq - 1 - rem / gg;
@@ -593,17 +595,25 @@ void fwd_kernel(const KParams p) {
     const unsigned lds_k = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::K_OFF + wave * 1024);
     const unsigned lds_v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::V_OFF + wave * 1024);
     const unsigned lds_i = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::I_OFF + wave * (BN * 8));
-    unsigned koff[T::K_PER_T], voff[T::V_PER_T];
+    // The rows of a thread's transfer `it` lie it * (NT / CPR) below those of its transfer 0.  When that step is a multiple
+    // of the swizzle's period in rows, the chunk a lane fetches is the same for every transfer, and one per-lane offset
+    // serves them all: the row step goes into the scalar base address instead of into a register per transfer.
+    constexpr int K_ROWS_PER_T = NT / LK::CPR, V_ROWS_PER_T = NT / LV::CPR;
+    constexpr bool kOneKoff = NT % LK::CPR == 0 && K_ROWS_PER_T % (LK::RPW * (LK::CPR >= 16 ? 16 : LK::CPR)) == 0;
+    constexpr bool kOneVoff = NT % LV::CPR == 0 && V_ROWS_PER_T % (LV::RPW * (LV::CPR >= 16 ? 16 : LV::CPR)) == 0;
+    unsigned koff[kOneKoff ? 1 : T::K_PER_T], voff[kOneVoff ? 1 : T::V_PER_T];
 #pragma unroll
-    for (int it = 0; it < T::K_PER_T; ++it) {
+    for (int it = 0; it < (kOneKoff ? 1 : T::K_PER_T); ++it) {
       const int id = it * NT + tid, row = id / LK::CPR, pc = id % LK::CPR;
       koff[it] = (unsigned)(row * (int)p.ks[2] + LK::swz_k(row, pc) * 8) * 2u;
     }
 #pragma unroll
-    for (int it = 0; it < T::V_PER_T; ++it) {
+    for (int it = 0; it < (kOneVoff ? 1 : T::V_PER_T); ++it) {
       const int id = it * NT + tid, row = id / LV::CPR, pc = id % LV::CPR;
       voff[it] = (unsigned)(row * (int)p.vs[2] + LV::swz_v(row, pc) * 8) * 2u;
     }
+    const uint32_t k_step_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(K_ROWS_PER_T * (uint32_t)p.ks[2] * 2u));
+    const uint32_t v_step_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(V_ROWS_PER_T * (uint32_t)p.vs[2] * 2u));
     // scalar base addresses; one key tile is less than 2^31 bytes from start to end (checked on the host)
     const uint64_t kbase = uniform_ptr(kptr), vbase = uniform_ptr(vptr);
     const uint32_t k_tile_bytes = (uint32_t)__builtin_amdgcn_readfirstlane((int)(BN * (uint32_t)p.ks[2] * 2u));
@@ -612,8 +622,10 @@ void fwd_kernel(const KParams p) {
       const uint64_t base = kbase + (uint64_t)(uint32_t)t * k_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
-        for (int it = 0; it < T::K_PER_T; ++it)
-          dma16(base, koff[it], lds_k + slot * T::KBYTES + it * NT * 16);
+        for (int it = 0; it < T::K_PER_T; ++it) {
+          if constexpr (kOneKoff) dma16(base + (uint64_t)((uint32_t)it * k_step_bytes), koff[0], lds_k + slot * T::KBYTES + it * NT * 16);
+          else dma16(base, koff[it], lds_k + slot * T::KBYTES + it * NT * 16);
+        }
       } else {
 #pragma unroll
         for (int it = 0; it < T::K_PER_T; ++it) {
@@ -623,8 +635,9 @@ void fwd_kernel(const KParams p) {
         }
       }
     };
-    auto load_v = [&](int t, int slot) FL_INLINE  {
-      if constexpr (kDoc) {
+    // (with_ids: some wave of the workgroup may apply the element mask to the tile, which compares document ids)
+    auto load_v = [&](int t, int slot, bool with_ids) FL_INLINE  {
+      if constexpr (kDoc) if (with_ids) {
         // this wave's copy of the tile's key ids, one dword per lane and transfer; keys past Lk repeat the last id
         const uint64_t ibase = uniform_ptr(p.doc_ids + (int64_t)batch * p.doc_stride + (int64_t)t * BN);
         const int last = p.Lk - 1 - t * BN;
@@ -637,8 +650,10 @@ void fwd_kernel(const KParams p) {
       const uint64_t base = vbase + (uint64_t)(uint32_t)t * v_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
-        for (int it = 0; it < T::V_PER_T; ++it)
-          dma16(base, voff[it], lds_v + slot * T::VBYTES + it * NT * 16);
+        for (int it = 0; it < T::V_PER_T; ++it) {
+          if constexpr (kOneVoff) dma16(base + (uint64_t)((uint32_t)it * v_step_bytes), voff[0], lds_v + slot * T::VBYTES + it * NT * 16);
+          else dma16(base, voff[it], lds_v + slot * T::VBYTES + it * NT * 16);
+        }
       } else {
 #pragma unroll
         for (int it = 0; it < T::V_PER_T; ++it) {
@@ -714,6 +729,13 @@ void fwd_kernel(const KParams p) {
     // tile index / this wave's class of a tile-list entry
     auto entry_tile = [&](uint32_t e) FL_INLINE  { return (int)(__builtin_amdgcn_readfirstlane(e) & 0xffffu); };
     auto entry_class = [&](uint32_t e) FL_INLINE  { return (int)((__builtin_amdgcn_readfirstlane(e) >> (16 + 2 * wave)) & 3u); };
+
+    // whether some wave may apply the element mask to the entry's tile: not when it is FULL (class bits 10) for every
+    // wave.  (A tile that is EMPTY for a wave can still lie inside that wave's run, where it is computed and masked.)
+    auto entry_masked = [&](uint32_t e) FL_INLINE {
+      constexpr uint32_t kAll = (1u << (2 * NW)) - 1u;
+      return ((__builtin_amdgcn_readfirstlane(e) >> 16) & kAll) != (0xAAAAu & kAll);
+    };
 
     // ---- S^T = K . Q^T for one tile: A = K fragment from LDS, B = Q fragment ---------------------------------------
     auto qk = [&](f32x16 (&s)[KB][QB], int buf) FL_INLINE {
@@ -1107,7 +1129,7 @@ void fwd_kernel(const KParams p) {
         }
 #pragma unroll
       for (int j = 0; j + 1 < NS; ++j)
-        if (j < n_list) load_v(entry_tile(ent[j]), j);
+        if (j < n_list) load_v(entry_tile(ent[j]), j, entry_masked(ent[j]));
       dma_wait<0>();
       __syncthreads();
       // The list positions whose tiles are not EMPTY for this wave's rows form one run [a_live, b_live) (an EMPTY tile
@@ -1156,7 +1178,7 @@ void fwd_kernel(const KParams p) {
           load_k(entry_tile(ent[NS]), slot);
           load_b(entry_tile(ent[NS]), slot);  // the bias of this step's tile was consumed at the end of the previous step
         }
-        if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS);
+        if (pos + NS - 1 < n_list) load_v(entry_tile(ent[NS - 1]), (slot + NS - 1) % NS, entry_masked(ent[NS - 1]));
         return steady;
       };
       auto end_step = [&](bool steady) FL_INLINE {

@@ -221,13 +221,15 @@ def _pad_head_dims(q, k, v, gate, diff):
 
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
-             dropout_seed=None) -> torch.Tensor:
+             dropout_seed=None, doc_workspace=None) -> torch.Tensor:
     """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise; the
     differentiable operator when a gradient with respect to q, k or v will be asked for.
 
     `dropout_p` > 0 drops softmax weights (the reference's functions ignore their `dropout_p`; see
     `attention_variants.honor_dropout`).  `dropout_seed=None` draws a fresh 63-bit seed from torch's default CPU
-    generator, so `torch.manual_seed` reproduces a run; the same seed gives the same decisions in forward and backward."""
+    generator, so `torch.manual_seed` reproduces a run; the same seed gives the same decisions in forward and backward.
+    `doc_workspace` (an `_ffi.DocWorkspace`) is used by the plain forward call only; traced and differentiable calls run
+    their pre-pass every time."""
     dropout_p = float(dropout_p)
     _ffi.dropout_threshold(dropout_p)  # range check
     padded = _pad_head_dims(q, k, v, gate, diff)
@@ -239,7 +241,8 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
             scale = 1.0 / math.sqrt(q.size(-1))
         out = dispatch(qp, kp, vp, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                        alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gp, diff=diff, lambda_full=lambda_full,
-                       seq_major_out=seq_major_out, dropout_p=dropout_p, dropout_seed=dropout_seed)
+                       seq_major_out=seq_major_out, dropout_p=dropout_p, dropout_seed=dropout_seed,
+                       doc_workspace=doc_workspace)
         return out[..., :v.size(-1)]
     if dropout_p > 0.0:
         if biases or gate is not None or diff or seq_major_out:
@@ -270,4 +273,5 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None
     return _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                          alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
-                         lambda_full=lambda_full, out=out, dropout_p=dropout_p, dropout_seed=dropout_seed)
+                         lambda_full=lambda_full, out=out, dropout_p=dropout_p, dropout_seed=dropout_seed,
+                         doc_workspace=doc_workspace)

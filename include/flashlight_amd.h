@@ -125,8 +125,16 @@ typedef struct fl_attn_params {
   uint32_t dropout_threshold;
   uint32_t dropout_seed[2]; /* low, high half of a 64-bit seed */
 
-  int32_t reserved[1]; /* must be 0 */
+  /* Bit set of FL_FLAG_*; unknown bits are rejected.  No counterpart in the reference. */
+  uint32_t flags;
 } fl_attn_params;
+
+/* fl_attn_fwd, document masks only: `workspace` still holds what an earlier fl_attn_fwd call (without this flag) wrote
+ * there for the same doc_ids contents, doc_stride, B, Lq = Lk, mask_kind, head dims, dtype and features, and the
+ * pre-pass that derives the key-tile lists from the ids is skipped.  For callers that run many layers over one packed
+ * batch, as the reference's Flex baseline builds its block mask once (benchmarks/run_flex_variants.py:66-90).  The ids
+ * are still read by the kernel itself; passing other ids than the workspace was prepared for gives wrong results. */
+#define FL_FLAG_DOC_PREPARED 1u
 
 /* ABI version of the loaded library (FL_ABI_VERSION it was built with). */
 int fl_version(void);

@@ -102,7 +102,8 @@ def test_plan_reports_launch_shape(lib):
     (lambda p: setattr(p, "dtype", 3), -4, "dtype"),
     (lambda p: (setattr(p, "Dqk", 48), setattr(p, "Dv", 48)), -4, "no kernel instance"),
     (lambda p: (setattr(p, "diff", 1), setattr(p, "lambda_", float("inf"))), -5, "lambda"),
-    (lambda p: p.reserved.__setitem__(0, 1), -5, "reserved"),
+    (lambda p: setattr(p, "flags", 2), -5, "flags"),
+    (lambda p: setattr(p, "flags", 1), -5, "FL_FLAG_DOC_PREPARED"),
     (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 0)), -5, "bias_batch_div"),
     (lambda p: (p.bias.__setitem__(0, 0x60000), p.bias_batch_div.__setitem__(0, 1),
                 p.bias_strides[0].__setitem__(3, 2)), -3, "key stride"),

@@ -173,8 +173,8 @@ def test_abi_validation_of_dropout_fields():
     p.dropout_threshold = 100
     assert rc(p) == -4, _ffi.last_error()
     p = good_params()
-    p.reserved[0] = 1
-    assert rc(p) == -5 and "reserved" in _ffi.last_error()
+    p.flags = 4
+    assert rc(p) == -5 and "flags" in _ffi.last_error()
 
 
 def test_front_end_switch_and_refusals():

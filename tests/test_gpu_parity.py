@@ -557,3 +557,26 @@ def test_shared_bias_streaming_kernel_matches_the_general_kernel():
     general = A.attention_reference(q, k, v, [zero, bias], gate=gt)
     assert (fast.float() - general.float()).abs().max().item() <= 2e-2
     assert_parity(fast, O.attention_evoformer(*f32(q, k, v), [bias.float()], gate=gt.float()), "streaming")
+
+
+def test_document_mask_prepared_workspace_skips_the_prepass_and_matches():
+    # A workspace handle keeps the key-tile lists across calls on the same ids (FL_FLAG_DOC_PREPARED); other ids, or ids
+    # modified in place, refill it.  Every result equals the plain call's bit for bit.
+    g = torch.Generator().manual_seed(41)
+    B, H, S, D = 2, 3, 700, 64
+    q, k, v = (torch.randn(B, H, S, D, generator=g).bfloat16().to(DEV) for _ in range(3))
+    ids = torch.sort(torch.randint(0, 5, (B, S), generator=g), dim=1).values.to(DEV)
+    ws = A.DocumentMaskWorkspace()
+    for causal in (False, True):
+        plain = A.attention_pytorch_document_mask(q, k, v, ids, is_causal=causal)
+        first = A.attention_pytorch_document_mask(q, k, v, ids, is_causal=causal, workspace=ws)
+        key = ws.key
+        again = A.attention_pytorch_document_mask(q * 2, k, v, ids, is_causal=causal, workspace=ws)  # other q, same ids
+        assert ws.key == key
+        assert torch.equal(plain, first)
+        assert torch.equal(again, A.attention_pytorch_document_mask(q * 2, k, v, ids, is_causal=causal))
+    ids[:, S // 2:] += 7  # in place: the handle notices the new version and runs the pre-pass again
+    out = A.attention_pytorch_document_mask(q, k, v, ids, is_causal=True, workspace=ws)
+    assert torch.equal(out, A.attention_pytorch_document_mask(q, k, v, ids, is_causal=True))
+    ref = O.attention_document_mask(*f32(q, k, v), ids, is_causal=True)
+    assert_parity(out, ref, "prepared workspace")

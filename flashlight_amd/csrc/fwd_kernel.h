@@ -635,10 +635,9 @@ void fwd_kernel(const KParams p) {
         }
       }
     };
-    // (with_ids: some wave of the workgroup may apply the element mask to the tile, which compares document ids)
-    auto load_v = [&](int t, int slot, bool with_ids) FL_INLINE  {
-      if constexpr (kDoc) if (with_ids) {
-        // this wave's copy of the tile's key ids, one dword per lane and transfer; keys past Lk repeat the last id
+    // this wave's copy of a tile's key ids (document masks), one dword per lane and transfer; keys past Lk repeat the last id
+    auto load_ids = [&](int t, int slot) FL_INLINE {
+      if constexpr (kDoc) {
         const uint64_t ibase = uniform_ptr(p.doc_ids + (int64_t)batch * p.doc_stride + (int64_t)t * BN);
         const int last = p.Lk - 1 - t * BN;
 #pragma unroll
@@ -647,6 +646,10 @@ void fwd_kernel(const KParams p) {
           dma4(ibase, (unsigned)(min(d / 2, last) * 8 + (d % 2) * 4), lds_i + slot * T::IBYTES + it * 256);
         }
       }
+    };
+    // (with_ids: some wave of the workgroup may apply the element mask to the tile, which compares document ids)
+    auto load_v = [&](int t, int slot, bool with_ids) FL_INLINE  {
+      if (with_ids) load_ids(t, slot);
       const uint64_t base = vbase + (uint64_t)(uint32_t)t * v_tile_bytes;
       if (t * BN + BN <= p.Lk) {
 #pragma unroll
@@ -1057,7 +1060,7 @@ void fwd_kernel(const KParams p) {
     // same row-sum test (measured: 2 % on the soft-cap configurations, nothing or a loss on the others).
     constexpr bool kLazyMasked = kFastRef && kSoftcap;
     auto weights_checked = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], bool check, auto in_loop,
-                               ex8 (&vfirst)[DVB], int vslot, int t) FL_INLINE {
+                               ex8 (&vfirst)[DVB], int vslot, int t, auto prefetch_v) FL_INLINE {
       float rs[QB];
       softmax_p(s, pf, rs, t);
       if constexpr (decltype(in_loop)::value) {
@@ -1067,7 +1070,7 @@ void fwd_kernel(const KParams p) {
         constexpr int n_exp = 16 * KB * QB;  // per lane: fma + exp per score, one pack and one dot2 per two
         sched_first_product<NA, (n_exp * (kDrop ? 9 : 3) + NA - 1) / NA>();
       }
-      if constexpr (decltype(in_loop)::value) {
+      if constexpr (decltype(in_loop)::value && decltype(prefetch_v)::value) {
         // the second product's first V fragments are fetched here, ahead of the branch below, so that their LDS
         // latency runs under the exponentials
 #pragma unroll
@@ -1111,32 +1114,32 @@ void fwd_kernel(const KParams p) {
     // (the previous branch is done with the LDS buffers; every wave's share of the tile list is visible to all)
     if (br > 0 || kDoc) __syncthreads();
     if constexpr (kDoc) n_list = __builtin_amdgcn_readfirstlane((int)tlist[-1]);
-    if (n_list > 0) {
-      constexpr int NS = T::NS;
-      constexpr int LPS = T::K_PER_T + T::V_PER_T + T::B_PER_T + T::R_PER_T + T::I_PER_T;  // transfers per thread per step
-      // ent[j] = tile-list entry of list position pos + j (the last entry again past the end of the list).  Entries are
-      // read from LDS NS steps before they are needed, so the read latency never shows.
-      int pos = 0;
-      uint32_t ent[NS + 1];
-#pragma unroll
-      for (int j = 0; j <= NS; ++j) ent[j] = list_entry(j);
-      // prologue: K of the first NS tiles and V of the first NS - 1 go to their ring slots; raw S of the first tile
-#pragma unroll
-      for (int j = 0; j < NS; ++j)
-        if (j < n_list) {
-          load_k(entry_tile(ent[j]), j);
-          load_b(entry_tile(ent[j]), j);
-        }
-#pragma unroll
-      for (int j = 0; j + 1 < NS; ++j)
-        if (j < n_list) load_v(entry_tile(ent[j]), j, entry_masked(ent[j]));
-      dma_wait<0>();
-      __syncthreads();
-      // The list positions whose tiles are not EMPTY for this wave's rows form one run [a_live, b_live) (an EMPTY tile
-      // between two others, possible under unsorted document ids, counts as live: it is computed and masked).  Before
-      // and after its run the wave takes part in the transfers and barriers of the steps and computes nothing: the far
-      // side of the diagonal, the keys outside a window, other documents.
-      int a_live = 0, b_live = n_list;
+    // whether the weights of a tile-list entry's tile are formed without looking at its row maxima first
+    auto reference_free = [&](uint32_t e) FL_INLINE { return kFastRef && (kLazyMasked || entry_class(e) == TILE_FULL); };
+    // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
+    // maxima, and the (rare) rescale.
+    auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e, int vslot) FL_INLINE {
+      const int t = entry_tile(e);
+      const bool full = entry_class(e) == TILE_FULL;
+      if constexpr (kLazyMasked) {
+        if (!full) apply_mask(sc, t, vslot);
+      } else if (!full || !kFastRef) {
+        if (!full) apply_mask(sc, t, vslot);
+        float mx[QB];
+        row_max(sc, mx);
+        rescale_if_grown(mx, false);
+      }
+      dump_attended(sc, t);
+    };
+    // This wave's run [a_live, b_live) of list positions: those whose tiles are not EMPTY for its rows (an EMPTY tile
+    // between two others, possible under unsorted document ids, counts as live: it is computed and masked).  Before
+    // and after its run the wave takes part in the transfers and barriers of the steps and computes nothing: the far
+    // side of the diagonal, the keys outside a window, other documents.  A run starts at an even position (the loops
+    // below are unrolled over the two ring slots and entered at slot 0): an EMPTY tile ahead of it is taken into the run
+    // and computed and masked like any other.
+    auto live_run = [&](int& a_live, int& b_live) FL_INLINE {
+      a_live = 0;
+      b_live = n_list;
       if constexpr (kDoc) {
         int a = n_list, b = 0;
         for (int base = 0; base < n_list; base += 64) {
@@ -1158,10 +1161,32 @@ void fwd_kernel(const KParams p) {
         b_live = min(n_list, e_hi - t_lo + 1);
       }
       if (a_live >= b_live) a_live = b_live = n_list;  // nothing for this wave
-      // A run starts at ring slot 0 (the unrolled loop below enters there, and a second way in would cost registers: the
-      // compiler then keeps both score buffers alive through both steps): up to NS - 1 EMPTY tiles ahead of it are taken
-      // into the run and computed and masked like any other.
-      else a_live -= a_live % NS;
+      else a_live -= a_live % T::NS;
+    };
+
+    if (n_list > 0) {
+      constexpr int NS = T::NS;
+      constexpr int LPS = T::K_PER_T + T::V_PER_T + T::B_PER_T + T::R_PER_T + T::I_PER_T;  // transfers per thread per step
+      // ent[j] = tile-list entry of list position pos + j (the last entry again past the end of the list).  Entries are
+      // read from LDS NS steps before they are needed, so the read latency never shows.
+      int pos = 0;
+      uint32_t ent[NS + 1];
+#pragma unroll
+      for (int j = 0; j <= NS; ++j) ent[j] = list_entry(j);
+      // prologue: K of the first NS tiles and V of the first NS - 1 go to their ring slots; raw S of the first tile
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        if (j < n_list) {
+          load_k(entry_tile(ent[j]), j);
+          load_b(entry_tile(ent[j]), j);
+        }
+#pragma unroll
+      for (int j = 0; j + 1 < NS; ++j)
+        if (j < n_list) load_v(entry_tile(ent[j]), j, entry_masked(ent[j]));
+      dma_wait<0>();
+      __syncthreads();
+      int a_live, b_live;
+      live_run(a_live, b_live);
       f32x16 s_a[KB][QB], s_b[KB][QB];
       if (a_live == 0 && b_live > 0) {
         qk(s_a, 0);
@@ -1189,23 +1214,6 @@ void fwd_kernel(const KParams p) {
         for (int j = 0; j < NS; ++j) ent[j] = ent[j + 1];
         ent[NS] = list_entry(pos + NS);
       };
-      // whether the weights of a tile-list entry's tile are formed without looking at its row maxima first
-      auto reference_free = [&](uint32_t e) FL_INLINE { return kFastRef && (kLazyMasked || entry_class(e) == TILE_FULL); };
-      // Head of a step, vector work only: element mask of the current tile if it is not FULL for this wave, its row
-      // maxima, and the (rare) rescale.
-      auto settle = [&](f32x16 (&sc)[KB][QB], uint32_t e, int vslot) FL_INLINE {
-        const int t = entry_tile(e);
-        const bool full = entry_class(e) == TILE_FULL;
-        if constexpr (kLazyMasked) {
-          if (!full) apply_mask(sc, t, vslot);
-        } else if (!full || !kFastRef) {
-          if (!full) apply_mask(sc, t, vslot);
-          float mx[QB];
-          row_max(sc, mx);
-          rescale_if_grown(mx, false);
-        }
-        dump_attended(sc, t);
-      };
       // One pipeline step for list position pos with pos % NS == slot: `sc` holds the (score-modified, unmasked)
       // scores of the current tile on entry and `sn` receives those of the next one.  K of list position j lives in K
       // slot j % NS, V likewise.  The body after `settle` is one straight-line block in which the scheduler
@@ -1224,7 +1232,7 @@ void fwd_kernel(const KParams p) {
         __builtin_amdgcn_s_setprio(3);
         qk(sn, (slot + 1) % NS);
         ex8 vfirst[DVB];
-        weights_checked(sc, pf, reference_free(ent[0]), std::true_type{}, vfirst, slot, entry_tile(ent[0]));
+        weights_checked(sc, pf, reference_free(ent[0]), std::true_type{}, vfirst, slot, entry_tile(ent[0]), std::true_type{});
         pv_mma(pf, slot, vfirst, std::true_type{});
         score_mods(sn, entry_tile(ent[1]), (slot + 1) % NS);
         {
@@ -1272,10 +1280,10 @@ void fwd_kernel(const KParams p) {
         ex8 vfirst[DVB];
         if constexpr (slot % 2 == 0) {
           settle(s_a, ent[0], slot);
-          weights_checked(s_a, pf, reference_free(ent[0]), std::false_type{}, vfirst, slot, entry_tile(ent[0]));
+          weights_checked(s_a, pf, reference_free(ent[0]), std::false_type{}, vfirst, slot, entry_tile(ent[0]), std::false_type{});
         } else {
           settle(s_b, ent[0], slot);
-          weights_checked(s_b, pf, reference_free(ent[0]), std::false_type{}, vfirst, slot, entry_tile(ent[0]));
+          weights_checked(s_b, pf, reference_free(ent[0]), std::false_type{}, vfirst, slot, entry_tile(ent[0]), std::false_type{});
         }
         pv_mma(pf, slot, vfirst, std::false_type{});
         return false;

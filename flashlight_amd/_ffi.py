@@ -520,6 +520,8 @@ def load_probe_library() -> C.CDLL:
         lib.fl_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         lib.fl_probe_step.restype = C.c_int
         lib.fl_probe_step.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        lib.fl_probe_coissue.restype = C.c_int
+        lib.fl_probe_coissue.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         _probe_lib = lib
     return _probe_lib
 
@@ -552,3 +554,25 @@ def probe_step(head_dim: int, level: int, iters: int, n_workgroups: int, sink: t
     if rc != 0:
         raise FlashlightError(rc, "fl_probe_step rejected its arguments" if rc < 0 else "probe launch failed")
     return 2 * int(iters)
+
+
+COISSUE_KINDS = {"fma": 0, "exp": 1, "cvt_pk_bf16": 2, "dot2c": 3, "add": 4}
+
+
+def probe_coissue(mfma_rows: int, valu_kind: str, valu_per_mfma: int, waves_per_simd: int, iters: int = 2000,
+                  device="cuda") -> dict:
+    """Runs the co-issue probe (include/flashlight_amd_probe.h) on every compute unit and returns shader cycles per unit
+    of matrix work (one 32x32x16 MFMA, or two 16x16x32) per SIMD: from the slowest wave and from the mean wave."""
+    n_cu = torch.cuda.get_device_properties(device).multi_processor_count
+    n_waves = n_cu * 4 * waves_per_simd
+    sink = torch.empty(n_cu * 256 * waves_per_simd, dtype=torch.float32, device=device)
+    cyc = torch.zeros(n_waves, dtype=torch.int64, device=device)
+    stream = torch.cuda.current_stream(sink.device).cuda_stream
+    rc = load_probe_library().fl_probe_coissue(int(mfma_rows), COISSUE_KINDS[valu_kind], int(valu_per_mfma), int(waves_per_simd),
+                                               int(iters), n_cu, sink.data_ptr(), cyc.data_ptr(), C.c_void_p(stream))
+    if rc != 0:
+        raise FlashlightError(rc, "fl_probe_coissue rejected its arguments" if rc < 0 else "probe launch failed")
+    torch.cuda.synchronize(sink.device)
+    c = cyc.double()
+    per = 8.0 * iters * waves_per_simd
+    return {"slowest_wave": float(c.max()) / per, "mean_wave": float(c.mean()) / per}

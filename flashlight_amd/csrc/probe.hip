@@ -184,3 +184,99 @@ extern "C" int fl_probe_step(int head_dim, int level, int iters, int n_workgroup
   return e == hipSuccess ? 0 : 1;
 }
 
+
+// ---- co-issue probe: how much vector work fits under matrix instructions -------------------------------------------------
+// A loop of 8 matrix instructions on independent accumulators (32x32x16 bf16, or twice as many 16x16x32 bf16), each
+// followed by K vector instructions of one kind on registers no matrix instruction touches; zero operands, nothing
+// else.  Written with fixed registers so that the compiler neither reorders nor merges anything.  The time per matrix
+// instruction against the bare loop's says how many cycles of an MFMA the vector ALU can use, whether the shorter
+// matrix instruction leaves more room, and which vector instructions do not overlap with the matrix pipe at all.
+namespace {
+
+#define FLP_CLOBBER                                                                                                      \
+  "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17",    \
+      "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33",    \
+      "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49",    \
+      "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v64", "v65",    \
+      "v66", "v67", "v68", "v69", "v70", "v71", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108",  \
+      "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v118", "v121", "s4"
+
+// one 32 x 32 x 16 matrix instruction on accumulator j (of four), or the same work as two 16 x 16 x 32 instructions on
+// accumulators 2j, 2j + 1 (of sixteen)
+#define FLP_M32(j) "v_mfma_f32_32x32x16_bf16 v[" #j "*16:" #j "*16+15], v[64:67], v[68:71], v[" #j "*16:" #j "*16+15]\n"
+#define FLP_M16(j)                                                                                       \
+  "v_mfma_f32_16x16x32_bf16 v[" #j "*8:" #j "*8+3], v[64:67], v[68:71], v[" #j "*8:" #j "*8+3]\n"            \
+  "v_mfma_f32_16x16x32_bf16 v[" #j "*8+4:" #j "*8+7], v[64:67], v[68:71], v[" #j "*8+4:" #j "*8+7]\n"
+// K vector instructions of kind KIND (0 multiply-add, 1 exponential, 2 pack to bf16, 3 dot product of two bf16 pairs with
+// accumulation, 4 addition): destinations v100.., sources v108.., v118, v121.  %0 = K, %1 = KIND (assembler constants).
+#define FLP_VALU                                                                                         \
+  ".set flp_k, 0\n .rept %0\n"                                                                           \
+  " .if %1 == 0\n v_fma_f32 v[100+flp_k], v[108+flp_k], v121, v118\n .endif\n"                           \
+  " .if %1 == 1\n v_exp_f32 v[100+flp_k], v[108+flp_k]\n .endif\n"                                       \
+  " .if %1 == 2\n v_cvt_pk_bf16_f32 v[100+flp_k], v[108+flp_k], v[108+((flp_k+1)&7)]\n .endif\n"         \
+  " .if %1 == 3\n v_dot2c_f32_bf16 v[100+flp_k], 0x3f803f80, v[108+flp_k]\n .endif\n"                    \
+  " .if %1 == 4\n v_add_f32 v[100+flp_k], v[100+flp_k], v[108+flp_k]\n .endif\n"                         \
+  " .set flp_k, flp_k+1\n .endr\n"
+
+template <int MF, int KIND, int K>
+__global__ void __launch_bounds__(512) coissue_kernel(float* out, int iters, long long* cycles) {
+  const long long c0 = clock64();
+  asm volatile("s_mov_b32 s4, 0\n .set flp_i, 0\n .rept 72\n v_mov_b32 v[flp_i], 0\n .set flp_i, flp_i+1\n .endr\n"
+               " .set flp_i, 100\n .rept 22\n v_mov_b32 v[flp_i], 0\n .set flp_i, flp_i+1\n .endr" ::: FLP_CLOBBER);
+  for (int it = 0; it < iters; ++it) {
+    if (MF == 32)
+      asm volatile(FLP_M32(0) FLP_VALU FLP_M32(1) FLP_VALU FLP_M32(2) FLP_VALU FLP_M32(3) FLP_VALU
+                   FLP_M32(0) FLP_VALU FLP_M32(1) FLP_VALU FLP_M32(2) FLP_VALU FLP_M32(3) FLP_VALU ::"n"(K), "n"(KIND) : FLP_CLOBBER);
+    else
+      asm volatile(FLP_M16(0) FLP_VALU FLP_M16(1) FLP_VALU FLP_M16(2) FLP_VALU FLP_M16(3) FLP_VALU
+                   FLP_M16(4) FLP_VALU FLP_M16(5) FLP_VALU FLP_M16(6) FLP_VALU FLP_M16(7) FLP_VALU ::"n"(K), "n"(KIND) : FLP_CLOBBER);
+  }
+  float r;
+  asm volatile("v_add_f32 %0, v0, v100" : "=v"(r)::FLP_CLOBBER);
+  const long long c1 = clock64();
+  out[blockIdx.x * blockDim.x + threadIdx.x] = r;
+  if (threadIdx.x % 64 == 0) cycles[blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64] = c1 - c0;
+}
+
+template <int MF, int KIND>
+hipError_t launch_coissue(int k, int waves_per_simd, int iters, int n_workgroups, float* sink, long long* cycles, hipStream_t st) {
+  const dim3 g(n_workgroups), b(256 * waves_per_simd);
+  switch (k) {
+    case 0: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 0>), g, b, 0, st, sink, iters, cycles); break;
+    case 1: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 1>), g, b, 0, st, sink, iters, cycles); break;
+    case 2: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 2>), g, b, 0, st, sink, iters, cycles); break;
+    case 3: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 3>), g, b, 0, st, sink, iters, cycles); break;
+    case 4: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 4>), g, b, 0, st, sink, iters, cycles); break;
+    case 6: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 6>), g, b, 0, st, sink, iters, cycles); break;
+    case 8: hipLaunchKernelGGL((coissue_kernel<MF, KIND, 8>), g, b, 0, st, sink, iters, cycles); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+template <int MF>
+hipError_t launch_coissue_kind(int kind, int k, int w, int iters, int n, float* sink, long long* cycles, hipStream_t st) {
+  switch (kind) {
+    case 0: return launch_coissue<MF, 0>(k, w, iters, n, sink, cycles, st);
+    case 1: return launch_coissue<MF, 1>(k, w, iters, n, sink, cycles, st);
+    case 2: return launch_coissue<MF, 2>(k, w, iters, n, sink, cycles, st);
+    case 3: return launch_coissue<MF, 3>(k, w, iters, n, sink, cycles, st);
+    case 4: return launch_coissue<MF, 4>(k, w, iters, n, sink, cycles, st);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+extern "C" int fl_probe_coissue(int mfma_rows, int valu_kind, int valu_per_mfma, int waves_per_simd, int iters,
+                                int n_workgroups, float* sink, long long* wave_cycles, void* stream) {
+  if (!sink || !wave_cycles || iters <= 0 || n_workgroups <= 0 || (waves_per_simd != 1 && waves_per_simd != 2))
+    return FLP_ERR_ARG;
+  if ((mfma_rows != 32 && mfma_rows != 16) || valu_kind < 0 || valu_kind > 4) return FLP_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const hipError_t e = mfma_rows == 32
+                           ? launch_coissue_kind<32>(valu_kind, valu_per_mfma, waves_per_simd, iters, n_workgroups, sink, wave_cycles, st)
+                           : launch_coissue_kind<16>(valu_kind, valu_per_mfma, waves_per_simd, iters, n_workgroups, sink, wave_cycles, st);
+  if (e == hipErrorInvalidValue) return FLP_ERR_UNSUPPORTED;
+  return e == hipSuccess ? 0 : 1;
+}

@@ -39,6 +39,17 @@ int fl_probe_mfma_rate(const void* operands, int64_t n_fragments, int iters, int
  * transfer or barrier enters.  One float per thread goes to `sink` (n_workgroups * 256 floats). */
 int fl_probe_step(int head_dim, int level, int iters, int n_workgroups, float* sink, void* stream);
 
+/* Measurement aid: how much vector work fits under matrix instructions.  Every wave runs `iters` times a loop of 8 units of
+ * matrix work on independent accumulators (mfma_rows = 32: one v_mfma_f32_32x32x16_bf16 per unit; 16: two
+ * v_mfma_f32_16x16x32_bf16), each unit followed by `valu_per_mfma` (0, 1, 2, 3, 4, 6 or 8) vector instructions of one kind
+ * on other registers (valu_kind 0: v_fma_f32, 1: v_exp_f32, 2: v_cvt_pk_bf16_f32, 3: v_dot2c_f32_bf16, 4: v_add_f32), in
+ * fixed registers and fixed order, zero operands.  Workgroups of 256 * waves_per_simd threads (1 or 2 waves per SIMD
+ * when n_workgroups is the number of compute units).  `wave_cycles` (n_workgroups * 4 * waves_per_simd int64) receives
+ * every wave's shader-clock cycles for the whole loop; `sink` one float per thread.  Cycles per unit of matrix work per
+ * SIMD = slowest wave's cycles / (8 * iters) / waves_per_simd (the waves of a SIMD share its matrix pipe). */
+int fl_probe_coissue(int mfma_rows, int valu_kind, int valu_per_mfma, int waves_per_simd, int iters, int n_workgroups,
+                     float* sink, long long* wave_cycles, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

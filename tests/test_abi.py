@@ -189,7 +189,7 @@ def test_probe_library_is_separate_and_rejects_bad_arguments_without_a_gpu(lib):
     lib = _ffi.load_probe_library()
     text = re.sub(r"/\*.*?\*/", "", (HEADER.parent / "flashlight_amd_probe.h").read_text(), flags=re.S)
     declared = re.findall(r"^\s*(?:const\s+)?[\w\s\*]+?\b(fl_\w+)\s*\(", text, flags=re.M)
-    assert set(declared) == {"fl_probe_mfma_rate", "fl_probe_step"}
+    assert set(declared) == {"fl_probe_mfma_rate", "fl_probe_step", "fl_probe_coissue"}
     for n in declared:
         assert hasattr(lib, n), f"{n} is declared in flashlight_amd_probe.h but not exported"
     assert lib.fl_probe_mfma_rate(None, 1, 1, 1, None, None) == -5
@@ -201,3 +201,7 @@ def test_probe_library_is_separate_and_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.fl_probe_step(64, 2, 1, 1, None, None) == -5
     assert lib.fl_probe_step(64, 4, 1, 1, C.c_void_p(aligned), None) == -5
     assert lib.fl_probe_step(96, 2, 1, 1, C.c_void_p(aligned), None) == -4
+    assert lib.fl_probe_coissue(32, 0, 2, 1, 1, 1, None, None, None) == -5
+    assert lib.fl_probe_coissue(32, 0, 2, 3, 1, 1, C.c_void_p(aligned), C.c_void_p(aligned), None) == -5   # waves per SIMD
+    assert lib.fl_probe_coissue(24, 0, 2, 1, 1, 1, C.c_void_p(aligned), C.c_void_p(aligned), None) == -4   # MFMA shape
+    assert lib.fl_probe_coissue(32, 7, 2, 1, 1, 1, C.c_void_p(aligned), C.c_void_p(aligned), None) == -4   # vector kind

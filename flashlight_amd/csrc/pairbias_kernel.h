@@ -13,7 +13,7 @@
 //   * the matrix pipe, which idles at head dim 32, adds it: S^T += Sel . Bias^T with Sel the 32 x 16 selector that puts
 //     key 16m + j on row j of the group, weighted 1/scale (split in two bf16 terms, relative error 2^-17), so the
 //     accumulators hold qk + bias/scale and the weights are exp2(scale * log2(e) * acc - ref): per score one
-//     multiply-add, one exponential, half a pack and half a row-sum instruction.
+//     multiply-add, one exponential, one addition for the row sum and half a pack.
 // Infinite bias entries are clamped to the largest finite value when the fragments are loaded (0 * inf inside the
 // selector product would poison the 15 other keys of the group); as an additive term that is the same mask.
 #pragma once
@@ -227,19 +227,22 @@ void pairbias_kernel(const PParams p) {
   float ref = 0.f, l_run = 0.f;
   constexpr float kBig = 0x1p24f, kTiny = std::is_same<E, f16_t>::value ? 0x1p-4f : 0x1p-24f;
   auto weights = [&](const f32x16& s, ex8 (&pf)[2]) FL_INLINE {
-    const ex2 ones = {(E)1.0f, (E)1.0f};
     auto form = [&]() FL_INLINE -> float {
       float rs = 0.f;
+      // (the row sum takes the weights before they are rounded, with plain additions: v_dot2c_f32_bf16, which would add
+      // two rounded weights at once, does not overlap with matrix instructions on this part)
+      float rs1 = 0.f;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pf[j][e] = (E)fast_exp2(__builtin_fmaf(s[8 * j + e], c2, -ref));
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 8; e += 2) {
-          const ex2 pr = {pf[j][e], pf[j][e + 1]};
-          rs = dot2acc(pr, ones, rs);
+          const float p0 = fast_exp2(__builtin_fmaf(s[8 * j + e], c2, -ref)), p1 = fast_exp2(__builtin_fmaf(s[8 * j + e + 1], c2, -ref));
+          pf[j][e] = (E)p0;
+          pf[j][e + 1] = (E)p1;
+          rs += p0;
+          rs1 += p1;
         }
-      }
+      rs += rs1;
       return rs;
     };
     float rs = form();

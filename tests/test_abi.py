@@ -127,6 +127,28 @@ def test_null_params(lib):
     assert lib.fl_workspace_bytes(None) == 0
 
 
+def test_backward_workspace_and_document_length_limit(lib):
+    # the backward needs the table of id ranges only (16 bytes per 32 positions of every batch row), not the forward's lists
+    p = good_params(B=3, L=1000)
+    assert lib.fl_bwd_workspace_bytes(C.byref(p)) == 0 and lib.fl_bwd_workspace_bytes(None) == 0
+    p.mask_kind = _ffi.MASK_DOCUMENT
+    assert lib.fl_bwd_workspace_bytes(C.byref(p)) == 3 * ((1000 + 31) // 32) * 16
+    assert lib.fl_bwd_workspace_bytes(C.byref(p)) < lib.fl_workspace_bytes(C.byref(p))
+    # the forward's pre-pass keeps 20 bytes of LDS per key tile: beyond (160 KiB - 128) / 20 tiles a document-mask call
+    # is refused by the host check, with the true maximum in the message, instead of failing at launch
+    shape = _ffi.plan(good_params(B=1, L=1000))
+    bn = shape["keys_per_tile"]
+    max_tiles = (160 * 1024 - 128) // 20
+    for L, ok in ((max_tiles * bn, True), ((max_tiles + 1) * bn, False)):
+        q = good_params(B=1, Hq=1, Hkv=1, L=L)
+        q.mask_kind, q.doc_ids = _ffi.MASK_DOCUMENT_CAUSAL, 0x50000
+        q.workspace, q.workspace_bytes = 0x80000, lib.fl_workspace_bytes(C.byref(q))
+        if ok:
+            assert rc(lib, q) == 0, _ffi.last_error()
+        else:
+            assert rc(lib, q) == -2 and str(max_tiles * bn) in _ffi.last_error(), _ffi.last_error()
+
+
 def test_workspace_size_for_document_masks(lib):
     p = good_params(B=3, L=1000)
     assert lib.fl_workspace_bytes(C.byref(p)) == 0

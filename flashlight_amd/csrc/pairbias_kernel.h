@@ -225,7 +225,9 @@ void pairbias_kernel(const PParams p) {
   // nothing accumulated yet): any reference gives the same O / l.
   f32x16 oacc;
   float ref = 0.f, l_run = 0.f;
-  constexpr float kBig = 0x1p24f, kTiny = std::is_same<E, f16_t>::value ? 0x1p-4f : 0x1p-24f;
+  // (the row sum adds the weights before they are rounded: an fp16 weight overflows at 65504 where its fp32 original is
+  // still an ordinary number, so the bound on the sum stays below that)
+  constexpr float kBig = std::is_same<E, f16_t>::value ? 0x1p15f : 0x1p24f, kTiny = std::is_same<E, f16_t>::value ? 0x1p-4f : 0x1p-24f;
   auto weights = [&](const f32x16& s, ex8 (&pf)[2]) FL_INLINE {
     auto form = [&]() FL_INLINE -> float {
       float rs = 0.f;

@@ -536,6 +536,12 @@ void fwd_kernel(const KParams p) {
   // The running maximum only moves when some row of the wave sees a score more than kTau (log2 units) above it,
   // so exp2 arguments stay <= kTau and the accumulators are rescaled on few tiles.  Any m gives the same O / l.
   constexpr float kTau = 8.0f;
+  // Soft-capped scores are bounded, so every tile of such a kernel forms its weights against the running reference as it
+  // stands (see weights_checked): the reference is then known when the tile's scores are modified, one step earlier,
+  // and is subtracted there, in the addend of a multiply-add that is issued anyway.  The modified scores of these
+  // kernels are relative to the reference of the moment; it can move only on the path that recomputes a tile's
+  // weights, which accounts for the difference.
+  constexpr bool kFoldRef = kSoftcap && !kDrop;  // (the dropout instances have no registers to spare for it)
 
   // Gate logits of this lane's output elements, fetched before the key loop when they fit the register budget so that
   // their latency is not paid in the epilogue.
@@ -558,6 +564,7 @@ void fwd_kernel(const KParams p) {
   f32x16 ofin[kDiff ? DVB : 1][kDiff ? QB : 1];  // branch-0 result kept while branch 1 runs (diff only)
   f32x16 oacc[DVB][QB];
   float m_run[QB], l_run[QB];
+  auto ref_now = [&](int qb) FL_INLINE { return (m_run[qb] == -INFINITY) ? 0.f : m_run[qb]; };
 
 #pragma unroll
   for (int br = 0; br < (kDiff ? 2 : 1); ++br) {
@@ -779,7 +786,7 @@ void fwd_kernel(const KParams p) {
             // ALiBi: slope * (rel0 + off) with off a per-register constant; slope * rel0 rides in the addend of the
             // multiply-add that precedes it, leaving one multiply-add with a literal per score
             const float alibi0 = kAlibi ? slope_l2 * rel0 : 0.f;
-            const float cap_shift = cap_c + alibi0;
+            const float cap_shift = cap_c + alibi0 - (kFoldRef ? ref_now(qb) : 0.f);
             auto combine = [&]() FL_INLINE {
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
@@ -1006,11 +1013,14 @@ void fwd_kernel(const KParams p) {
     // ---- P = exp2(s - m) (bf16 B operand of the second product) and row sums ----------------------------------------------
     // (the row sums take every weight; with dropout the weights that go on to the second product are then thinned:
     // t is the tile, whose keys enter the hash)
-    auto softmax_p = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], float (&rsum)[QB], int t) FL_INLINE {
+    // (kernels whose scores already are relative to a reference pass what the reference has moved by since, or the
+    // tag `relative` when it has not moved)
+    auto softmax_p = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], float (&rsum)[QB], int t, auto relative,
+                         const float (&moved)[QB]) FL_INLINE {
       const ex2 ones = {(E)1.0f, (E)1.0f};
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
-        const float mc = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2;
+        const float mc = kFoldRef ? moved[qb] : ((m_run[qb] == -INFINITY) ? 0.f : m_run[qb] * c2);
         float rs = 0.f;
         uint32_t drop_x0 = 0;
         if constexpr (kDrop) drop_x0 = drop_q[qb] + (uint32_t)(t * (BN / 2) + 2 * h) * kDropK;
@@ -1018,7 +1028,10 @@ void fwd_kernel(const KParams p) {
         for (int kb = 0; kb < KB; ++kb) {
           float pv[16];
 #pragma unroll
-          for (int i = 0; i < 16; ++i) pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
+          for (int i = 0; i < 16; ++i) {
+            if constexpr (kFoldRef && decltype(relative)::value) pv[i] = fast_exp2(s[kb][qb][i]);
+            else pv[i] = fast_exp2(__builtin_fmaf(s[kb][qb][i], c2, -mc));
+          }
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -1062,7 +1075,8 @@ void fwd_kernel(const KParams p) {
     auto weights_checked = [&](const f32x16 (&s)[KB][QB], ex8 (&pf)[QB][2 * KB], bool check, auto in_loop,
                                ex8 (&vfirst)[DVB], int vslot, int t, auto prefetch_v) FL_INLINE {
       float rs[QB];
-      softmax_p(s, pf, rs, t);
+      float moved[QB] = {};
+      softmax_p(s, pf, rs, t, std::true_type{}, moved);
       if constexpr (decltype(in_loop)::value) {
         // inside the pipelined step the exponentials share a block with the first product's MFMAs (issued by the
         // caller just before): interleave them
@@ -1085,8 +1099,20 @@ void fwd_kernel(const KParams p) {
         if (__builtin_amdgcn_ballot_w64(bad) != 0) {
           float mx[QB];
           row_max(s, mx);
+          if constexpr (kFoldRef) {
+            // the maxima are relative to the reference the scores were formed against, which is still the current one
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+              moved[qb] = ref_now(qb);
+              mx[qb] += moved[qb];
+            }
+          }
           rescale_if_grown(mx, true);
-          softmax_p(s, pf, rs, t);
+          if constexpr (kFoldRef) {
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) moved[qb] = ref_now(qb) - moved[qb];
+          }
+          softmax_p(s, pf, rs, t, std::false_type{}, moved);
         }
       }
 #pragma unroll

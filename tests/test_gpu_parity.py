@@ -306,6 +306,14 @@ def test_reference_free_weights_survive_extreme_logit_ranges(D, offsets):
     q, k, v = (t.bfloat16().to(DEV) for t in (q, k, v))
     assert_parity(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v)), "vanilla")
     assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(*f32(q, k, v), enable_gqa=True), "causal")
+    # soft-cap kernels subtract the running reference while they modify the scores, one step before the weights are
+    # formed; with a cap this wide the capped logits still jump by hundreds of nats, so the recomputing path runs on
+    # scores that are relative to a reference which then moves
+    cap = 1500.0
+    assert_parity(A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(cap)),
+                  O.attention_softcapped(*f32(q, k, v), score_mod=cap), "softcap")
+    assert_parity(A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(2), is_causal=True, softcap=cap),
+                  O.attention_alibi(*f32(q, k, v), score_mod=2, is_causal=True, honor_causal=True, softcap=cap), "alibi+softcap+causal")
 
 
 # ---- dense score_mod and invariant point attention -------------------------------------------------------------------------

@@ -70,3 +70,24 @@ def test_tiny_sweep_with_dropout_on_gpu(tmp_path):
     rows = R.main(["--suite", "backward", "--batch_size", "2", "--seqlen", "512", "--group_size", "1", "--dropout_p", "0.1",
                    "--output", str(tmp_path / "e")])
     assert {r[0] for r in rows} == {n + "_bwd" for n in R.dropout_registry(0.1)}
+
+
+def test_measured_traffic_file_covers_every_workload_and_agrees_with_the_summaries():
+    # bench.py reports roofline.traffic from profiles/hbm_traffic.json; the figure has to be the one the per-workload
+    # profiler summary beside it states, for every benchmark workload
+    import glob
+    import json
+    import os
+    import re
+    from flashlight_amd import workloads as W
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "profiles")
+    table = json.load(open(os.path.join(root, "hbm_traffic.json")))["bytes_per_launch"]
+    assert set(table) == {w.name for w in W.build_workloads()}
+    seen = {}
+    for path in glob.glob(os.path.join(root, "*_cfg*.md")):
+        text = open(path).read()
+        name = re.match(r"# (\S+) ", text).group(1)
+        seen[name] = float(re.search(r"^Total ([\d.]+) MB against", text, re.M).group(1)) * 1e6
+    assert set(seen) == set(table)
+    for name, measured in seen.items():
+        assert abs(table[name] - measured) <= 0.5e5, name

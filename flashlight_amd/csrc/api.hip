@@ -429,15 +429,27 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
 bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   static const bool disabled = std::getenv("FL_NO_PAIRBIAS") != nullptr;  // A/B knob: the general kernel instead
   if (disabled) return false;
-  if (p->Dqk != 32 || p->Dv != 32 || p->mask_kind != FL_MASK_NONE || p->alibi_heads > 0 || p->softcap > 0.f ||
+  if (p->Dqk != p->Dv || p->mask_kind != FL_MASK_NONE || p->alibi_heads > 0 || p->softcap > 0.f ||
       p->diff || p->attended_dump || p->dropout_threshold || p->lse)
     return false;
-  if (!p->bias[0] || p->bias[1] || p->bias_dtype[0] != p->dtype) return false;
-  const int64_t* bst = p->bias_strides[0];
-  const int div = p->bias_batch_div[0];
-  if (div < 2 || p->B % div != 0 || bst[3] != 1 || bst[2] == 0 || bst[1] == 0) return false;
-  if (p->Lk % 32 != 0 || !fl::pairbias_has_shape(p->Lk / 32)) return false;
-  if (reinterpret_cast<uintptr_t>(p->bias[0]) % 16 != 0 || bst[0] % 8 || bst[1] % 8 || bst[2] % 8) return false;
+  // one operand that several consecutive batch entries share (dense over heads, queries and keys), and optionally one
+  // that is a row of keys per batch entry, the same for every head and query; in either order
+  int pi = -1, ri = -1;
+  for (int i = 0; i < 2; ++i) {
+    if (!p->bias[i]) continue;
+    const int64_t* st = p->bias_strides[i];
+    if (p->bias_dtype[i] != p->dtype || st[3] != 1) return false;
+    if (p->bias_batch_div[i] >= 2 && st[1] != 0 && st[2] != 0 && pi < 0) pi = i;
+    else if (p->bias_batch_div[i] == 1 && st[1] == 0 && st[2] == 0 && ri < 0) ri = i;
+    else return false;
+  }
+  if (pi < 0) return false;
+  const int64_t* bst = p->bias_strides[pi];
+  const int div = p->bias_batch_div[pi];
+  if (p->B % div != 0) return false;
+  if (p->Lk % 32 != 0 || !fl::pairbias_has_shape(p->Dqk, p->Lk / 32, p->gate != nullptr, ri >= 0)) return false;
+  if (reinterpret_cast<uintptr_t>(p->bias[pi]) % 16 != 0 || bst[0] % 8 || bst[1] % 8 || bst[2] % 8) return false;
+  if (ri >= 0 && (reinterpret_cast<uintptr_t>(p->bias[ri]) % 16 != 0 || p->bias_strides[ri][0] % 8)) return false;
   if (reinterpret_cast<uintptr_t>(p->o) % 8 != 0 || (p->gate && reinterpret_cast<uintptr_t>(p->gate) % 8 != 0)) return false;
   // per-lane byte offsets inside one (batch entry, head) slice are 32-bit
   const int64_t worst = std::max(std::max(p->q_strides[2], p->o_strides[2]), p->gate ? p->gate_strides[2] : 0);
@@ -471,8 +483,12 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   k.Lq = p->Lq;
   k.Lk = p->Lk;
   k.scale = p->scale;
-  k.bias = static_cast<const fl::bf16_t*>(p->bias[0]);
+  k.bias = static_cast<const fl::bf16_t*>(p->bias[pi]);
   k.bdiv = div;
+  if (ri >= 0) {
+    k.rowb = static_cast<const fl::bf16_t*>(p->bias[ri]);
+    k.rbs = p->bias_strides[ri][0];
+  }
   k.gate = static_cast<const fl::bf16_t*>(p->gate);
   k.n_qtiles = (p->Lq + 127) / 128;
   // Launch shape: every workgroup should be resident at once (two per compute unit, 32 compute units per XCD), and a
@@ -545,7 +561,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]) {
       out[1] = 64;
       out[2] = 256;
       out[3] = pb_grid;
-      out[4] = 32768;
+      out[4] = 2 * (p->Dqk == 32 ? 6 : 4) * 64 * p->Dqk * 2 + (pb.rowb ? 4 * 2 * 1024 : 0);
       out[6] = 1;
     }
   }
@@ -564,7 +580,7 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
     int pb_grid = 0;
     if (plan_pairbias(p, &pb, &pb_grid)) {
       const hipError_t e = (p->dtype == FL_F16 ? fl::launch_pairbias_f16 : fl::launch_pairbias_bf16)(
-          p->Lk / 32, p->gate != nullptr, pb, pb_grid, stream);
+          p->Dqk, p->Lk / 32, p->gate != nullptr, pb.rowb != nullptr, pb, pb_grid, stream);
       if (e != hipSuccess) return fail((int)e, "launch of the shared-bias forward failed: %s", hipGetErrorString(e));
       return 0;
     }

@@ -1,6 +1,8 @@
 // Attention with one dense bias that many batch entries share (the Evoformer's row attention: N_seq rows of an MSA
 // attend over N_res residues, and every row adds the same pair bias [H, N_res, N_res]; reference
-// attention_variants/evoformer.py:8-36), head dim 32, a few hundred keys.
+// attention_variants/evoformer.py:8-36), head dim 32 or 64, a few hundred keys; optionally a second bias that is one
+// row of keys per batch entry, the same for every head and query (the mask bias [B, N_seq, 1, 1, N_res] of the
+// reference's benchmark inputs, evoformer.py:45).
 //
 // The general forward (fwd_kernel.h) gives such a call one short-lived workgroup per (row, head, 128 queries): six key
 // tiles, a bias tile staged next to every K/V tile, and eight or nine vector instructions per score against eight
@@ -14,6 +16,9 @@
 //     key 16m + j on row j of the group, weighted 1/scale (split in two bf16 terms, relative error 2^-17), so the
 //     accumulators hold qk + bias/scale and the weights are exp2(scale * log2(e) * acc - ref): per score one
 //     multiply-add, one exponential, one addition for the row sum and half a pack.
+//   * the row bias takes the same road as a rank-one product: A = the row's values down the keys (two copies side by
+//     side), B = the two terms of 1/scale across the queries; the row of the next entry rides into LDS with the
+//     transfers of the current one.
 // Infinite bias entries are clamped to the largest finite value when the fragments are loaded (0 * inf inside the
 // selector product would poison the 15 other keys of the group); as an additive term that is the same mask.
 #pragma once
@@ -39,6 +44,8 @@ struct PParams {
   int32_t chunk_len;  // batch entries per chunk (the last chunk of a group may be shorter)
   int32_t hgroup;     // heads whose workgroups are kept on one XCD (they share cache lines when heads are adjacent)
   int32_t n_units;    // (bias groups * chunks) * (H / hgroup)
+  const bf16_t* rowb;  // optional second bias: one row of Lk values per batch entry, unit key stride
+  int64_t rbs;         // its element stride between batch entries
 };
 
 // 16 / 8 bytes per lane from global memory into registers, and 8 bytes back, as asm: inside the streaming loop every
@@ -64,18 +71,39 @@ __device__ __forceinline__ void pin_loaded(V& v) {
   asm volatile("" : "+v"(v));
 }
 
-template <int NKB_, bool GATE_, class Elem_>
+template <int NKB_, bool GATE_, class Elem_, int D_ = 32, bool ROWB_ = false, bool EXACT_ = false>
 struct PairBiasTraits {
   using Elem = Elem_;
   static constexpr int NKB = NKB_;       // 32-key blocks per row: Lk = 32 * NKB
   static constexpr bool GATE = GATE_;
-  static constexpr int D = 32, BN = 64, NW = 4, NT = 256, BM = 128;
+  static constexpr bool ROWB = ROWB_;    // a row bias per batch entry besides the shared one
+  // 1 / scale is exact in the element type (a power of two, say): its second term is zero and the products with it go
+  static constexpr bool EXACT = EXACT_;
+  static constexpr int D = D_, BN = 64, NW = 4, NT = 256, BM = 128;
+  static constexpr int KS = D / 16;      // k-steps of the first product
+  static constexpr int DVB = D / 32;     // 32-column blocks of the result
   static constexpr int NTI = NKB / 2;    // key tiles per batch entry
-  static constexpr int NS = 6;           // K/V tiles resident in LDS
+#ifdef FL_PB_NS64
+  static constexpr int NS = D == 32 ? 6 : FL_PB_NS64;
+#else
+  static constexpr int NS = D == 32 ? 6 : 4;  // K/V tiles resident in LDS
+#endif
   static constexpr int AHEAD = NS - 1;   // transfers run this many tiles ahead of their use
+  // K fragments read from LDS one block ahead of the scores that use them (head dim 64 has no registers for that)
+#ifdef FL_PB_KAHEAD
+  static constexpr bool KAHEAD = FL_PB_KAHEAD;
+#else
+  static constexpr bool KAHEAD = D == 32;
+#endif
+  static_assert(D == 32 || D == 64, "head dim");
   static_assert(NKB % 2 == 0 && NTI >= 2, "whole tiles");
   static constexpr int TILE_BYTES = BN * D * 2;
-  static constexpr int K_OFF = 0, V_OFF = NS * TILE_BYTES, LDS_BYTES = 2 * NS * TILE_BYTES;
+  static constexpr int XPW = TILE_BYTES / (NW * 1024);  // 1 KiB wave transfers per wave and operand tile
+  static constexpr int ROW_SLOT = 1024;                 // LDS bytes of one staged bias row (a whole wave transfer)
+  static_assert(32 * NKB * 2 <= ROW_SLOT, "a bias row fits one wave transfer");
+  // per wave two row slots: the current entry's row and the next one's
+  static constexpr int K_OFF = 0, V_OFF = NS * TILE_BYTES, R_OFF = 2 * NS * TILE_BYTES;
+  static constexpr int LDS_BYTES = R_OFF + (ROWB ? NW * 2 * ROW_SLOT : 0);
 };
 
 template <class T>
@@ -85,13 +113,14 @@ void pairbias_kernel(const PParams p) {
   typedef E ex8 __attribute__((ext_vector_type(8)));
   typedef E ex4 __attribute__((ext_vector_type(4)));
   typedef E ex2 __attribute__((ext_vector_type(2)));
-  constexpr int NKB = T::NKB, NTI = T::NTI, NS = T::NS, D = T::D, BN = T::BN;
-  constexpr bool kGate = T::GATE;
+  constexpr int NKB = T::NKB, NTI = T::NTI, NS = T::NS, D = T::D, BN = T::BN, KS = T::KS, DVB = T::DVB, XPW = T::XPW;
+  constexpr bool kGate = T::GATE, kRowB = T::ROWB, kAheadK = T::KAHEAD;
+  constexpr int kParts = T::EXACT ? 1 : 2;  // terms of 1 / scale
   constexpr float kLog2e = 1.4426950408889634f;
   using LK = TileLayout<D>;
   using LV = TileLayout<D>;
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[T::LDS_BYTES];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // T::LDS_BYTES
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
@@ -154,10 +183,27 @@ void pairbias_kernel(const PParams p) {
         sel[m][1][j] = on ? w_lo : (E)0.0f;
       }
   }
+  // row bias: B operand of the rank-one product, lane (query r, h) holds rows 8 h .. 8 h + 7 of the 16: rows 0 and 1
+  // carry the two terms of 1 / scale, the A operand has the row's value in columns 0 and 1
+  ex8 rsel;
+  uint32_t rkeep = 0;  // all ones in the lanes that hold columns 0 .. 7 of the A operand
+  if constexpr (kRowB) {
+    const float w = 1.0f / p.scale;
+    const E w_hi = (E)w;
+    const E w_lo = (E)(w - (float)w_hi);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) rsel[j] = (E)0.0f;
+    if (h == 0) {
+      rsel[0] = w_hi;
+      rsel[1] = w_lo;
+      rkeep = 0xFFFFFFFFu;
+    }
+  }
   const float c2 = p.scale * kLog2e;  // acc * c2 = (qk * scale + bias) in log2 units
 
   // ---- addresses.  Per-lane byte offsets are constant; scalar bases move with the batch entry and the tile.
-  // K/V tile = 64 rows x 64 bytes = 4 wave transfers of 1 KiB: wave w brings transfer w, lane l -> (row, physical chunk)
+  // K/V tile = 64 rows x 2 D bytes = 4 XPW wave transfers of 1 KiB: wave w brings transfers w, w + 4, ...; lane l ->
+  // (row, physical chunk); transfer j of a wave lies 64 / XPW rows (whole swizzle periods) below its transfer j - 1
   unsigned koff, voff;
   {
     const int id = wave * 64 + lane, row = id / LK::CPR, pc = id % LK::CPR;
@@ -170,46 +216,72 @@ void pairbias_kernel(const PParams p) {
   const uint64_t qbase = uniform_ptr(p.q + (int64_t)head * p.qs[1]);
   const uint64_t obase = uniform_ptr(p.o + (int64_t)head * p.os[1]);
   const uint64_t gbase = kGate ? uniform_ptr(p.gate + (int64_t)head * p.gs[1]) : 0;
-  const unsigned qoff = (unsigned)(qrow * (int)p.qs[2] + 8 * h) * 2u;  // + 32 bytes for the second k-step
+  const unsigned qoff = (unsigned)(qrow * (int)p.qs[2] + 8 * h) * 2u;  // + 32 bytes per k-step
   const unsigned ooff = (unsigned)(qrow * (int)p.os[2] + 4 * h) * 2u;  // + 16 bytes per group of 8 value columns
   const unsigned goff = kGate ? (unsigned)(qrow * (int)p.gs[2] + 4 * h) * 2u : 0u;
+  // the row bias: every wave stages its own copy of the row (lane l brings 16 bytes; lanes past the row's end repeat
+  // its start), slot (entry % 2) of the wave's two
+  const uint64_t rbase = kRowB ? uniform_ptr(p.rowb) : 0;
+  const unsigned roff = (unsigned)(lane % (NKB * 4)) * 16u;
+  const unsigned lds_r = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)smem + T::R_OFF + wave * 2 * T::ROW_SLOT);
+  const unsigned k_step_bytes = __builtin_amdgcn_readfirstlane((unsigned)((64 / XPW) * (int)p.ks[2] * 2));
+  const unsigned v_step_bytes = __builtin_amdgcn_readfirstlane((unsigned)((64 / XPW) * (int)p.vs[2] * 2));
 
   // tile j of the stream (entry j / NTI of the chunk, tile j % NTI of its keys; past the end the last entry again, so
   // that every step issues the same operations) -> ring slot j % NS
   auto issue_tile = [&](int item, int t, int slot) FL_INLINE {
     const int64_t fb = fb0 + min(item, n_items - 1);
-    dma16(kbase + (uint64_t)((fb * p.ks[0] + (int64_t)t * BN * p.ks[2]) * 2), koff, lds_k + slot * T::TILE_BYTES);
-    dma16(vbase + (uint64_t)((fb * p.vs[0] + (int64_t)t * BN * p.vs[2]) * 2), voff, lds_v + slot * T::TILE_BYTES);
+    const uint64_t kb_ = kbase + (uint64_t)((fb * p.ks[0] + (int64_t)t * BN * p.ks[2]) * 2);
+    const uint64_t vb_ = vbase + (uint64_t)((fb * p.vs[0] + (int64_t)t * BN * p.vs[2]) * 2);
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) dma16(kb_ + (uint64_t)(j * k_step_bytes), koff, lds_k + slot * T::TILE_BYTES + j * 4096);
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) dma16(vb_ + (uint64_t)(j * v_step_bytes), voff, lds_v + slot * T::TILE_BYTES + j * 4096);
+  };
+  auto issue_row = [&](int item) FL_INLINE {
+    const int64_t fb = fb0 + min(item, n_items - 1);
+    dma16(rbase + (uint64_t)(fb * p.rbs * 2), roff, lds_r + (item % 2) * T::ROW_SLOT);
+  };
+  // A operand of the row-bias product for block kb of entry `item`: the value of key 32 kb + r, twice, in the lanes
+  // of the first half; infinite values clamped like the shared bias
+  auto row_frag = [&](int item, int kb) FL_INLINE -> ex8 {
+    const unsigned char* rp = smem + T::R_OFF + (wave * 2 + item % 2) * T::ROW_SLOT;
+    uint32_t x = *reinterpret_cast<const uint16_t*>(rp + (32 * kb + r) * 2);
+    constexpr uint32_t kInf = std::is_same<E, f16_t>::value ? 0x7C00u : 0x7F80u;
+    x -= ((x & 0x7FFFu) == kInf) ? 1u : 0u;
+    u32x4 raw = {(x | (x << 16)) & rkeep, 0u, 0u, 0u};
+    return __builtin_bit_cast(ex8, raw);
   };
 
   // ---- K fragments (A operands of S^T = K . Q^T) of block b of the tile in ring slot `slot`
-  auto k_frags = [&](ex8 (&kf)[2], int slot, int b) FL_INLINE {
+  auto k_frags = [&](ex8 (&kf)[KS], int slot, int b) FL_INLINE {
     const unsigned char* kt = smem + T::K_OFF + slot * T::TILE_BYTES;
     const int row = 32 * b + r;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int ks = 0; ks < KS; ++ks)
       kf[ks] = *reinterpret_cast<const ex8*>(kt + row * (D * 2) + LK::swz_k(row, 2 * ks + h) * 16);
   };
   // ---- S^T block: K fragments as A operand, Q fragments as B; then the bias through the selectors
-  auto scores = [&](f32x16& s, const ex8 (&kf)[2], const ex8 (&qf)[2], int kb) FL_INLINE {
+  auto scores = [&](f32x16& s, const ex8 (&kf)[KS], const ex8 (&qf)[KS], int kb, const ex8& rowf) FL_INLINE {
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) s = mfma32(kf[ks], qf[ks], s);
+    for (int ks = 0; ks < KS; ++ks) s = mfma32(kf[ks], qf[ks], s);
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int part = 0; part < 2; ++part) s = mfma32(sel[m][part], bfrag[kb][m], s);
+      for (int part = 0; part < kParts; ++part) s = mfma32(sel[m][part], bfrag[kb][m], s);
+    if constexpr (kRowB) s = mfma32(rowf, rsel, s);
   };
   // A operand of O^T += V^T . P^T for 16-key chunk c of the tile (the transposing LDS read of the general kernel)
-  auto v_frag = [&](int slot, int c) FL_INLINE -> ex8 {
+  auto v_frag = [&](int slot, int c, int dvb) FL_INLINE -> ex8 {
     const unsigned char* vt = smem + T::V_OFF + slot * T::TILE_BYTES;
     ex8 vf;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int i16 = lane % 16, g = (lane / 16) % 2;
       const int row = 16 * c + 8 * j + 4 * h + i16 / 4;
-      const int col = g * 16 + 4 * (i16 % 4);
+      const int col = dvb * 32 + g * 16 + 4 * (i16 % 4);
       const unsigned char* ap = vt + row * (D * 2) + LV::swz_v(row, col / 8) * 16 + (col % 8) * 2;
       typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
       const s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(ap));
@@ -223,7 +295,7 @@ void pairbias_kernel(const PParams p) {
   // ---- softmax state of the current entry.  ref is the reference the weights are formed against, in log2 units; it
   // starts at 0 and moves only when a row sum says it must (a weight overflowed, or a whole block underflowed with
   // nothing accumulated yet): any reference gives the same O / l.
-  f32x16 oacc;
+  f32x16 oacc[DVB];
   float ref = 0.f, l_run = 0.f;
   // (the row sum adds the weights before they are rounded: an fp16 weight overflows at 65504 where its fp32 original is
   // still an ordinary number, so the bound on the sum stays below that)
@@ -263,56 +335,67 @@ void pairbias_kernel(const PParams p) {
       ref = use;
       l_run *= alpha;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[i] *= alpha;
+      for (int dvb = 0; dvb < DVB; ++dvb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dvb][i] *= alpha;
       rs = form();
     }
     l_run += rs;
   };
 
-  // ---- prologue: queries of the first entry, the first AHEAD tiles, scores of the first block
-  ex8 qf[2];
+  // ---- prologue: queries (and bias row) of the first entry, the first AHEAD tiles, scores of the first block
+  ex8 qf[KS];
   {
     const uint64_t qb0 = qbase + (uint64_t)((int64_t)fb0 * p.qs[0] * 2);
-    u32x4 a = load16_counted(qb0, qoff), b = load16_counted(qb0, qoff + 32u);
+    u32x4 qraw[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qraw[ks] = load16_counted(qb0, qoff + 32u * ks);
+    if constexpr (kRowB) issue_row(0);
 #pragma unroll
     for (int j = 0; j < T::AHEAD; ++j) issue_tile(j / NTI, j % NTI, j);
     dma_wait<0>();
-    pin_loaded(a);
-    pin_loaded(b);
-    qf[0] = __builtin_bit_cast(ex8, a);
-    qf[1] = __builtin_bit_cast(ex8, b);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      pin_loaded(qraw[ks]);
+      qf[ks] = __builtin_bit_cast(ex8, qraw[ks]);
+    }
   }
   __syncthreads();
   f32x16 s_a, s_b;
-  ex8 kf[2];  // K fragments of the block whose scores are formed next, read from LDS one block ahead of their use
+  ex8 kf[KS];  // K fragments of the block whose scores are formed next (with KAHEAD: read one block ahead of their use)
+  ex8 rowf;    // row-bias fragment of that block
   k_frags(kf, 0, 0);
-  scores(s_a, kf, qf, 0);
-  k_frags(kf, 0, 1);
+  if constexpr (kRowB) rowf = row_frag(0, 0);
+  scores(s_a, kf, qf, 0, rowf);
+  if constexpr (kAheadK) k_frags(kf, 0, 1);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+  for (int dvb = 0; dvb < DVB; ++dvb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dvb][i] = 0.f;
 
-  // Operations a wave issues, in order, per entry:  at the barrier point of tile t: the two transfers of the tile AHEAD
-  // tiles on, and at t == 0 also the gate loads of this entry (4, if there is a gate) and the query loads of the next (2);
-  // after the entry's last block: 4 stores.  The barrier point of tile t waits for the transfers of tile t + 1, issued
-  // AHEAD - 1 barrier points earlier; allowed(t) counts what was issued after them: the extras of that point, and
-  // everything of the points since.  Running far ahead keeps the stores out of the way: a wait completes in issue
-  // order, so a transfer issued after the stores is only known to have landed once the stores are acknowledged, and
-  // with AHEAD = 5 that is first asked four tiles after them.
-  constexpr int NI = 2 + (kGate ? 4 : 0);
+  // Operations a wave issues, in order, per entry:  at the barrier point of tile t: the PT transfers of the tile AHEAD
+  // tiles on, and at t == 0 also the gate loads of this entry (if there is a gate), the query loads of the next and
+  // the transfer of its bias row (NI in all); after the entry's last block: ST stores.  The barrier point of tile t
+  // waits for the transfers of tile t + 1, issued AHEAD - 1 barrier points earlier; allowed(t) counts what was issued
+  // after them: the extras of that point, and everything of the points since.  Running far ahead keeps the stores out
+  // of the way: a wait completes in issue order, so a transfer issued after the stores is only known to have landed
+  // once the stores are acknowledged.
+  constexpr int PT = 2 * XPW, ST = 4 * DVB;
+  constexpr int NI = KS + (kGate ? 4 * DVB : 0) + (kRowB ? 1 : 0);
   constexpr int AHEAD = T::AHEAD;
-  auto extras = [](int j) constexpr { const int t = ((j % NTI) + NTI) % NTI; return (t == 0 ? NI : 0) + (t == NTI - 1 ? 4 : 0); };
+  auto extras = [](int j) constexpr { const int t = ((j % NTI) + NTI) % NTI; return (t == 0 ? NI : 0) + (t == NTI - 1 ? ST : 0); };
   auto allowed = [extras](int t) constexpr {
     int n = extras(t + 1 - AHEAD);
-    for (int j = t + 2 - AHEAD; j < t; ++j) n += 2 + extras(j);
+    for (int j = t + 2 - AHEAD; j < t; ++j) n += PT + extras(j);
     return n;
   };
   for (int item = 0; item < n_items; ++item) {
     const int slot0 = (item * NTI) % NS;
-    u32x4 qn_a, qn_b;        // next entry's query fragments, in flight from tile 0 on
-    u32x2 gl[4];             // this entry's gate logits, likewise
+    u32x4 qn[KS];            // next entry's query fragments, in flight from tile 0 on
+    u32x2 gl[4 * DVB];       // this entry's gate logits, likewise
     const int64_t fbn = fb0 + min(item + 1, n_items - 1);
     const int64_t fbc = fb0 + item;
-    ex8 qnext[2];
+    ex8 qnext[KS];
     static_while<0, NTI>([&](auto tt) FL_INLINE {
       constexpr int t = decltype(tt)::value;
       const int slot = (slot0 + t) % NS;
@@ -323,7 +406,7 @@ void pairbias_kernel(const PParams p) {
         if constexpr (b == 0) {
           // barrier point of tile t, before anything of the tile after it is touched
           // (the last point of an entry also takes the loads of point 0 into use: only the transfers issued since may stay out)
-          constexpr int kAllowed = t == NTI - 1 && 2 * (NTI - 2) < allowed(t) ? 2 * (NTI - 2) : allowed(t);
+          constexpr int kAllowed = t == NTI - 1 && PT * (NTI - 2) < allowed(t) ? PT * (NTI - 2) : allowed(t);
           static_assert(kAllowed < 64, "vmcnt is a 6-bit counter");
           dma_wait<kAllowed>();
           __syncthreads();  // tile t + 1 is visible; everyone is done with tile t - 1, whose slot the new tile takes
@@ -332,49 +415,65 @@ void pairbias_kernel(const PParams p) {
             if constexpr (kGate) {
               const uint64_t gb = gbase + (uint64_t)(fbc * p.gs[0] * 2);
 #pragma unroll
-              for (int g = 0; g < 4; ++g) gl[g] = load8_counted(gb, goff + 16u * g);
+              for (int dvb = 0; dvb < DVB; ++dvb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) gl[4 * dvb + g] = load8_counted(gb, goff + 64u * dvb + 16u * g);
             }
             const uint64_t qb = qbase + (uint64_t)(fbn * p.qs[0] * 2);
-            qn_a = load16_counted(qb, qoff);
-            qn_b = load16_counted(qb, qoff + 32u);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) qn[ks] = load16_counted(qb, qoff + 32u * ks);
+            // (the slot it goes to held the previous entry's row, last read a whole entry ago)
+            if constexpr (kRowB) issue_row(item + 1);
           }
           if constexpr (t == NTI - 1) {
             // everything issued at tile 0 has landed (the wait above covers later transfers): next entry's queries
-            pin_loaded(qn_a);
-            pin_loaded(qn_b);
-            qnext[0] = __builtin_bit_cast(ex8, qn_a);
-            qnext[1] = __builtin_bit_cast(ex8, qn_b);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              pin_loaded(qn[ks]);
+              qnext[ks] = __builtin_bit_cast(ex8, qn[ks]);
+            }
             if constexpr (kGate) {
 #pragma unroll
-              for (int g = 0; g < 4; ++g) pin_loaded(gl[g]);
+              for (int g = 0; g < 4 * DVB; ++g) pin_loaded(gl[g]);
             }
           }
         }
         // Scores of the next block (the first block of the next entry after the last one of this) go to the matrix pipe
-        // under this block's exponentials; their K fragments were read from LDS during the previous block, and the
-        // LDS reads issued now (K fragments for the block after next, V fragments for this block's second product) have
-        // the exponentials to land under.
+        // under this block's exponentials.  With KAHEAD their K fragments were read from LDS during the previous block
+        // and the reads issued now are for the block after next; without, they are read now, first thing.  The V
+        // fragments for this block's second product have the exponentials to land under.
         f32x16& cur = (kb % 2 == 0) ? s_a : s_b;
         f32x16& nxt = (kb % 2 == 0) ? s_b : s_a;
-        ex8 kf_ahead[2], vf[2];
-        k_frags(kf_ahead, (slot + 1) % NS, b);  // block kb + 2: same half of the next tile in the ring
+        ex8 kf_ahead[KS], vf[2][DVB];
+        if constexpr (kAheadK) k_frags(kf_ahead, (slot + 1) % NS, b);  // block kb + 2: same half of the next tile in the ring
+        else k_frags(kf, (slot + (b == 1 ? 1 : 0)) % NS, 1 - b);          // block kb + 1
+        if constexpr (kRowB) rowf = last_block ? row_frag(item + 1, 0) : row_frag(item, kb + 1);
 #pragma unroll
-        for (int c = 0; c < 2; ++c) vf[c] = v_frag(slot, 2 * b + c);
-        if constexpr (last_block) scores(nxt, kf, qnext, 0);
-        else scores(nxt, kf, qf, kb + 1);
-        kf[0] = kf_ahead[0];
-        kf[1] = kf_ahead[1];
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+          for (int dvb = 0; dvb < DVB; ++dvb) vf[c][dvb] = v_frag(slot, 2 * b + c, dvb);
+        if constexpr (last_block) scores(nxt, kf, qnext, 0, rowf);
+        else scores(nxt, kf, qf, kb + 1, rowf);
+        if constexpr (kAheadK) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) kf[ks] = kf_ahead[ks];
+        }
         ex8 pf[2];
         weights(cur, pf);
-        // 6 LDS reads first, then the 6 score MFMAs spread over the exponentials (64 vector instructions per block)
-        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 6, 0);
+        // the LDS reads first, then the score MFMAs spread over the exponentials (64 vector instructions per block)
+        constexpr int kReads = KS + 4 * DVB + (kRowB ? 1 : 0), kScoreMfmas = KS + 2 * kParts + (kRowB ? 1 : 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, kReads, 0);
+        // (without KAHEAD the first MFMA waits for the K fragments just asked for: some exponentials go first)
+        if constexpr (!kAheadK) __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, 8, 0);
 #pragma unroll
-        for (int i = 0; i < 6; ++i) {
+        for (int i = 0; i < kScoreMfmas; ++i) {
           __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, (60 + kScoreMfmas - 1) / kScoreMfmas, 0);
         }
 #pragma unroll
-        for (int c = 0; c < 2; ++c) oacc = mfma32(vf[c], pf[c], oacc);
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+          for (int dvb = 0; dvb < DVB; ++dvb) oacc[dvb] = mfma32(vf[c][dvb], pf[c], oacc[dvb]);
         return true;
       });
       return true;
@@ -385,27 +484,31 @@ void pairbias_kernel(const PParams p) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const uint64_t ob = obase + (uint64_t)(fbc * p.os[0] * 2);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        ex4 o4;
-        if constexpr (kGate) {
-          const ex4 g4 = __builtin_bit_cast(ex4, gl[g]);
+      for (int dvb = 0; dvb < DVB; ++dvb)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
-            o4[e] = (E)(oacc[4 * g + e] * inv * sg);
+        for (int g = 0; g < 4; ++g) {
+          ex4 o4;
+          if constexpr (kGate) {
+            const ex4 g4 = __builtin_bit_cast(ex4, gl[4 * dvb + g]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
+              o4[e] = (E)(oacc[dvb][4 * g + e] * inv * sg);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o4[e] = (E)(oacc[dvb][4 * g + e] * inv);
           }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o4[e] = (E)(oacc[4 * g + e] * inv);
+          store8_counted(ob, ooff + 64u * dvb + 16u * g, __builtin_bit_cast(u32x2, o4));
         }
-        store8_counted(ob, ooff + 16u * g, __builtin_bit_cast(u32x2, o4));
-      }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+      for (int dvb = 0; dvb < DVB; ++dvb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dvb][i] = 0.f;
       ref = 0.f;
       l_run = 0.f;
-      qf[0] = qnext[0];
-      qf[1] = qnext[1];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[ks] = qnext[ks];
     }
   }
   dma_wait<0>();  // nothing of this wave may still be on its way into LDS when the workgroup's allocation is released

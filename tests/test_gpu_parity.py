@@ -553,14 +553,51 @@ def test_shared_bias_streaming_kernel_half_masked_lanes(dtype, drop):
     assert_parity(out, O.attention_evoformer(*f32(q, k, v), [bias.float()]), f"half-masked lanes {dtype}")
 
 
+@pytest.mark.parametrize("D,B,N,S,H,gate,dtype,mask,scale", [
+    (64, 2, 8, 256, 4, False, torch.bfloat16, "1e9", None),      # the reference benchmark's inputs (evoformer.py:41-49)
+    (64, 1, 5, 256, 2, False, torch.bfloat16, "randn", None),    # an odd number of entries: the last chunk is short
+    (64, 1, 9, 256, 4, False, torch.bfloat16, "inf", 0.1),       # 1 / scale inexact in bf16: both selector terms
+    (64, 1, 6, 256, 2, False, torch.float16, "randn", None),
+    (32, 1, 13, 384, 8, True, torch.bfloat16, "1e9", None),      # head dim 32 with mask bias, pair bias and gate
+    (32, 2, 7, 256, 4, False, torch.bfloat16, "inf", None),
+    (32, 1, 10, 320, 2, True, torch.float16, "randn", None),
+])
+def test_shared_bias_streaming_kernel_with_a_row_bias(D, B, N, S, H, gate, dtype, mask, scale):
+    # two operands: a row of keys per batch entry (the reference's mask bias [B, N, 1, 1, S]) and the shared pair bias
+    # [B, 1, H, S, S]; the streaming kernel adds both on the matrix pipe.  Either order of the operands.
+    g = torch.Generator().manual_seed(35)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dtype).to(DEV)  # noqa: E731
+    q, k, v = mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D)
+    pair = mk(B, 1, H, S, S)
+    if mask == "randn":
+        row = mk(B, N, 1, 1, S)
+    else:
+        keep = (torch.rand(B, N, 1, 1, S, generator=g) > 0.25).to(DEV)
+        keep[..., 0] = True
+        low = float("-inf") if mask == "inf" else (-1e9 if dtype == torch.bfloat16 else -6e4)
+        row = torch.where(keep, 0.0, low).to(dtype)
+    gt = mk(B, N, S, H, D) if gate else None
+    ops4 = [t.reshape(-1, S, H, D).transpose(1, 2) for t in (q, k, v)]
+    p, _keep = _ffi._fill_params(_ffi.load_library(), *ops4, torch.empty(B * N, H, S, D, dtype=dtype, device=DEV), H, H, None,
+                                 _ffi.MASK_NONE, 0, 0, None, 0, 0.0,
+                                 [(row.reshape(B * N, 1, 1, S), 1), (pair.reshape(B, H, S, S), N)], None, False, 0.0, None)
+    assert _ffi.plan(p)["streaming"] == 1
+    kw = {} if scale is None else {"sm_scale": scale}
+    ref = O.attention_evoformer(*f32(q, k, v), [row.float(), pair.float()], gate=None if gt is None else gt.float(), **kw)
+    for biases in ([row, pair], [pair, row]):
+        out = A.attention_reference(q, k, v, biases, gate=gt, **kw) if gate else A.attention_reference(q, k, v, biases, **kw)
+        assert_parity(out, ref, f"D{D} B{B} N{N} S{S} H{H} {mask}")
+
+
 def test_shared_bias_streaming_kernel_matches_the_general_kernel():
-    # same call through both kernels: a second bias operand (all zeros) makes the library take the general one
+    # same call through both kernels: a second bias operand that differs by head (all zeros) makes the library take the
+    # general one
     g = torch.Generator().manual_seed(32)
     mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(DEV)  # noqa: E731
     B, N, S, H = 1, 24, 384, 4
     q, k, v, gt = mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32), mk(B, N, S, H, 32)
     bias = mk(B, 1, H, S, S)
-    zero = torch.zeros(B, N, 1, 1, S, dtype=torch.bfloat16, device=DEV)
+    zero = torch.zeros(B, N, H, 1, S, dtype=torch.bfloat16, device=DEV)
     fast = A.attention_reference(q, k, v, [bias], gate=gt)
     general = A.attention_reference(q, k, v, [zero, bias], gate=gt)
     assert (fast.float() - general.float()).abs().max().item() <= 2e-2

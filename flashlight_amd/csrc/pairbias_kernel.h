@@ -63,8 +63,17 @@ __device__ __forceinline__ u32x2 load8_counted(uint64_t sbase, unsigned voff) {
   asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
   return v;
 }
-__device__ __forceinline__ void store8_counted(uint64_t sbase, unsigned voff, u32x2 data) {
-  asm volatile("global_store_dwordx2 %0, %1, %2" ::"v"(voff), "v"(data), "s"(sbase));
+// (a store of more than 8 bytes still reads its data registers for two cycles after it has issued, and the compiler,
+// which inserts that distance for its own stores, does not look into an asm: the idle cycles are part of it)
+__device__ __forceinline__ void store16_counted(uint64_t sbase, unsigned voff, u32x4 data) {
+  asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(voff), "v"(data), "s"(sbase));
+}
+// a <-> b across the two halves of the wave: lanes 32..63 of `a` change places with lanes 0..31 of `b`
+__device__ __forceinline__ void swap_halves(uint32_t& a, uint32_t& b) {
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];  // (copied out element by element: see xhalf_pair)
+  a = r0;
+  b = r1;
 }
 template <class V>
 __device__ __forceinline__ void pin_loaded(V& v) {
@@ -217,7 +226,7 @@ void pairbias_kernel(const PParams p) {
   const uint64_t obase = uniform_ptr(p.o + (int64_t)head * p.os[1]);
   const uint64_t gbase = kGate ? uniform_ptr(p.gate + (int64_t)head * p.gs[1]) : 0;
   const unsigned qoff = (unsigned)(qrow * (int)p.qs[2] + 8 * h) * 2u;  // + 32 bytes per k-step
-  const unsigned ooff = (unsigned)(qrow * (int)p.os[2] + 4 * h) * 2u;  // + 16 bytes per group of 8 value columns
+  const unsigned ooff = (unsigned)(qrow * (int)p.os[2] + 8 * h) * 2u;  // + 32 bytes per group of 16 value columns
   const unsigned goff = kGate ? (unsigned)(qrow * (int)p.gs[2] + 4 * h) * 2u : 0u;
   // the row bias: every wave stages its own copy of the row (lane l brings 16 bytes; lanes past the row's end repeat
   // its start), slot (entry % 2) of the wave's two
@@ -380,7 +389,7 @@ void pairbias_kernel(const PParams p) {
   // after them: the extras of that point, and everything of the points since.  Running far ahead keeps the stores out
   // of the way: a wait completes in issue order, so a transfer issued after the stores is only known to have landed
   // once the stores are acknowledged.
-  constexpr int PT = 2 * XPW, ST = 4 * DVB;
+  constexpr int PT = 2 * XPW, ST = 2 * DVB;
   constexpr int NI = KS + (kGate ? 4 * DVB : 0) + (kRowB ? 1 : 0);
   constexpr int AHEAD = T::AHEAD;
   auto extras = [](int j) constexpr { const int t = ((j % NTI) + NTI) % NTI; return (t == 0 ? NI : 0) + (t == NTI - 1 ? ST : 0); };
@@ -484,7 +493,8 @@ void pairbias_kernel(const PParams p) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       const uint64_t ob = obase + (uint64_t)(fbc * p.os[0] * 2);
 #pragma unroll
-      for (int dvb = 0; dvb < DVB; ++dvb)
+      for (int dvb = 0; dvb < DVB; ++dvb) {
+        u32x2 quad[4];  // group g: columns 32 dvb + 8 g + 4 h .. + 4 of this lane's query
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           ex4 o4;
@@ -499,8 +509,19 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) o4[e] = (E)(oacc[dvb][4 * g + e] * inv);
           }
-          store8_counted(ob, ooff + 64u * dvb + 16u * g, __builtin_bit_cast(u32x2, o4));
+          quad[g] = __builtin_bit_cast(u32x2, o4);
         }
+        // the two lanes of a query trade halves of two groups, after which the first holds columns 16 j .. + 8 and the
+        // second the next 8: one 16-byte store each instead of two of 8 bytes, and half as many partial lines
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          uint32_t a0 = quad[2 * j][0], a1 = quad[2 * j][1], b0 = quad[2 * j + 1][0], b1 = quad[2 * j + 1][1];
+          swap_halves(a0, b0);
+          swap_halves(a1, b1);
+          const u32x4 w = {a0, a1, b0, b1};
+          store16_counted(ob, ooff + 64u * dvb + 32u * j, w);
+        }
+      }
 #pragma unroll
       for (int dvb = 0; dvb < DVB; ++dvb)
 #pragma unroll

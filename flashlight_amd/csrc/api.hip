@@ -678,6 +678,8 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
     static const int knob = std::getenv("FL_HEAD_GROUP") ? std::atoi(std::getenv("FL_HEAD_GROUP")) : 0;  // tuning knob
     kp.head_group = !growing ? 1 : (knob > 0 ? knob : 4);
   }
+  kp.o_wide = reinterpret_cast<uintptr_t>(p->o) % 16 == 0 && p->o_strides[0] % 8 == 0 && p->o_strides[1] % 8 == 0 &&
+              p->o_strides[2] % 8 == 0;
   const int grid = p->B * p->Hq * kp.n_qtiles;
 
   if (is_doc(p->mask_kind)) {

@@ -90,6 +90,7 @@ struct KParams {
   uint32_t drop_seed[2];  // low and high half of the 64-bit seed
   float drop_rescale;     // 65536 / (65536 - drop_thr), applied to the kept weights
   int32_t head_group;  // (batch, head) pairs whose query tiles are dealt together, longest first (1: head by head)
+  int32_t o_wide;      // o is 16-byte aligned with strides that are multiples of 8 elements: 16-byte stores
   int32_t n_qtiles;  // ceil(Lq / BM)
   int32_t n_ktiles;  // ceil(Lk / BN)
 };
@@ -156,6 +157,15 @@ __device__ __forceinline__ float xhalf_sum(float x) {
   float a, b;
   xhalf_pair(x, a, b);
   return a + b;
+}
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// a <-> b across the two halves of the wave: lanes 32..63 of `a` change places with lanes 0..31 of `b`
+__device__ __forceinline__ void swap_halves(uint32_t& a, uint32_t& b) {
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];  // (copied out element by element: see xhalf_pair)
+  a = r0;
+  b = r1;
 }
 
 // 16 bytes per lane from global memory straight into LDS (global_load_lds_dwordx4): lane l of the wave reads
@@ -1360,11 +1370,14 @@ void fwd_kernel(const KParams p) {
   // ---- epilogue: O^T register i of block (dvb, qb) is out[q = qrow[qb]][dv = 32*dvb + 8*(i/4) + 4h + i%4] ----------
   bf16_t* optr = p.o + (int64_t)batch * p.os[0] + (int64_t)head * p.os[1];
   const bf16_t* gptr = (kGate && p.gate) ? p.gate + (int64_t)batch * p.gs[0] + (int64_t)head * p.gs[1] : nullptr;
+  const bool wide = __builtin_amdgcn_readfirstlane(p.o_wide) != 0;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    if (qrow[qb] >= p.Lq) continue;
+    // (the wide path trades register halves between the two lanes of a query: rows past Lq go along and store nothing)
+    if (!wide && qrow[qb] >= p.Lq) continue;
 #pragma unroll
-    for (int dvb = 0; dvb < DVB; ++dvb)
+    for (int dvb = 0; dvb < DVB; ++dvb) {
+      ex4 quad[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int dv = 32 * dvb + 8 * g + 4 * h;
@@ -1372,7 +1385,7 @@ void fwd_kernel(const KParams p) {
         if (kGate && gptr) {
           ex4 g4;
           if constexpr (kGateEarly) g4 = gpre[dvb][qb][g];
-          else g4 = *reinterpret_cast<const ex4*>(gptr + (int64_t)qrow[qb] * p.gs[2] + dv);
+          else g4 = *reinterpret_cast<const ex4*>(gptr + (int64_t)min(qrow[qb], p.Lq - 1) * p.gs[2] + dv);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));
@@ -1382,8 +1395,26 @@ void fwd_kernel(const KParams p) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) o4[e] = (E)oacc[dvb][qb][4 * g + e];
         }
-        *reinterpret_cast<ex4*>(optr + (int64_t)qrow[qb] * p.os[2] + dv) = o4;
+        quad[g] = o4;
       }
+      if (wide) {
+        // the two lanes of a query trade halves of two groups of 4 columns, after which the first holds columns
+        // 16 j .. + 8 of the block and the second the next 8: 16-byte stores, half as many partial lines per store
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const u32x2 qa = __builtin_bit_cast(u32x2, quad[2 * j]), qb_ = __builtin_bit_cast(u32x2, quad[2 * j + 1]);
+          uint32_t a0 = qa[0], a1 = qa[1], b0 = qb_[0], b1 = qb_[1];
+          swap_halves(a0, b0);
+          swap_halves(a1, b1);
+          const u32x4 w = {a0, a1, b0, b1};
+          if (qrow[qb] < p.Lq) *reinterpret_cast<u32x4*>(optr + (int64_t)qrow[qb] * p.os[2] + 32 * dvb + 16 * j + 8 * h) = w;
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          *reinterpret_cast<ex4*>(optr + (int64_t)qrow[qb] * p.os[2] + 32 * dvb + 8 * g + 4 * h) = quad[g];
+      }
+    }
   }
 }
 

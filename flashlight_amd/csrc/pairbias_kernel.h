@@ -57,7 +57,6 @@ __device__ __forceinline__ u32x4 load16_counted(uint64_t sbase, unsigned voff) {
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
   return v;
 }
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ u32x2 load8_counted(uint64_t sbase, unsigned voff) {
   u32x2 v;
   asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
@@ -68,13 +67,7 @@ __device__ __forceinline__ u32x2 load8_counted(uint64_t sbase, unsigned voff) {
 __device__ __forceinline__ void store16_counted(uint64_t sbase, unsigned voff, u32x4 data) {
   asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(voff), "v"(data), "s"(sbase));
 }
-// a <-> b across the two halves of the wave: lanes 32..63 of `a` change places with lanes 0..31 of `b`
-__device__ __forceinline__ void swap_halves(uint32_t& a, uint32_t& b) {
-  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
-  const uint32_t r0 = r[0], r1 = r[1];  // (copied out element by element: see xhalf_pair)
-  a = r0;
-  b = r1;
-}
+
 template <class V>
 __device__ __forceinline__ void pin_loaded(V& v) {
   asm volatile("" : "+v"(v));

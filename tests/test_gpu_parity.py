@@ -316,6 +316,24 @@ def test_reference_free_weights_survive_extreme_logit_ranges(D, offsets):
                   O.attention_alibi(*f32(q, k, v), score_mod=2, is_causal=True, honor_causal=True, softcap=cap), "alibi+softcap+causal")
 
 
+@pytest.mark.parametrize("D,mask", [(128, "none"), (64, "causal"), (32, "none")])
+def test_results_written_to_an_8_byte_aligned_view_match_the_16_byte_path(D, mask):
+    # a result tensor that is 16-byte aligned with strides that are multiples of 8 elements is written in 16-byte stores
+    # (the two lanes of a query trade register halves first); any other placement the ABI admits (8-byte alignment,
+    # strides that are multiples of 4) takes 8-byte stores.  Both give the same bits.  S = 333: rows past the end.
+    B, H, S = 2, 3, 333
+    q, k, v = qkv(B, H, H, S, D, seed=44)
+    kind = _ffi.MASK_CAUSAL if mask == "causal" else _ffi.MASK_NONE
+    wide = _ffi.attn_fwd(q, k, v, mask_kind=kind)
+    big = torch.full((B, H, S, D + 12), 7.0, dtype=q.dtype, device=DEV)
+    view = big[..., 4:4 + D]
+    assert view.data_ptr() % 16 == 8 and view.stride(2) % 8 == 4
+    out = _ffi.attn_fwd(q, k, v, mask_kind=kind, out=view)
+    assert out.data_ptr() == view.data_ptr()
+    assert torch.equal(view, wide)
+    assert torch.all(big[..., :4] == 7.0) and torch.all(big[..., 4 + D:] == 7.0)  # nothing written beside the view
+
+
 # ---- dense score_mod and invariant point attention -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("gqa", [False, True])

@@ -450,9 +450,11 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   if (p->Lk % 32 != 0 || !fl::pairbias_has_shape(p->Dqk, p->Lk / 32, p->gate != nullptr, ri >= 0)) return false;
   if (reinterpret_cast<uintptr_t>(p->bias[pi]) % 16 != 0 || bst[0] % 8 || bst[1] % 8 || bst[2] % 8) return false;
   if (ri >= 0 && (reinterpret_cast<uintptr_t>(p->bias[ri]) % 16 != 0 || p->bias_strides[ri][0] % 8)) return false;
-  // (results leave in 16-byte stores, gate logits arrive in 8-byte loads)
+  // (results leave in 16-byte stores, gate logits arrive in 16-byte loads)
   if (reinterpret_cast<uintptr_t>(p->o) % 16 != 0 || p->o_strides[0] % 8 || p->o_strides[1] % 8 || p->o_strides[2] % 8) return false;
-  if (p->gate && reinterpret_cast<uintptr_t>(p->gate) % 8 != 0) return false;
+  if (p->gate && (reinterpret_cast<uintptr_t>(p->gate) % 16 != 0 || p->gate_strides[0] % 8 || p->gate_strides[1] % 8 ||
+                  p->gate_strides[2] % 8))
+    return false;
   // per-lane byte offsets inside one (batch entry, head) slice are 32-bit
   const int64_t worst = std::max(std::max(p->q_strides[2], p->o_strides[2]), p->gate ? p->gate_strides[2] : 0);
   if (((int64_t)p->Lq * worst + 64) * 2 >= ((int64_t)1 << 31)) return false;

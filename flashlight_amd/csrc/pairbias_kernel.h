@@ -48,18 +48,13 @@ struct PParams {
   int64_t rbs;         // its element stride between batch entries
 };
 
-// 16 / 8 bytes per lane from global memory into registers, and 8 bytes back, as asm: inside the streaming loop every
+// 16 bytes per lane from global memory into registers, and 16 bytes back, as asm: inside the streaming loop every
 // vector-memory operation is issued by hand in a fixed order, because the waits there count operations
 // (s_waitcnt vmcnt(N): at most N still outstanding, completion in issue order) and a compiler-issued access would not
 // be in the count.  The loaded registers may be read only after the wait that covers them and a pin_loaded() on them.
 __device__ __forceinline__ u32x4 load16_counted(uint64_t sbase, unsigned voff) {
   u32x4 v;
   asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
-  return v;
-}
-__device__ __forceinline__ u32x2 load8_counted(uint64_t sbase, unsigned voff) {
-  u32x2 v;
-  asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase));
   return v;
 }
 // (a store of more than 8 bytes still reads its data registers for two cycles after it has issued, and the compiler,
@@ -220,7 +215,7 @@ void pairbias_kernel(const PParams p) {
   const uint64_t gbase = kGate ? uniform_ptr(p.gate + (int64_t)head * p.gs[1]) : 0;
   const unsigned qoff = (unsigned)(qrow * (int)p.qs[2] + 8 * h) * 2u;  // + 32 bytes per k-step
   const unsigned ooff = (unsigned)(qrow * (int)p.os[2] + 8 * h) * 2u;  // + 32 bytes per group of 16 value columns
-  const unsigned goff = kGate ? (unsigned)(qrow * (int)p.gs[2] + 4 * h) * 2u : 0u;
+  const unsigned goff = kGate ? (unsigned)(qrow * (int)p.gs[2] + 8 * h) * 2u : 0u;  // 16-byte loads, see the epilogue
   // the row bias: every wave stages its own copy of the row (lane l brings 16 bytes; lanes past the row's end repeat
   // its start), slot (entry % 2) of the wave's two
   const uint64_t rbase = kRowB ? uniform_ptr(p.rowb) : 0;
@@ -383,7 +378,7 @@ void pairbias_kernel(const PParams p) {
   // of the way: a wait completes in issue order, so a transfer issued after the stores is only known to have landed
   // once the stores are acknowledged.
   constexpr int PT = 2 * XPW, ST = 2 * DVB;
-  constexpr int NI = KS + (kGate ? 4 * DVB : 0) + (kRowB ? 1 : 0);
+  constexpr int NI = KS + (kGate ? 2 * DVB : 0) + (kRowB ? 1 : 0);
   constexpr int AHEAD = T::AHEAD;
   auto extras = [](int j) constexpr { const int t = ((j % NTI) + NTI) % NTI; return (t == 0 ? NI : 0) + (t == NTI - 1 ? ST : 0); };
   auto allowed = [extras](int t) constexpr {
@@ -394,7 +389,7 @@ void pairbias_kernel(const PParams p) {
   for (int item = 0; item < n_items; ++item) {
     const int slot0 = (item * NTI) % NS;
     u32x4 qn[KS];            // next entry's query fragments, in flight from tile 0 on
-    u32x2 gl[4 * DVB];       // this entry's gate logits, likewise
+    u32x4 gl[2 * DVB];       // this entry's gate logits, likewise (8 consecutive columns per load)
     const int64_t fbn = fb0 + min(item + 1, n_items - 1);
     const int64_t fbc = fb0 + item;
     ex8 qnext[KS];
@@ -419,7 +414,7 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
               for (int dvb = 0; dvb < DVB; ++dvb)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) gl[4 * dvb + g] = load8_counted(gb, goff + 64u * dvb + 16u * g);
+                for (int j = 0; j < 2; ++j) gl[2 * dvb + j] = load16_counted(gb, goff + 64u * dvb + 32u * j);
             }
             const uint64_t qb = qbase + (uint64_t)(fbn * p.qs[0] * 2);
 #pragma unroll
@@ -436,7 +431,7 @@ void pairbias_kernel(const PParams p) {
             }
             if constexpr (kGate) {
 #pragma unroll
-              for (int g = 0; g < 4 * DVB; ++g) pin_loaded(gl[g]);
+              for (int g = 0; g < 2 * DVB; ++g) pin_loaded(gl[g]);
             }
           }
         }
@@ -488,11 +483,22 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
       for (int dvb = 0; dvb < DVB; ++dvb) {
         u32x2 quad[4];  // group g: columns 32 dvb + 8 g + 4 h .. + 4 of this lane's query
+        u32x2 gq[4];    // their gate logits: loaded as 8 consecutive columns per lane, the trade below in reverse
+        if constexpr (kGate) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            uint32_t a0 = gl[2 * dvb + j][0], a1 = gl[2 * dvb + j][1], b0 = gl[2 * dvb + j][2], b1 = gl[2 * dvb + j][3];
+            swap_halves(a0, b0);
+            swap_halves(a1, b1);
+            gq[2 * j] = u32x2{a0, a1};
+            gq[2 * j + 1] = u32x2{b0, b1};
+          }
+        }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           ex4 o4;
           if constexpr (kGate) {
-            const ex4 g4 = __builtin_bit_cast(ex4, gl[4 * dvb + g]);
+            const ex4 g4 = __builtin_bit_cast(ex4, gq[g]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const float sg = fast_rcp(1.0f + fast_exp2(-kLog2e * (float)g4[e]));

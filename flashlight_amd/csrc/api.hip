@@ -747,10 +747,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     return fail(FL_ERR_SHAPE, "backward: too many workgroups");
   uint32_t want = 0;
   if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
-  if (is_doc(p->mask_kind)) {
-    if (want) return fail(FL_ERR_UNSUPPORTED, "backward: document masks cannot be combined with ALiBi or a soft-cap");
-    want = fl::F_DOC;
-  }
+  if (is_doc(p->mask_kind)) want |= fl::F_DOC;
   if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() has excluded document masks
   if (has_bias) want = fl::F_BIAS;
   const fl::BwdInstance* in = nullptr;

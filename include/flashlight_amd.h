@@ -172,7 +172,8 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * softmax attention, recomputing the weights from the forward's row statistics.
  * `fwd` describes the forward call whose gradients are wanted: same q, k, v, sizes, scale, mask and score
  * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
- * kind, grouped-query heads, ALiBi, the tanh soft-cap; Dqk == Dv in {32, 64, 128}.  Bias operands (fwd.bias, as in the
+ * kind, grouped-query heads, ALiBi, the tanh soft-cap (either of them under a document mask at head dims 64 and 128);
+ * Dqk == Dv in {32, 64, 128}.  Bias operands (fwd.bias, as in the
  * forward) go with positional masks only, not with ALiBi, a soft-cap, a document mask or dropout.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
  * (both are compositions of calls that are supported: out * sigmoid(gate); one call per branch and half of the value
  * columns), the attended_dump hook.

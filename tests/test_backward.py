@@ -214,6 +214,31 @@ def test_gradients_document_mask(D, causal):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("cap", [None, 12.0])
+@pytest.mark.parametrize("D", [64, 128])
+def test_gradients_document_mask_with_alibi_and_softcap(D, cap):
+    """Document ids in the element predicate together with the in-kernel ALiBi term and / or the soft-cap: the oracle is
+    autograd through the eager fp32 composition cap * tanh(q k^T s / cap) + slope_h (k - q), masked where ids differ."""
+    import math
+    from flashlight_amd import _ffi, ops
+    from oracle.attention import _softmax_attention, alibi_slopes
+    B, H, S = 2, 4, 600
+    q, k, v, dout = _inputs(B, H, H, S, D, seed=123 + D)
+    g = torch.Generator().manual_seed(17)
+    ids = torch.sort(torch.randint(0, 6, (B, S), generator=g), dim=1).values.to(DEV)
+    slopes = alibi_slopes(H).float().view(1, H, 1, 1).to(DEV)
+    for causal in (False, True):
+        def masked(qi, ki):
+            m = ids[:, qi.view(-1)].view(B, 1, -1, 1) != ids[:, ki.view(-1)].view(B, 1, 1, -1)
+            return (m | (ki > qi)) if causal else m
+        _check(f"document + alibi + cap={cap} causal={causal} D={D}",
+               lambda q, k, v: ops.dispatch(q, k, v, mask_kind=_ffi.MASK_DOCUMENT_CAUSAL if causal else _ffi.MASK_DOCUMENT,
+                                            doc_ids=ids, alibi_heads=H, softcap=cap or 0.0),
+               lambda q, k, v: _softmax_attention(q, k, v, 1.0 / math.sqrt(D), masked=masked, softcap=cap,
+                                                  bias=lambda qi, ki: slopes * (ki - qi).float()), q, k, v, dout)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("D", [64, 128])
 def test_gradients_document_mask_many_dead_tiles(D):
     """Several documents over many tiles: most (owner block, streamed tile) pairs are dead, and the backward hops from

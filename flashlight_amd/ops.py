@@ -15,7 +15,7 @@ import torch
 
 from . import _ffi
 
-__all__ = ["attn_fwd", "attn_fwd_lse", "attn_bwd", "dispatch"]
+__all__ = ["attn_fwd", "attn_fwd_lse", "attn_bwd", "attn_fwd_bias_lse", "attn_bwd_bias", "dispatch"]
 
 
 def _out_shape(q: torch.Tensor, v: torch.Tensor, diff: bool):
@@ -114,44 +114,82 @@ def _backward(ctx, dout, dlse):
 attn_fwd_lse.register_autograd(_backward, setup_context=_setup_context)
 
 
-class _BiasAttention(torch.autograd.Function):
+@torch.library.custom_op("flashlight_amd::attn_fwd_bias_lse", mutates_args=())
+def attn_fwd_bias_lse(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, mask_kind: int, window: int,
+                      prefix: int, bias0: Optional[torch.Tensor], bias0_div: int, bias1: Optional[torch.Tensor],
+                      bias1_div: int) -> tuple[torch.Tensor, torch.Tensor]:
     """The forward with bias operands for calls that will be differentiated (the reference's Evoformer function and its
     dense `score_mod` tensors, attention_variants/evoformer.py:24-27, alibi.py:26-30; the reference itself has no
-    backward).  The backward kernels return, next to dq, dk, dv, the gradient with respect to the scores; the gradient of
-    a bias operand is that array summed over the batch entries and axes the operand broadcasts over."""
+    backward): result and row statistics, like `attn_fwd_lse`.  An operator of its own, so that `torch.compile` traces
+    the differentiable call and its backward like any other node."""
+    out = _alloc_out(q, v, False, False)
+    lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
+    biases = [(b, d) for b, d in ((bias0, bias0_div), (bias1, bias1_div)) if b is not None]
+    _ffi.attn_fwd(q, k, v, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window, prefix=prefix,
+                  biases=biases, out=out, lse=lse)
+    return out, lse
 
-    @staticmethod
-    def forward(ctx, q, k, v, scale, mask_kind, window, prefix, div0, div1, bias0, bias1):
-        out = _alloc_out(q, v, False, False)
-        lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
-        biases = [(b, d) for b, d in ((bias0, div0), (bias1, div1)) if b is not None]
-        _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, biases=biases, out=out, lse=lse)
-        ctx.save_for_backward(q, k, v, out, lse, bias0, bias1)
-        ctx.args = (scale, mask_kind, window, prefix, div0, div1)
-        return out
 
-    @staticmethod
-    def backward(ctx, dout):
-        q, k, v, out, lse, bias0, bias1 = ctx.saved_tensors
-        scale, mask_kind, window, prefix, div0, div1 = ctx.args
-        biases = [(b, d) for b, d in ((bias0, div0), (bias1, div1)) if b is not None]
-        want = [b is not None and ctx.needs_input_grad[9 + i] for i, b in enumerate((bias0, bias1))]
-        dscores = None
-        if any(want):
-            dscores = torch.zeros((q.size(0), q.size(1), q.size(2), k.size(2)), dtype=torch.float32, device=q.device)
-        dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout.to(q.dtype), scale=scale, mask_kind=mask_kind, window=window,
-                                   prefix=prefix, biases=biases, dscores=dscores)
-        dbs = []
-        for b, d, w in ((bias0, div0, want[0]), (bias1, div1, want[1])):
-            if not w:
-                dbs.append(None)
-                continue
-            g = dscores.view(dscores.size(0) // d, d, *dscores.shape[1:]).sum(1)
-            axes = [i for i in range(4) if b.size(i) == 1 and g.size(i) != 1]
-            if axes:
-                g = g.sum(axes, keepdim=True)
-            dbs.append(g.to(b.dtype))
-        return dq, dk, dv, None, None, None, None, None, None, dbs[0], dbs[1]
+@attn_fwd_bias_lse.register_fake
+def _attn_fwd_bias_lse_fake(q, k, v, scale, mask_kind, window, prefix, bias0, bias0_div, bias1, bias1_div):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("query, key and value must be 4-D [batch, heads, seq, dim]")
+    return _alloc_out(q, v, False, False), torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
+
+
+@torch.library.custom_op("flashlight_amd::attn_bwd_bias", mutates_args=())
+def attn_bwd_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
+                  dout: torch.Tensor, scale: float, mask_kind: int, window: int, prefix: int,
+                  bias0: Optional[torch.Tensor], bias0_div: int, bias1: Optional[torch.Tensor], bias1_div: int,
+                  want_dscores: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dq, dk, dv, dscores) of `attn_fwd_bias_lse`: dscores, float32 [B, Hq, Lq, Lk], is the gradient with respect to
+    whatever was added to q k^T scale (empty when `want_dscores` is false: no bias operand asks for a gradient)."""
+    biases = [(b, d) for b, d in ((bias0, bias0_div), (bias1, bias1_div)) if b is not None]
+    shape = (q.size(0), q.size(1), q.size(2), k.size(2)) if want_dscores else (0,)
+    dscores = torch.zeros(shape, dtype=torch.float32, device=q.device)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, scale=scale if scale > 0 else None, mask_kind=mask_kind,
+                               window=window, prefix=prefix, biases=biases, dscores=dscores if want_dscores else None)
+    return dq, dk, dv, dscores
+
+
+@attn_bwd_bias.register_fake
+def _attn_bwd_bias_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefix, bias0, bias0_div, bias1, bias1_div,
+                        want_dscores):
+    c = torch.contiguous_format
+    shape = (q.size(0), q.size(1), q.size(2), k.size(2)) if want_dscores else (0,)
+    return (torch.empty_like(q, memory_format=c), torch.empty_like(k, memory_format=c), torch.empty_like(v, memory_format=c),
+            torch.empty(shape, dtype=torch.float32, device=q.device))
+
+
+def _bias_setup_context(ctx, inputs, output):
+    q, k, v, scale, mask_kind, window, prefix, bias0, div0, bias1, div1 = inputs
+    out, lse = output
+    ctx.save_for_backward(q, k, v, out, lse, bias0, bias1)
+    ctx.args = (scale, mask_kind, window, prefix, div0, div1)
+
+
+def _bias_backward(ctx, dout, dlse):
+    """The gradient of a bias operand is the score gradient summed over the batch entries and axes the operand
+    broadcasts over."""
+    q, k, v, out, lse, bias0, bias1 = ctx.saved_tensors
+    scale, mask_kind, window, prefix, div0, div1 = ctx.args
+    want = [b is not None and ctx.needs_input_grad[7 + 2 * i] for i, b in enumerate((bias0, bias1))]
+    dq, dk, dv, dscores = attn_bwd_bias(q, k, v, out, lse, dout.to(q.dtype), scale, mask_kind, window, prefix, bias0, div0,
+                                        bias1, div1, any(want))
+    dbs = []
+    for b, d, w in ((bias0, div0, want[0]), (bias1, div1, want[1])):
+        if not w:
+            dbs.append(None)
+            continue
+        g = dscores.view(dscores.size(0) // d, d, *dscores.shape[1:]).sum(1)
+        axes = [i for i in range(4) if b.size(i) == 1 and g.size(i) != 1]
+        if axes:
+            g = g.sum(axes, keepdim=True)
+        dbs.append(g.to(b.dtype))
+    return dq, dk, dv, None, None, None, None, dbs[0], None, dbs[1], None
+
+
+attn_fwd_bias_lse.register_autograd(_bias_backward, setup_context=_bias_setup_context)
 
 
 def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases, gate, diff,
@@ -177,8 +215,8 @@ def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi
             raise NotImplementedError("gradients with bias operands are built for positional masks without ALiBi, soft-cap, "
                                       "document ids or dropout")
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
-        out = _BiasAttention.apply(q, k, v, None if scale is None else float(scale), int(mask_kind), int(window), int(prefix),
-                                   int(bl[0][1]), int(bl[1][1]), bl[0][0], bl[1][0])
+        out, _ = attn_fwd_bias_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
+                                   int(prefix), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]))
     else:
         out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
                               int(prefix), doc_ids, int(alibi_heads), float(softcap), dropout_p, int(dropout_seed))
@@ -258,9 +296,6 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     wants_grad = torch.is_grad_enabled() and any(
         t is not None and t.requires_grad for t in (q, k, v, gate, *(b for b, _ in biases)))
     if wants_grad or (dropout_p > 0.0 and torch.compiler.is_compiling()):
-        if torch.compiler.is_compiling() and (biases or gate is not None or diff):
-            raise NotImplementedError("gradients with bias operands, the gate or differential attention are not traceable "
-                                      "by torch.compile: differentiate the eager call")
         # (the result comes back in [B, H, L, Dv] memory order whatever seq_major_out asks for)
         return _differentiable(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                                alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,

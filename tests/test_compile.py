@@ -116,3 +116,35 @@ def test_compiled_equals_eager_on_gpu():
     assert got.shape == want.shape and torch.equal(got, want)
     torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd.default,
                           (q, k, v, -1.0, 1, 0, 0, None, 0, 0.0, None, 1, None, 1, None, False, 0.0, False))
+
+
+@pytest.mark.gpu
+def test_compiled_gradients_with_bias_gate_and_differential_attention():
+    """Gradients through `torch.compile` (aot_eager: forward and backward graphs are traced, the fused calls stay opaque
+    operators) for the calls whose backward is a composition: Evoformer attention with two bias operands and the
+    gate, and differential attention.  Each must give what differentiating the eager call gives."""
+    dev = "cuda"
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s: torch.randn(*s, generator=g).to(BF).to(dev)  # noqa: E731
+
+    def grads(fn, args):
+        leaves = [a.detach().clone().requires_grad_(True) for a in args]
+        out = fn(*leaves)
+        out.float().square().sum().backward()
+        return [out.detach()] + [leaf.grad for leaf in leaves]
+
+    Q, K, V, G = (mk(1, 3, 104, 2, 32) for _ in range(4))
+    pair, mask = mk(1, 1, 2, 104, 104), mk(1, 3, 1, 1, 104)
+    evo = lambda Q, K, V, m, p, G: A.attention_reference(Q, K, V, [m, p], gate=G)  # noqa: E731
+    q, k, v = mk(2, 8, 200, 64), mk(2, 8, 200, 64), mk(2, 4, 200, 128)
+    diff = lambda q, k, v: A.diffattn(q, k, v, lambda_full=0.3, is_causal=True)  # noqa: E731
+    for name, fn, args in (("evoformer", evo, (Q, K, V, mask, pair, G)), ("diffattn", diff, (q, k, v))):
+        torch._dynamo.reset()
+        want = grads(fn, args)
+        got = grads(torch.compile(fn, backend="aot_eager", fullgraph=True), args)
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert a.shape == b.shape, f"{name}: output {i}"
+            scale = max(1.0, b.float().abs().max().item())
+            assert (a.float() - b.float()).abs().max().item() <= 2e-2 * scale, f"{name}: output {i}"
+    torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd_bias_lse.default,
+                          (mk(2, 2, 64, 32), mk(2, 2, 64, 32), mk(2, 2, 64, 32), -1.0, 0, 0, 0, mk(1, 2, 64, 64), 2, None, 1))

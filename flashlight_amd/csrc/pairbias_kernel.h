@@ -13,9 +13,10 @@
 //   * the bias of the workgroup's queries against ALL keys stays in registers for the whole chunk, already laid out as
 //     MFMA B operands (8 consecutive keys of one query per lane and 16-key group);
 //   * the matrix pipe, which idles at head dim 32, adds it: S^T += Sel . Bias^T with Sel the 32 x 16 selector that puts
-//     key 16m + j on row j of the group, weighted 1/scale (split in two bf16 terms, relative error 2^-17), so the
-//     accumulators hold qk + bias/scale and the weights are exp2(scale * log2(e) * acc - ref): per score one
-//     multiply-add, one exponential, one addition for the row sum and half a pack.
+//     key 16m + j on row j of the group, weighted 1/scale (in fp16 unless the element type holds it exactly: relative
+//     error of the bias term at most 2^-12), so the accumulators hold qk + bias/scale and the weights are
+//     exp2(scale * log2(e) * acc - ref): per score one multiply-add, one exponential, one addition for the row sum and
+//     half a pack.
 //   * the row bias takes the same road as a rank-one product: A = the row's values down the keys (two copies side by
 //     side), B = the two terms of 1/scale across the queries; the row of the next entry rides into LDS with the
 //     transfers of the current one.
@@ -74,7 +75,7 @@ struct PairBiasTraits {
   static constexpr int NKB = NKB_;       // 32-key blocks per row: Lk = 32 * NKB
   static constexpr bool GATE = GATE_;
   static constexpr bool ROWB = ROWB_;    // a row bias per batch entry besides the shared one
-  // 1 / scale is exact in the element type (a power of two, say): its second term is zero and the products with it go
+  // 1 / scale is exact in the element type (a power of two, say): the selector product runs in that type as it is
   static constexpr bool EXACT = EXACT_;
   static constexpr int D = D_, BN = 64, NW = 4, NT = 256, BM = 128;
   static constexpr int KS = D / 16;      // k-steps of the first product
@@ -112,7 +113,6 @@ void pairbias_kernel(const PParams p) {
   typedef E ex2 __attribute__((ext_vector_type(2)));
   constexpr int NKB = T::NKB, NTI = T::NTI, NS = T::NS, D = T::D, BN = T::BN, KS = T::KS, DVB = T::DVB, XPW = T::XPW;
   constexpr bool kGate = T::GATE, kRowB = T::ROWB, kAheadK = T::KAHEAD;
-  constexpr int kParts = T::EXACT ? 1 : 2;  // terms of 1 / scale
   constexpr float kLog2e = 1.4426950408889634f;
   using LK = TileLayout<D>;
   using LV = TileLayout<D>;
@@ -143,8 +143,15 @@ void pairbias_kernel(const PParams p) {
   }
   const int qrow = min(qt * T::BM + wave * 32 + r, p.Lq - 1);  // rows past Lq repeat the last row (same values stored)
 
-  // ---- the resident bias: B operands of the selector products, lane (r, h) holds bias[qrow][32 kb + 16 m + 8 h .. + 8]
-  ex8 bfrag[NKB][2];
+  // ---- the resident bias: B operands of the selector products, lane (r, h) holds bias[qrow][32 kb + 16 m + 8 h .. + 8].
+  // The selector product has one term, 1 / scale times the bias, and runs in the type that holds 1 / scale best: the
+  // element type when the value is exact in it (EXACT), fp16 otherwise (11 bits: the bias enters the logits with a
+  // relative error of at most 2^-12; bf16's 8 bits would need a second product for the remainder).  bf16 bias values
+  // are fp16 values as they stand up to 65504; larger ones (masks like -1e9) saturate there, which times 1 / scale is
+  // still tens of thousands below any score.
+  using SE = std::conditional_t<T::EXACT, E, f16_t>;
+  typedef SE sx8 __attribute__((ext_vector_type(8)));
+  sx8 bfrag[NKB][2];
   {
     const bf16_t* brow = p.bias + (int64_t)grp * p.bs[0] + (int64_t)head * p.bs[1] + (int64_t)qrow * p.bs[2];
 #pragma unroll
@@ -162,23 +169,25 @@ void pairbias_kernel(const PParams p) {
           const uint32_t hi_inf = (((x >> 16) & 0x7FFFu) == kInf) ? 0x10000u : 0u;
           raw[w] = x - lo_inf - hi_inf;
         }
-        bfrag[kb][m] = __builtin_bit_cast(ex8, raw);
+        if constexpr (!std::is_same<SE, E>::value) {
+          // bf16 pair -> fp16 pair (rounding toward zero: exact in range, the largest finite value beyond it)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            const float lo = __builtin_bit_cast(float, raw[w] << 16), hi = __builtin_bit_cast(float, raw[w] & 0xFFFF0000u);
+            raw[w] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+          }
+        }
+        bfrag[kb][m] = __builtin_bit_cast(sx8, raw);
       }
   }
   // selectors: A operand of group m puts key 16 m + j on row j; lane (r, h) holds Sel[key = r][j = 8 h .. 8 h + 7]
-  ex8 sel[2][2];
+  sx8 sel[2];
   {
-    const float w = 1.0f / p.scale;
-    const E w_hi = (E)w;
-    const E w_lo = (E)(w - (float)w_hi);
+    const SE w = (SE)(1.0f / p.scale);
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const bool on = r == 16 * m + 8 * h + j;
-        sel[m][0][j] = on ? w_hi : (E)0.0f;
-        sel[m][1][j] = on ? w_lo : (E)0.0f;
-      }
+      for (int j = 0; j < 8; ++j) sel[m][j] = (r == 16 * m + 8 * h + j) ? w : (SE)0.0f;
   }
   // row bias: B operand of the rank-one product, lane (query r, h) holds rows 8 h .. 8 h + 7 of the 16: rows 0 and 1
   // carry the two terms of 1 / scale, the A operand has the row's value in columns 0 and 1
@@ -265,9 +274,7 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) s = mfma32(kf[ks], qf[ks], s);
 #pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int part = 0; part < kParts; ++part) s = mfma32(sel[m][part], bfrag[kb][m], s);
+    for (int m = 0; m < 2; ++m) s = mfma32(sel[m], bfrag[kb][m], s);
     if constexpr (kRowB) s = mfma32(rowf, rsel, s);
   };
   // A operand of O^T += V^T . P^T for 16-key chunk c of the tile (the transposing LDS read of the general kernel)
@@ -458,7 +465,7 @@ void pairbias_kernel(const PParams p) {
         ex8 pf[2];
         weights(cur, pf);
         // the LDS reads first, then the score MFMAs spread over the exponentials (64 vector instructions per block)
-        constexpr int kReads = KS + 4 * DVB + (kRowB ? 1 : 0), kScoreMfmas = KS + 2 * kParts + (kRowB ? 1 : 0);
+        constexpr int kReads = KS + 4 * DVB + (kRowB ? 1 : 0), kScoreMfmas = KS + 2 + (kRowB ? 1 : 0);
         __builtin_amdgcn_sched_group_barrier(SG_DS_READ, kReads, 0);
         // (without KAHEAD the first MFMA waits for the K fragments just asked for: some exponentials go first)
         if constexpr (!kAheadK) __builtin_amdgcn_sched_group_barrier(SG_VALU | SG_TRANS, 8, 0);

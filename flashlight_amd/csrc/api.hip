@@ -243,6 +243,13 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
   const int64_t visited = p->mask_kind == FL_MASK_SLIDING ? std::min<int64_t>(p->Lk, (int64_t)p->window + 128) : p->Lk;
   // (measured: from a window of 256 on the 4-wave tile ties or wins on warm operands and wins by 4 % on cold ones)
   const bool short_loop = p->mask_kind == FL_MASK_SLIDING && visited < 384;
+  // Unmasked calls at head dim 128 whose grid still fills the part twice over with 256-row workgroups take the
+  // 8-wave tile: one workgroup per compute unit brings every K/V tile in once for 256 rows instead of twice, which on
+  // ordinary data is worth more than the second workgroup's independence (2.4 % on N(0,1) operands; at head dim 64,
+  // under masks and on all-zero operands it is not).
+  const bool wide_group = p->mask_kind == FL_MASK_NONE && want == 0 && p->Dqk == 128 && p->Dv == 128 &&
+                          (int64_t)p->B * p->Hq * ((p->Lq + 255) / 256) >= 512;
+  const int preferred_nw = short_loop ? 2 : (wide_group ? 8 : 4);
   for (int i = 0; i < fl::kNumInstances; ++i) {
     const fl::Instance& in = fl::kInstances[i];
     if (in.dqk != p->Dqk || in.dv != p->Dv || in.dtype != p->dtype) continue;
@@ -250,9 +257,8 @@ const fl::Instance* select_instance(const fl_attn_params* p) {
     const uint32_t extra = in.feat & ~want;
     if (extra & ~kOptionalFeatures) continue;
     if (want_rw && (in.rw != want_rw || in.bn != want_bn || in.nw != want_nw || (want_ns && in.ns != want_ns))) continue;
-    // fewer unused features first; among equals the listed order, except that a short key loop prefers the small
-    // workgroup
-    const int n = 2 * __builtin_popcount(extra) + ((in.nw == 2) == short_loop ? 0 : 1);
+    // fewer unused features first; among equals the preferred workgroup size, then the listed order
+    const int n = 2 * __builtin_popcount(extra) + (in.nw == preferred_nw ? 0 : 1);
     if (n < best_extra) {
       best = &in;
       best_extra = n;

@@ -82,6 +82,22 @@ def test_plan_reports_launch_shape(lib):
     assert plan["workgroups"] == 2 * 4 * ((300 + bm - 1) // bm)
 
 
+def test_large_unmasked_calls_at_head_dim_128_take_256_row_workgroups(lib):
+    # one 8-wave workgroup per compute unit brings each K/V tile in once for 256 query rows; chosen only without a mask
+    # or score modification, at head dim 128, and when such workgroups still fill the part twice over
+    big = good_params(B=4, Hq=16, Hkv=16, L=4096, D=128)
+    assert _ffi.plan(big)["rows_per_workgroup"] == 256 and _ffi.plan(big)["threads"] == 512
+    assert _ffi.plan(big)["workgroups"] == 4 * 16 * 16
+    for change in (dict(L=1024), dict(D=64), dict(B=1, Hq=8, Hkv=8)):
+        assert _ffi.plan(good_params(**{**dict(B=4, Hq=16, Hkv=16, L=4096, D=128), **change}))["rows_per_workgroup"] == 128
+    masked = good_params(B=4, Hq=16, Hkv=16, L=4096, D=128)
+    masked.mask_kind = _ffi.MASK_CAUSAL
+    assert _ffi.plan(masked)["rows_per_workgroup"] == 128
+    capped = good_params(B=4, Hq=16, Hkv=16, L=4096, D=128)
+    capped.softcap = 30.0
+    assert _ffi.plan(capped)["rows_per_workgroup"] == 128
+
+
 @pytest.mark.parametrize("mutate, code, word", [
     (lambda p: setattr(p, "q", 0), -1, "q pointer is null"),
     (lambda p: setattr(p, "o", None), -1, "o pointer"),

@@ -316,6 +316,22 @@ def test_reference_free_weights_survive_extreme_logit_ranges(D, offsets):
                   O.attention_alibi(*f32(q, k, v), score_mod=2, is_causal=True, honor_causal=True, softcap=cap), "alibi+softcap+causal")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_256_row_workgroups_ragged_and_cross_lengths(dtype):
+    # enough (batch, head) pairs that the unmasked head-dim-128 call takes the 8-wave tile; 300 query rows leave the
+    # second workgroup of every head 44 rows (six of its eight waves have none), 333 keys a ragged last tile; GQA 4:1
+    B, Hq, Hkv, Lq, Lk, D = 4, 64, 16, 300, 333, 128
+    g = torch.Generator().manual_seed(52)
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(dtype).to(DEV)
+    k = torch.randn(B, Hkv, Lk, D, generator=g).to(dtype).to(DEV)
+    v = torch.randn(B, Hkv, Lk, D, generator=g).to(dtype).to(DEV)
+    p, _keep = _ffi._fill_params(_ffi.load_library(), q, k, v, torch.empty_like(q), Hq, Hkv, None, _ffi.MASK_NONE, 0, 0, None,
+                                 0, 0.0, [], None, False, 0.0, None)
+    assert _ffi.plan(p)["rows_per_workgroup"] == 256
+    out = A.attention_pytorch(q, k, v, enable_gqa=True)
+    assert_parity(out, O.attention_vanilla(*f32(q, k, v), enable_gqa=True), f"8-wave tile {dtype}")
+
+
 @pytest.mark.parametrize("D,mask", [(128, "none"), (64, "causal"), (32, "none")])
 def test_results_written_to_an_8_byte_aligned_view_match_the_16_byte_path(D, mask):
     # a result tensor that is 16-byte aligned with strides that are multiples of 8 elements is written in 16-byte stores

@@ -326,11 +326,14 @@ def main():
         del tens, zeros, ops
         # The forward's step as a register-only probe (zero operands): nominal-clock cycles per 32 x 32 block of scores
         # and SIMD for the MFMAs alone, for the step as the forward has it (softmax vector work, data dependences), and
-        # with the K / V fragments read from LDS; last, the forward itself on zero inputs.
+        # with the K / V fragments read from LDS; last, the forward itself on zero inputs.  The three-stage order of the
+        # step (second product on the previous block's weights, both MFMA groups under the vector work) is the rung
+        # the forward was built and measured on and does not use: its gain shows on zero operands only.
         sink2 = torch.empty(2 * n_cu * 256, dtype=torch.float32, device=dev)
         ladder = {}
         for D in (64, 128):
-            for level, tag in ((0, "mfma_only"), (2, "step_in_registers"), (3, "plus_lds_operand_reads")):
+            for level, tag in ((0, "mfma_only"), (2, "step_in_registers"), (4, "three_stage_step_in_registers"),
+                               (3, "plus_lds_operand_reads")):
                 blocks = [0]
 
                 def run(D=D, level=level):

@@ -53,7 +53,9 @@ enum : int { PSG_VALU = 0x2, PSG_MFMA = 0x8, PSG_TRANS = 0x400 };
 // dot products on S(current), D / 16 MFMAs O += V . P from the packed weights.  No global memory, no transfers, no
 // barriers, no masks.  LEVEL 0: the MFMAs alone; 1: MFMAs and vector work without dependences between them (the
 // vector work runs on constants); 2: the step as the forward has it, operands in registers; 3: the same with the K
-// and V fragments read from LDS like the forward's (ds_read_b128, transposing ds_read_b64).
+// and V fragments read from LDS like the forward's (ds_read_b128, transposing ds_read_b64); 4: level 2 in a
+// three-stage order: the second product takes the PREVIOUS block's weights, so that both groups of MFMAs are issued
+// under this block's vector work (a rung the forward was built and measured on, and does not use).
 template <int D, int LEVEL>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) step_probe_kernel(float* out, int iters, float c2, float seed) {
   constexpr int KS = D / 16, DVB = D / 32, CPR = D / 8;
@@ -129,10 +131,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   bf16x8 pconst[2];
   for (int c = 0; c < 2; ++c)
     for (int e = 0; e < 8; ++e) pconst[c][e] = (__bf16)seed;
-  auto step = [&](f32x16& sc, f32x16& sn) __attribute__((always_inline)) {
+  bf16x8 pa[2], pb[2];  // level 4: the weights of one block live until the next block's second product
+  for (int c = 0; c < 2; ++c)
+    for (int e = 0; e < 8; ++e) pa[c][e] = pb[c][e] = (__bf16)seed;
+  auto step = [&](f32x16& sc, f32x16& sn, bf16x8 (&pnew)[2], const bf16x8 (&pold)[2]) __attribute__((always_inline)) {
     bf16x8 pf[2];
     qk(sn);
-    if (LEVEL == 0) {
+    if (LEVEL == 4) {
+      weights(sc, pnew);
+      pv(pold);
+      constexpr int NM = KS + 2 * DVB;
+#pragma unroll
+      for (int i = 0; i < NM; ++i) {
+        __builtin_amdgcn_sched_group_barrier(PSG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(PSG_VALU | PSG_TRANS, (48 + NM - 1) / NM, 0);
+      }
+    } else if (LEVEL == 0) {
       pv(pconst);
     } else if (LEVEL == 1) {
       asm volatile("" : "+v"(fixed));
@@ -151,10 +165,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     __builtin_amdgcn_sched_barrier(0);
   };
   for (int it = 0; it < iters; ++it) {
-    step(sa, sb);
-    step(sb, sa);
+    step(sa, sb, pa, pb);
+    step(sb, sa, pb, pa);
   }
   float s = l;
+  for (int c = 0; c < 2; ++c) s += (float)pa[c][0] + (float)pb[c][0];
   for (int i = 0; i < DVB; ++i)
     for (int e = 0; e < 16; ++e) s += oacc[i][e];
   for (int e = 0; e < 16; ++e) s += sa[e] + sb[e];
@@ -167,6 +182,7 @@ hipError_t launch_step_probe(int level, int iters, int n_workgroups, float* sink
     case 0: hipLaunchKernelGGL((step_probe_kernel<D, 0>), dim3(n_workgroups), dim3(256), 0, stream, sink, iters, 0.f, 0.f); break;
     case 1: hipLaunchKernelGGL((step_probe_kernel<D, 1>), dim3(n_workgroups), dim3(256), 0, stream, sink, iters, 0.f, 0.f); break;
     case 2: hipLaunchKernelGGL((step_probe_kernel<D, 2>), dim3(n_workgroups), dim3(256), 0, stream, sink, iters, 0.f, 0.f); break;
+    case 4: hipLaunchKernelGGL((step_probe_kernel<D, 4>), dim3(n_workgroups), dim3(256), 0, stream, sink, iters, 0.f, 0.f); break;
     default: hipLaunchKernelGGL((step_probe_kernel<D, 3>), dim3(n_workgroups), dim3(256), 0, stream, sink, iters, 0.f, 0.f); break;
   }
   return hipGetLastError();
@@ -175,7 +191,7 @@ hipError_t launch_step_probe(int level, int iters, int n_workgroups, float* sink
 }  // namespace
 
 extern "C" int fl_probe_step(int head_dim, int level, int iters, int n_workgroups, float* sink, void* stream) {
-  if (!sink || iters <= 0 || n_workgroups <= 0 || level < 0 || level > 3) return FLP_ERR_ARG;
+  if (!sink || iters <= 0 || n_workgroups <= 0 || level < 0 || level > 4) return FLP_ERR_ARG;
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipError_t e;
   if (head_dim == 64) e = launch_step_probe<64>(level, iters, n_workgroups, sink, st);

@@ -34,7 +34,8 @@ int fl_probe_mfma_rate(const void* operands, int64_t n_fragments, int iters, int
  * data dependences, on zero operands held in registers (head_dim 64 or 128; 2 * iters blocks of 32 keys x 32 queries
  * per wave, workgroups of 4 waves).  level 0: the block's MFMAs alone; 1: MFMAs and the softmax's vector work with no
  * dependence between them; 2: the step as the forward has it (scores chained on one accumulator, weights from the
- * scores, P.V from the weights); 3: the same with the K and V fragments read from LDS.  The time per block against the
+ * scores, P.V from the weights); 3: the same with the K and V fragments read from LDS; 4: level 2 in a three-stage
+ * order (P.V on the previous block's weights, so that both groups of MFMAs run under this block's vector work).  The time per block against the
  * MFMAs' own time says what the instruction mix, its dependences and the operand reads cost before any global memory,
  * transfer or barrier enters.  One float per thread goes to `sink` (n_workgroups * 256 floats). */
 int fl_probe_step(int head_dim, int level, int iters, int n_workgroups, float* sink, void* stream);

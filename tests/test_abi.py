@@ -237,7 +237,7 @@ def test_probe_library_is_separate_and_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.fl_probe_mfma_rate(C.c_void_p(aligned), 0, 1, 1, C.c_void_p(aligned), None) == -5
     assert lib.fl_probe_mfma_rate(C.c_void_p(aligned + 2), 1, 1, 1, C.c_void_p(aligned), None) == -7
     assert lib.fl_probe_step(64, 2, 1, 1, None, None) == -5
-    assert lib.fl_probe_step(64, 4, 1, 1, C.c_void_p(aligned), None) == -5
+    assert lib.fl_probe_step(64, 5, 1, 1, C.c_void_p(aligned), None) == -5
     assert lib.fl_probe_step(96, 2, 1, 1, C.c_void_p(aligned), None) == -4
     assert lib.fl_probe_coissue(32, 0, 2, 1, 1, 1, None, None, None) == -5
     assert lib.fl_probe_coissue(32, 0, 2, 3, 1, 1, C.c_void_p(aligned), C.c_void_p(aligned), None) == -5   # waves per SIMD

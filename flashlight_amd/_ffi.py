@@ -46,6 +46,7 @@ class FlAttnParams(C.Structure):
         ("lse", C.c_void_p),
         ("dropout_threshold", C.c_uint32), ("dropout_seed", C.c_uint32 * 2),
         ("flags", C.c_uint32),
+        ("score_fn", C.c_int32), ("score_fn_params", C.c_float * 4),
     ]
 
 
@@ -215,6 +216,7 @@ class DocWorkspace:
 
 
 FLAG_DOC_PREPARED = 1
+SCORE_NONE, SCORE_SIGMOID, SCORE_CLAMP, SCORE_POLY = 0, 1, 2, 3  # fl_attn_params.score_fn
 
 
 def _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, biases,
@@ -334,6 +336,7 @@ def attn_fwd(
     dropout_p: float = 0.0,
     dropout_seed: int = 0,
     doc_workspace: Optional[DocWorkspace] = None,
+    score_fn: Optional[tuple] = None,
 ) -> torch.Tensor:
     """Fused attention forward on 4-D views: q [B, Hq(x2 if diff), Lq, Dqk], k [B, Hkv(x2), Lk, Dqk], v [B, Hkv, Lk, Dv].
 
@@ -344,6 +347,9 @@ def attn_fwd(
     `dropout_p` > 0 drops softmax weights (torch.nn.functional.dropout semantics) by a hash of (`dropout_seed`, batch,
     head, query, key); positional masks and GQA only.
     `doc_workspace` (document masks): a `DocWorkspace` handle that keeps the pre-pass's result across calls.
+    `score_fn` = (kind, (p0, p1, p2, p3)): a function of the scaled score z from the compiled-in set, in the soft-cap's
+    place: SCORE_SIGMOID p2 * sigmoid(p0 z + p1) + p3, SCORE_CLAMP min(max(p0 z + p1, p2), p3), SCORE_POLY
+    p0 + p1 z + p2 z^2 + p3 z^3.  Forward only; positional masks and bias operands.
     """
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v)):
@@ -383,12 +389,19 @@ def attn_fwd(
                      out=out[..., c:c + _MAX_DV_DIFF], validate_only=validate_only,
                      lse=lse if c == 0 else None,  # the row statistics depend on q and k only
                      dropout_p=dropout_p, dropout_seed=dropout_seed,  # so do the dropout decisions
-                     doc_workspace=doc_workspace)  # (and the key-tile lists: the slabs share one instance)
+                     doc_workspace=doc_workspace,  # (and the key-tile lists: the slabs share one instance)
+                     score_fn=score_fn)
         return out
 
     p, keep = _fill_params(lib, q, k, v, out, Hq, Hkv, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap,
                            biases, gate, diff, lambda_full, attended_dump, dropout_p, dropout_seed,
                            doc_workspace=doc_workspace)
+    if score_fn is not None:
+        kind, consts = score_fn
+        if len(consts) != 4:
+            raise ValueError("score_fn takes four constants")
+        p.score_fn = int(kind)
+        p.score_fn_params[:] = [float(c) for c in consts]
     if lse is not None:
         if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Lq) or not lse.is_contiguous() or lse.device != q.device:
             raise ValueError("lse must be a contiguous float32 [B, Hq, Lq] tensor on the inputs' device")

@@ -212,6 +212,7 @@ uint32_t wanted_features(const fl_attn_params* p) {
   uint32_t f = 0;
   if (p->alibi_heads > 0) f |= fl::F_ALIBI;
   if (p->softcap > 0.f) f |= fl::F_SOFTCAP;
+  if (p->score_fn != FL_SCORE_NONE) f |= fl::F_SCOREFN;
   if (p->bias[0] || p->bias[1]) f |= fl::F_BIAS;
   if (is_doc(p->mask_kind)) f |= fl::F_DOC;
   if (p->diff) f |= fl::F_DIFF;
@@ -377,6 +378,18 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   }
   if (p->alibi_heads < 0) return fail(FL_ERR_ARG, "alibi_heads must be >= 0");
   if (!(p->softcap >= 0.f) || !std::isfinite(p->softcap)) return fail(FL_ERR_ARG, "softcap must be finite and >= 0");
+  if (p->score_fn != FL_SCORE_NONE) {
+    if (p->score_fn < FL_SCORE_SIGMOID || p->score_fn > FL_SCORE_POLY) return fail(FL_ERR_ARG, "unknown score_fn %d", p->score_fn);
+    const float* c = p->score_fn_params;
+    // clamp bounds may be infinite (a one-sided clamp); every other constant is an ordinary number
+    const int n_finite = p->score_fn == FL_SCORE_CLAMP ? 2 : 4;
+    for (int i = 0; i < n_finite; ++i)
+      if (!std::isfinite(c[i])) return fail(FL_ERR_ARG, "score_fn_params[%d] must be finite", i);
+    if (p->score_fn == FL_SCORE_CLAMP && !(c[2] <= c[3])) return fail(FL_ERR_ARG, "score_fn clamp: lower bound above upper bound");
+    if (p->softcap > 0.f || p->alibi_heads > 0 || is_doc(p->mask_kind) || p->gate || p->diff || p->dropout_threshold)
+      return fail(FL_ERR_UNSUPPORTED, "score_fn goes with positional masks and bias operands only (no soft-cap, ALiBi, "
+                                      "document mask, gate, differential attention or dropout)");
+  }
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb]) continue;
     if (p->bias_dtype[nb] != p->dtype && p->bias_dtype[nb] != FL_F32)
@@ -398,7 +411,8 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   const fl::Instance* in = select_instance(p);
   if (!in)
     return fail(FL_ERR_UNSUPPORTED,
-                "no kernel instance for Dqk=%d Dv=%d features=0x%x (alibi=1 softcap=2 bias=4 doc=8 diff=16 gate=32 dump=64)",
+                "no kernel instance for Dqk=%d Dv=%d features=0x%x (alibi=1 softcap=2 bias=4 doc=8 diff=16 gate=32 dump=64 "
+                "dropout=128 score_fn=256)",
                 p->Dqk, p->Dv, wanted_features(p));
   const int64_t nkt = ((int64_t)p->Lk + in->bn - 1) / in->bn;
   if (nkt > fl::kMaxKeyTiles || lds_bytes_for(in, p) > fl::kMaxLdsBytes)
@@ -436,7 +450,7 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   static const bool disabled = std::getenv("FL_NO_PAIRBIAS") != nullptr;  // A/B knob: the general kernel instead
   if (disabled) return false;
   if (p->Dqk != p->Dv || p->mask_kind != FL_MASK_NONE || p->alibi_heads > 0 || p->softcap > 0.f ||
-      p->diff || p->attended_dump || p->dropout_threshold || p->lse)
+      p->diff || p->attended_dump || p->dropout_threshold || p->lse || p->score_fn != FL_SCORE_NONE)
     return false;
   // one operand that several consecutive batch entries share (dense over heads, queries and keys), and optionally one
   // that is a row of keys per batch entry, the same for every head and query; in either order
@@ -632,6 +646,28 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   kp.doc_stride = p->doc_stride;
   kp.alibi_heads = p->alibi_heads;
   kp.softcap = p->softcap;
+  if (p->score_fn != FL_SCORE_NONE) {
+    // scale and log2(e) folded into the constants (in double): the kernel works on the raw q.k and in log2 units
+    const double l2e = 1.4426950408889634, sc = p->scale;
+    const float* c = p->score_fn_params;
+    kp.score_fn = p->score_fn;
+    if (p->score_fn == FL_SCORE_SIGMOID) {
+      kp.score_k[0] = (float)(-(double)c[0] * sc * l2e);
+      kp.score_k[1] = (float)(-(double)c[1] * l2e);
+      kp.score_k[2] = (float)((double)c[2] * l2e);
+      kp.score_k[3] = (float)((double)c[3] * l2e);
+    } else if (p->score_fn == FL_SCORE_CLAMP) {
+      kp.score_k[0] = (float)((double)c[0] * sc * l2e);
+      kp.score_k[1] = (float)((double)c[1] * l2e);
+      kp.score_k[2] = (float)((double)c[2] * l2e);
+      kp.score_k[3] = (float)((double)c[3] * l2e);
+    } else {
+      kp.score_k[0] = (float)((double)c[0] * l2e);
+      kp.score_k[1] = (float)((double)c[1] * sc * l2e);
+      kp.score_k[2] = (float)((double)c[2] * sc * sc * l2e);
+      kp.score_k[3] = (float)((double)c[3] * sc * sc * sc * l2e);
+    }
+  }
   for (int nb = 0; nb < 2; ++nb) {
     kp.bias[nb] = static_cast<const fl::bf16_t*>(p->bias[nb]);
     kp.bdiv[nb] = p->bias[nb] ? p->bias_batch_div[nb] : 1;
@@ -728,6 +764,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (rc) return rc;
   if (p->gate || p->diff || p->attended_dump)
     return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
+  if (p->score_fn != FL_SCORE_NONE) return fail(FL_ERR_UNSUPPORTED, "backward: score_fn is forward-only");
   const bool has_bias = p->bias[0] || p->bias[1];
   if (has_bias && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind) || p->dropout_threshold))
     return fail(FL_ERR_UNSUPPORTED, "backward: bias operands go with positional masks only (no ALiBi, soft-cap, document mask or dropout)");

@@ -38,6 +38,7 @@ enum : uint32_t {
   F_GATE = 32u,    // out *= sigmoid(gate)
   F_DUMP = 64u,    // write the attended-pair bitmap (test hook), skip nothing else
   F_DROPOUT = 128u,  // softmax weights are dropped by a counter-based hash of (seed, batch, head, query, key)
+  F_SCOREFN = 256u,  // a function of the scaled score from a small compiled-in set (KParams::score_fn), in the soft-cap's place
 };
 
 enum : int { MASK_NONE = 0, MASK_CAUSAL = 1, MASK_SLIDING = 2, MASK_PREFIX = 3, MASK_DOC = 4, MASK_DOC_CAUSAL = 5 };
@@ -91,6 +92,11 @@ struct KParams {
   float drop_rescale;     // 65536 / (65536 - drop_thr), applied to the kept weights
   int32_t head_group;  // (batch, head) pairs whose query tiles are dealt together, longest first (1: head by head)
   int32_t o_wide;      // o is 16-byte aligned with strides that are multiples of 8 elements: 16-byte stores
+  // F_SCOREFN: 1 sigmoid, 2 clamp, 3 cubic polynomial, with four constants the host has folded scale and log2(e) into
+  // (x = the raw q.k; results in log2 units):  1: k2 / (1 + 2^(k0 x + k1)) + k3;  2: med3(k0 x + k1, k2, k3);
+  // 3: ((k3 x + k2) x + k1) x + k0
+  int32_t score_fn;
+  float score_k[4];
   int32_t n_qtiles;  // ceil(Lq / BM)
   int32_t n_ktiles;  // ceil(Lk / BN)
 };
@@ -399,7 +405,9 @@ void fwd_kernel(const KParams p) {
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kBias = FEAT & F_BIAS, kDoc = FEAT & F_DOC;
   constexpr bool kDiff = FEAT & F_DIFF, kGate = FEAT & F_GATE, kDump = FEAT & F_DUMP;
   constexpr bool kDrop = FEAT & F_DROPOUT;
-  constexpr bool kMod = kAlibi || kSoftcap || kBias;  // scores are transformed before the softmax
+  constexpr bool kScoreFn = FEAT & F_SCOREFN;
+  static_assert(!(kScoreFn && (kSoftcap || kAlibi)), "one function of the score per kernel");
+  constexpr bool kMod = kAlibi || kSoftcap || kBias || kScoreFn;  // scores are transformed before the softmax
   constexpr float kLog2e = 1.4426950408889634f;
   using E = typename T::Elem;  // pointers in KParams are typed bf16_t whatever E is: 16 opaque bits
   typedef E ex8 __attribute__((ext_vector_type(8)));
@@ -524,6 +532,13 @@ void fwd_kernel(const KParams p) {
     cap_k1 = p.scale / p.softcap * 2.0f * kLog2e;  // exp2 argument of e^{2x/cap}
     cap_c = p.softcap * kLog2e;                    // cap in log2 units
   }
+  int fn_kind = 0;
+  float fn_k[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (kScoreFn) {
+    fn_kind = __builtin_amdgcn_readfirstlane(p.score_fn);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fn_k[i] = p.score_k[i];
+  }
   int64_t qdoc[QB];
   if constexpr (kDoc) {
 #pragma unroll
@@ -541,7 +556,7 @@ void fwd_kernel(const KParams p) {
   }
   // With dense biases as the only score modification the modified scores stay in natural units (s = qk * scale + bias)
   // and the factor log2(e) rides in the exponential's multiply-add; other modifications produce log2 units directly.
-  constexpr bool kNatural = kBias && !kSoftcap && !kAlibi;
+  constexpr bool kNatural = kBias && !kSoftcap && !kAlibi && !kScoreFn;
   const float c2 = kNatural ? kLog2e : (kMod ? 1.0f : p.scale_log2);  // s * c2 is the logit in log2 units
   // The running maximum only moves when some row of the wave sees a score more than kTau (log2 units) above it,
   // so exp2 arguments stay <= kTau and the accumulators are rescaled on few tiles.  Any m gives the same O / l.
@@ -797,7 +812,8 @@ void fwd_kernel(const KParams p) {
             // multiply-add that precedes it, leaving one multiply-add with a literal per score
             const float alibi0 = kAlibi ? slope_l2 * rel0 : 0.f;
             const float cap_shift = cap_c + alibi0 - (kFoldRef ? ref_now(qb) : 0.f);
-            auto combine = [&]() FL_INLINE {
+            auto combine_as = [&](auto fn_tag) FL_INLINE {
+              constexpr int kFn = decltype(fn_tag)::value;
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
                 const float x = s[kb][qb][i];
@@ -809,6 +825,12 @@ void fwd_kernel(const KParams p) {
                     const float e = fast_exp2(x * cap_k1);
                     const float rc = fast_rcp(e + 1.0f);
                     tl2 = __builtin_fmaf(rc, -2.0f * cap_c, cap_shift);
+                  } else if constexpr (kFn == 1) {
+                    tl2 = __builtin_fmaf(fast_rcp(1.0f + fast_exp2(__builtin_fmaf(x, fn_k[0], fn_k[1]))), fn_k[2], fn_k[3]);
+                  } else if constexpr (kFn == 2) {
+                    tl2 = __builtin_amdgcn_fmed3f(__builtin_fmaf(x, fn_k[0], fn_k[1]), fn_k[2], fn_k[3]);
+                  } else if constexpr (kFn == 3) {
+                    tl2 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(x, fn_k[3], fn_k[2]), x, fn_k[1]), x, fn_k[0]);
                   } else {
                     tl2 = kAlibi ? __builtin_fmaf(x, p.scale_log2, alibi0) : x * p.scale_log2;
                   }
@@ -816,6 +838,16 @@ void fwd_kernel(const KParams p) {
                   if constexpr (kBias) tl2 = __builtin_fmaf(bv[i], kLog2e, tl2);
                 }
                 s[kb][qb][i] = tl2;
+              }
+            };
+            // (the kind of score function is uniform: one branch per block, outside the loop over the scores)
+            auto combine = [&]() FL_INLINE {
+              if constexpr (kScoreFn) {
+                if (fn_kind == 1) combine_as(std::integral_constant<int, 1>{});
+                else if (fn_kind == 2) combine_as(std::integral_constant<int, 2>{});
+                else combine_as(std::integral_constant<int, 3>{});
+              } else {
+                combine_as(std::integral_constant<int, 0>{});
               }
             };
             if constexpr (kBias) {

@@ -33,21 +33,24 @@ def _alloc_out(q: torch.Tensor, v: torch.Tensor, diff: bool, seq_major_out: bool
 def attn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, mask_kind: int, window: int, prefix: int,
              doc_ids: Optional[torch.Tensor], alibi_heads: int, softcap: float,
              bias0: Optional[torch.Tensor], bias0_div: int, bias1: Optional[torch.Tensor], bias1_div: int,
-             gate: Optional[torch.Tensor], diff: bool, lambda_full: float, seq_major_out: bool) -> torch.Tensor:
+             gate: Optional[torch.Tensor], diff: bool, lambda_full: float, seq_major_out: bool, score_fn: int = 0,
+             score_p0: float = 0.0, score_p1: float = 0.0, score_p2: float = 0.0, score_p3: float = 0.0) -> torch.Tensor:
     """Same arguments as `_ffi.attn_fwd`, flattened to what an operator schema can carry: scale <= 0 selects the
     default 1/sqrt(Dqk); bias operands with their batch divisors; `seq_major_out` asks for the result in [B, L, H, Dv]
-    memory order."""
+    memory order; a score function as its kind and four constants."""
     out = _alloc_out(q, v, diff, seq_major_out)
     biases = [(b, d) for b, d in ((bias0, bias0_div), (bias1, bias1_div)) if b is not None]
     _ffi.attn_fwd(q, k, v, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window, prefix=prefix,
                   doc_ids=doc_ids, alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
-                  lambda_full=lambda_full, out=out)
+                  lambda_full=lambda_full, out=out,
+                  score_fn=(score_fn, (score_p0, score_p1, score_p2, score_p3)) if score_fn else None)
     return out
 
 
 @attn_fwd.register_fake
 def _attn_fwd_fake(q, k, v, scale, mask_kind, window, prefix, doc_ids, alibi_heads, softcap, bias0, bias0_div, bias1,
-                   bias1_div, gate, diff, lambda_full, seq_major_out):
+                   bias1_div, gate, diff, lambda_full, seq_major_out, score_fn=0, score_p0=0.0, score_p1=0.0, score_p2=0.0,
+                   score_p3=0.0):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, dim]")
     return _alloc_out(q, v, diff, seq_major_out)
@@ -259,7 +262,7 @@ def _pad_head_dims(q, k, v, gate, diff):
 
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
-             dropout_seed=None, doc_workspace=None) -> torch.Tensor:
+             dropout_seed=None, doc_workspace=None, score_fn=None) -> torch.Tensor:
     """What the front-ends call: the registered operator while `torch.compile` is tracing, the C ABI otherwise; the
     differentiable operator when a gradient with respect to q, k or v will be asked for.
 
@@ -267,7 +270,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     `attention_variants.honor_dropout`).  `dropout_seed=None` draws a fresh 63-bit seed from torch's default CPU
     generator, so `torch.manual_seed` reproduces a run; the same seed gives the same decisions in forward and backward.
     `doc_workspace` (an `_ffi.DocWorkspace`) is used by the plain forward call only; traced and differentiable calls run
-    their pre-pass every time."""
+    their pre-pass every time.  `score_fn` = (kind, four constants), see `_ffi.attn_fwd`: forward only."""
     dropout_p = float(dropout_p)
     _ffi.dropout_threshold(dropout_p)  # range check
     padded = _pad_head_dims(q, k, v, gate, diff)
@@ -280,7 +283,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         out = dispatch(qp, kp, vp, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                        alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gp, diff=diff, lambda_full=lambda_full,
                        seq_major_out=seq_major_out, dropout_p=dropout_p, dropout_seed=dropout_seed,
-                       doc_workspace=doc_workspace)
+                       doc_workspace=doc_workspace, score_fn=score_fn)
         return out[..., :v.size(-1)]
     if dropout_p > 0.0:
         if biases or gate is not None or diff or seq_major_out:
@@ -295,6 +298,8 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         dropout_seed = 0
     wants_grad = torch.is_grad_enabled() and any(
         t is not None and t.requires_grad for t in (q, k, v, gate, *(b for b, _ in biases)))
+    if score_fn is not None and (wants_grad or dropout_p > 0.0):
+        raise NotImplementedError("score functions other than the tanh soft-cap are forward-only and take no dropout")
     if wants_grad or (dropout_p > 0.0 and torch.compiler.is_compiling()):
         # (the result comes back in [B, H, L, Dv] memory order whatever seq_major_out asks for)
         return _differentiable(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
@@ -302,11 +307,12 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
                                lambda_full=lambda_full, dropout_p=dropout_p, dropout_seed=dropout_seed)
     if torch.compiler.is_compiling():
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
+        fn_kind, fn_c = (int(score_fn[0]), [float(c) for c in score_fn[1]]) if score_fn is not None else (0, [0.0] * 4)
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),
                         doc_ids, int(alibi_heads), float(softcap), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), gate,
-                        bool(diff), float(lambda_full), bool(seq_major_out))
+                        bool(diff), float(lambda_full), bool(seq_major_out), fn_kind, fn_c[0], fn_c[1], fn_c[2], fn_c[3])
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None
     return _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                          alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
                          lambda_full=lambda_full, out=out, dropout_p=dropout_p, dropout_seed=dropout_seed,
-                         doc_workspace=doc_workspace)
+                         doc_workspace=doc_workspace, score_fn=score_fn)

@@ -127,7 +127,25 @@ typedef struct fl_attn_params {
 
   /* Bit set of FL_FLAG_*; unknown bits are rejected.  No counterpart in the reference. */
   uint32_t flags;
+
+  /* A function of the scaled score other than the tanh soft-cap, applied where `softcap` would be: the reference's
+   * softcap.py:49 calls an arbitrary score_mod(score, b, h, q_idx, kv_idx) on the score matrix inside its fused kernel;
+   * this is the part of that freedom the kernel has compiled in.  With z = qk * scale:
+   *   FL_SCORE_SIGMOID  y = p[2] * sigmoid(p[0] * z + p[1]) + p[3]
+   *   FL_SCORE_CLAMP    y = min(max(p[0] * z + p[1], p[2]), p[3])      (p[2] <= p[3], either may be infinite: a ReLU
+   *                                                                     is (1, 0, 0, +inf))
+   *   FL_SCORE_POLY     y = p[0] + p[1] z + p[2] z^2 + p[3] z^3
+   * y takes the place of the scaled score (biases and the mask follow).  Positional masks, grouped heads and bias
+   * operands go with it; soft-cap, ALiBi, document masks, gate, differential attention, dropout and fl_attn_bwd do
+   * not.  Head dims 64 and 128. */
+  int32_t score_fn; /* FL_SCORE_NONE (0, what a zeroed struct says) or one of the above */
+  float score_fn_params[4];
 } fl_attn_params;
+
+#define FL_SCORE_NONE 0
+#define FL_SCORE_SIGMOID 1
+#define FL_SCORE_CLAMP 2
+#define FL_SCORE_POLY 3
 
 /* fl_attn_fwd, document masks only: `workspace` still holds what an earlier fl_attn_fwd call (without this flag) wrote
  * there for the same doc_ids contents, doc_stride, B, Lq = Lk, mask_kind, head dims, dtype and features, and the

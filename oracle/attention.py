@@ -36,8 +36,10 @@ def _group(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, enable_g
 
 def _softmax_attention(query, key, value, scale, *, masked: Optional[MaskFn] = None, fill: float = NEG_INF,
                        bias: Optional[BiasFn] = None, softcap: Optional[float] = None,
-                       q_block: Optional[int] = None) -> torch.Tensor:
-    """softmax(mask(cap(q k^T * scale) + bias)) v over the last two axes; leading axes broadcast like matmul."""
+                       q_block: Optional[int] = None, score_fn=None) -> torch.Tensor:
+    """softmax(mask(cap(q k^T * scale) + bias)) v over the last two axes; leading axes broadcast like matmul.
+    `score_fn`, a callable on the scaled score block, takes the cap's place (softcap.py:49 applies whatever
+    `score_mod` it is given there)."""
     L, S = query.size(-2), key.size(-2)
     step = L if not q_block else q_block
     k_t = key.transpose(-2, -1)
@@ -49,6 +51,8 @@ def _softmax_attention(query, key, value, scale, *, masked: Optional[MaskFn] = N
         w = torch.matmul(query[..., a:b, :], k_t) * scale
         if softcap is not None:
             w = softcap * torch.tanh(w / softcap)
+        if score_fn is not None:
+            w = score_fn(w)
         if bias is not None:
             terms = bias(q_idx, k_idx)
             for term in (terms if isinstance(terms, (tuple, list)) else (terms,)):
@@ -174,10 +178,14 @@ def tanh_softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
 def attention_softcapped(query, key, value, score_mod=None, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
                          enable_gqa=False, softcap_threshold=30.0, *, honor_causal=False, q_block=None):
     """attention_variants/softcap.py:4-53: softmax(score_mod(q k^T * scale)) v.  `score_mod` here is the cap value
-    (None = softcap_threshold, which the reference declares but never reads)."""
-    cap = float(softcap_threshold if score_mod is None else score_mod)
+    (None = softcap_threshold, which the reference declares but never reads), or a callable of the reference's
+    signature `(score, b, h, q_idx, kv_idx)`, which is applied to the scaled scores as softcap.py:49 does."""
     q, k, v = _group(query, key, value, enable_gqa)
     masked = (lambda qi, ki: ki > qi) if (honor_causal and is_causal) else None
+    if callable(score_mod):
+        return _softmax_attention(q, k, v, _default_scale(query, scale), masked=masked, fill=NEG_INF, q_block=q_block,
+                                  score_fn=lambda w: score_mod(w, query.size(0), query.size(1), None, None))
+    cap = float(softcap_threshold if score_mod is None else score_mod)
     return _softmax_attention(q, k, v, _default_scale(query, scale), softcap=cap, masked=masked, fill=NEG_INF,
                               q_block=q_block)
 

@@ -82,6 +82,29 @@ def test_plan_reports_launch_shape(lib):
     assert plan["workgroups"] == 2 * 4 * ((300 + bm - 1) // bm)
 
 
+def test_score_function_arguments(lib):
+    # fl_attn_params.score_fn: a function of the scaled score from the compiled-in set, in the soft-cap's place
+    def with_fn(kind, consts, **kw):
+        p = good_params(D=kw.pop("D", 64))
+        p.score_fn = kind
+        p.score_fn_params[:] = consts
+        for name, value in kw.items():
+            setattr(p, name, value)
+        return p
+    inf = float("inf")
+    assert rc(lib, with_fn(_ffi.SCORE_SIGMOID, (0.5, -1.0, 3.0, 2.0))) == 0, _ffi.last_error()
+    assert rc(lib, with_fn(_ffi.SCORE_CLAMP, (1.0, 0.0, 0.0, inf), D=128, mask_kind=_ffi.MASK_CAUSAL)) == 0, _ffi.last_error()
+    assert rc(lib, with_fn(_ffi.SCORE_POLY, (0.0, -1.0, 0.1, 0.01))) == 0, _ffi.last_error()
+    assert _ffi.plan(with_fn(_ffi.SCORE_POLY, (0.0, 1.0, 0.0, 0.0)))["features"] & 256
+    assert rc(lib, with_fn(4, (0.0,) * 4)) == -5 and "score_fn" in _ffi.last_error()
+    assert rc(lib, with_fn(_ffi.SCORE_CLAMP, (1.0, 0.0, 2.0, 1.0))) == -5 and "bound" in _ffi.last_error()
+    assert rc(lib, with_fn(_ffi.SCORE_SIGMOID, (1.0, 0.0, inf, 0.0))) == -5 and "finite" in _ffi.last_error()
+    assert rc(lib, with_fn(_ffi.SCORE_POLY, (float("nan"), 1.0, 0.0, 0.0))) == -5
+    for bad in (dict(softcap=30.0), dict(alibi_heads=4), dict(dropout_threshold=1000), dict(diff=1)):
+        assert rc(lib, with_fn(_ffi.SCORE_POLY, (0.0, 1.0, 0.1, 0.0), **bad)) == -4, bad
+    assert rc(lib, with_fn(_ffi.SCORE_POLY, (0.0, 1.0, 0.1, 0.0), D=32)) == -4 and "no kernel instance" in _ffi.last_error()
+
+
 def test_large_unmasked_calls_at_head_dim_128_take_256_row_workgroups(lib):
     # one 8-wave workgroup per compute unit brings each K/V tile in once for 256 query rows; chosen only without a mask
     # or score modification, at head dim 128, and when such workgroups still fill the part twice over

@@ -187,10 +187,10 @@ def test_score_mod_callables_of_the_softcap_signature(D):
 
 def test_score_mod_the_kernel_cannot_apply_is_refused():
     q, k, v = qkv(1, 2, 2, 64, 64, seed=50)
-    for fn in (lambda s, b, h, qi, ki: torch.relu(s),
+    for fn in (lambda s, b, h, qi, ki: torch.exp(s),
                lambda s, b, h, qi, ki: torch.tanh(torch.tanh(s)),
-               lambda s, b, h, qi, ki: s * s,
-               lambda s, b, h, qi, ki: -s):
+               lambda s, b, h, qi, ki: s ** 4,
+               lambda s, b, h, qi, ki: torch.sigmoid(s) * s):
         with pytest.raises(NotImplementedError):
             A.attention_softcapped(q, k, v, score_mod=fn)
 

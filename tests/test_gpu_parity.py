@@ -350,6 +350,44 @@ def test_results_written_to_an_8_byte_aligned_view_match_the_16_byte_path(D, mas
     assert torch.all(big[..., :4] == 7.0) and torch.all(big[..., 4 + D:] == 7.0)  # nothing written beside the view
 
 
+SCORE_MODS = {
+    "relu": lambda s, *_: torch.relu(s),
+    "sigmoid": lambda s, *_: 6.0 * torch.sigmoid(0.5 * s - 1.0) + 2.0,
+    "clamp": lambda s, *_: torch.clamp(2.0 * s + 1.0, min=-3.0, max=5.0),
+    "negated clamp": lambda s, *_: 1.0 - torch.clamp(s, min=-2.0) * 1.5,
+    "cubic": lambda s, *_: 0.02 * s ** 3 - 0.5 * s + 4.0,
+    "square": lambda s, *_: -0.25 * s * s,
+}
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name", sorted(SCORE_MODS))
+def test_score_mod_callables_beyond_the_soft_cap(name, D):
+    # softcap.py:49 applies whatever score_mod it is handed to the scaled score matrix; callables that trace to a
+    # sigmoid, ReLU / clamp or polynomial (up to the cube) of the score run in the kernel's registers like the tanh
+    fn = SCORE_MODS[name]
+    B, Hq, Hkv, S = 2, 8, 2, 333
+    q, k, v = qkv(B, Hq, Hkv, S, D, seed=61)
+    q = (q.float() * 2.0).to(q.dtype)  # logits of a few units, so that every branch of the functions is exercised
+    for causal in (False, True):
+        out = A.attention_softcapped(q, k, v, score_mod=fn, enable_gqa=True, is_causal=causal)
+        ref = O.attention_softcapped(*f32(q, k, v), score_mod=fn, enable_gqa=True, is_causal=causal, honor_causal=True)
+        assert_parity(out, ref, f"{name} D={D} causal={causal}")
+    # with a tensor addend (a dense bias operand rides along) and a caller's scale
+    t = torch.randn(Hq, S, S, generator=torch.Generator().manual_seed(7)).to(DEV)  # (under GQA the reference views it as [Hkv, G, L, S])
+    fn_t = lambda s, *a: fn(s) + t  # noqa: E731
+    out = A.attention_softcapped(q, k, v, score_mod=fn_t, enable_gqa=True, scale=0.2)
+    ref = O.attention_softcapped(*f32(q, k, v), score_mod=lambda s, *a: fn(s) + t.float().view(Hkv, Hq // Hkv, S, S), enable_gqa=True, scale=0.2)
+    assert_parity(out, ref, f"{name} D={D} + tensor")
+
+
+def test_score_functions_are_forward_only():
+    q, k, v = qkv(1, 2, 2, 64, 64, seed=3)
+    q.requires_grad_(True)
+    with pytest.raises(NotImplementedError, match="forward-only"):
+        A.attention_softcapped(q, k, v, score_mod=lambda s, *_: torch.relu(s))
+
+
 # ---- dense score_mod and invariant point attention -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("gqa", [False, True])

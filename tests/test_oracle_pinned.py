@@ -143,6 +143,29 @@ def test_identities():
     assert torch.allclose(O.attention_evoformer(qe, ke, ve, [z], gate=big), ref)          # sigmoid(50) == 1
 
 
+def test_callable_score_mod_against_pure_python_loops_and_identities():
+    # softcap.py:49 hands the scaled score matrix to whatever callable it was given: the oracle's callable path against
+    # the triple loops with math.* functions on single logits, and the identities that tie it to the pinned variants
+    q, k, v = small()
+    sc = 1 / math.sqrt(4)
+    cases = [
+        (lambda s, *_: torch.relu(s), lambda s, h, i, j: max(s, 0.0)),
+        (lambda s, *_: 6.0 * torch.sigmoid(0.5 * s - 1.0) + 2.0, lambda s, h, i, j: 6.0 / (1.0 + math.exp(-(0.5 * s - 1.0))) + 2.0),
+        (lambda s, *_: torch.clamp(2.0 * s + 1.0, min=-0.5, max=0.75), lambda s, h, i, j: min(max(2.0 * s + 1.0, -0.5), 0.75)),
+        (lambda s, *_: 0.5 * s ** 3 - s + 4.0, lambda s, h, i, j: 0.5 * s * s * s - s + 4.0),
+    ]
+    for fn, logit in cases:
+        assert torch.allclose(O.attention_softcapped(q, k, v, score_mod=fn), brute_force(q, k, v, sc, logit=logit), atol=1e-12)
+        assert torch.allclose(O.attention_softcapped(q, k, v, score_mod=fn, is_causal=True, honor_causal=True),
+                              brute_force(q, k, v, sc, lambda n, i, j: j <= i, logit=logit), atol=1e-12)
+    assert torch.allclose(O.attention_softcapped(q, k, v, score_mod=lambda s, *_: s), O.attention_vanilla_nogqa(q, k, v))
+    assert torch.allclose(O.attention_softcapped(q, k, v, score_mod=lambda s, *_: 2.5 * torch.tanh(s / 2.5)),
+                          O.attention_softcapped(q, k, v, score_mod=2.5))
+    # the callable sees the score times `scale`, nothing else
+    assert torch.allclose(O.attention_softcapped(q, k, v, score_mod=lambda s, *_: torch.relu(s), scale=0.3),
+                          brute_force(q, k, v, 0.3, logit=lambda s, h, i, j: max(s, 0.0)), atol=1e-12)
+
+
 def test_row_blocks_do_not_change_results():
     q, k, v = (torch.randn(1, 2, 50, 8) for _ in range(3))
     ids = torch.from_numpy(O.document_ids_from_lengths([20, 30]))[None]

@@ -269,7 +269,7 @@ def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...],
 def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: Optional[torch.Tensor],
                     biases: Sequence[torch.Tensor], masks: Sequence[torch.Tensor], *, scale: float, mask_kind: int,
                     window: int, prefix: int, alibi_heads: int, softcap: float, gqa: bool,
-                    mask_invert: Sequence[bool] = (), diff_lambda: Optional[float] = None) -> torch.Tensor:
+                    mask_invert: Sequence[bool] = (), diff_lambda: Optional[float] = None, score_fn=None) -> torch.Tensor:
     """Target of the replacement node.  q [*lead, H, L, E] (or [N, Hkv, G, L, E] with `gqa`), k/v likewise with S keys;
     `biases` are added to the scaled scores, `masks` (bool, True = masked unless the matching `mask_invert` entry is
     set) are those the rewrite could not map to a positional or document mask.  Returns what the eager region
@@ -307,7 +307,7 @@ def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: 
         kb[-2:] = [(b1.float() + b2.float(), d1)]
     if diff_lambda is None:
         out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
-                           alibi_heads=alibi_heads, softcap=softcap, biases=kb)
+                           alibi_heads=alibi_heads, softcap=softcap, biases=kb, score_fn=score_fn)
         return out.reshape(result_shape)
     out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                        alibi_heads=alibi_heads, softcap=softcap, biases=kb, diff=True, lambda_full=float(diff_lambda))
@@ -322,9 +322,74 @@ class _Region:
         self.q = self.k = self.v = None
         self.scale = 1.0
         self.softcap = 0.0
+        self.score_fn = None                 # (kind, four constants) of fl_attn_params.score_fn
         self.biases: List[fx.Node] = []
         self.masks: List[Tuple[fx.Node, bool]] = []   # (mask node, invert)
         self.out: Optional[fx.Node] = None
+
+
+_PASS_OPS = ("to", "type_as", "float", "contiguous", "clone")
+_FN_OPS = ("relu", "sigmoid", "tanh", "clamp", "clip", "clamp_min", "clamp_max", "pow", "square", "neg", "sub", "rsub",
+           "mul", "div", "add")
+
+
+def _peel_function(n: fx.Node, r: _Region, qk_memo, mods_below: List[str]):
+    """`n` and everything between it and the q k^T matmul is a function of the scores and numbers alone (no tensor
+    enters): the chain is handed, as a callable, to the analysis the soft-cap front-end uses for a caller's score_mod
+    (scale, tanh soft-cap, or one of the compiled-in score functions: sigmoid, clamp / ReLU, polynomial)."""
+    from .attention_variants.softcap import analyse_score_mod
+    chain: List[fx.Node] = []
+    seen = set()
+    root: List[Optional[fx.Node]] = [None]
+
+    def visit(x: fx.Node):
+        if x in seen:
+            return
+        nm = _name(x)
+        if nm == "matmul" and len(x.args) >= 2 and _is_last2_transpose(x.args[1]) is not None:
+            if root[0] is not None and root[0] is not x:
+                raise _NoMatch("a function of two score matrices")
+            root[0] = x
+            seen.add(x)
+            return
+        if nm not in _FN_OPS and nm not in _PASS_OPS:
+            raise _NoMatch(f"unsupported operation on the scores: {nm}")
+        for a in list(x.args) + list(x.kwargs.values()):
+            if isinstance(a, fx.Node):
+                visit(a)
+            elif not (a is None or _is_number(a) or isinstance(a, (torch.dtype, bool))):
+                raise _NoMatch(f"{nm} of the scores with an argument that is not a number")
+        seen.add(x)
+        chain.append(x)
+
+    visit(n)
+    if root[0] is None:
+        raise _NoMatch("scores do not come from a matmul")
+
+    def fn(score, *_ignored):
+        env = {root[0]: score}
+        for x in chain:
+            if _name(x) in _PASS_OPS:  # casts and copies leave the value as it is
+                env[x] = env[x.args[0]]
+                continue
+            args = [env[a] if isinstance(a, fx.Node) else a for a in x.args]
+            kwargs = {k: env[v] if isinstance(v, fx.Node) else v for k, v in x.kwargs.items()}
+            env[x] = x.target(*args, **kwargs) if x.op == "call_function" else getattr(args[0], x.target)(*args[1:], **kwargs)
+        return env[n]
+
+    try:
+        mult, cap, bias, score_fn = analyse_score_mod(fn)
+    except NotImplementedError as e:
+        raise _NoMatch(str(e)) from e
+    if bias is not None or (cap and (r.softcap or "softcap" in mods_below)):
+        raise _NoMatch("a second soft-cap, or a tensor inside the score function")
+    r.scale *= mult
+    if cap:
+        r.softcap = cap
+    r.score_fn = score_fn
+    r.nodes += list(reversed(chain))
+    mods_below.append("softcap" if (cap or score_fn is not None) else "scale")
+    return _peel_scores(root[0], r, qk_memo, mods_below)
 
 
 def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
@@ -369,8 +434,10 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
     if nm == "add":
         a, b = n.args[0], n.args[1]
         if _is_number(a) or _is_number(b):
-            raise _NoMatch("scalar added to the scores")
+            return _peel_function(n, r, qk_memo, mods_below)
         a_has = _contains_qk(a, qk_memo)
+        if a_has and _contains_qk(b, qk_memo):
+            return _peel_function(n, r, qk_memo, mods_below)  # a sum of two functions of the scores
         inner, bias = (a, b) if a_has else (b, a)
         if not a_has and not _contains_qk(b, qk_memo):
             raise _NoMatch("add without a score operand")
@@ -383,6 +450,9 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
         if nm == "mul" and _is_number(a):
             a, b = b, a
         if not _is_number(b) or not isinstance(a, fx.Node):
+            if isinstance(n.args[0], fx.Node) and isinstance(n.args[1], fx.Node) and nm == "mul" \
+                    and _contains_qk(n.args[0], qk_memo) and _contains_qk(n.args[1], qk_memo):
+                return _peel_function(n, r, qk_memo, mods_below)  # a product of two functions of the scores
             raise _NoMatch("scores multiplied by a tensor")
         c = float(b) if nm == "mul" else 1.0 / float(b)
         if _name(a) == "tanh":  # cap * tanh(x / cap)
@@ -399,12 +469,14 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
             r.nodes += [n, a, t_in]
             mods_below.append("softcap")
             return _peel_scores(t_in.args[0], r, qk_memo, mods_below)
-        if not c > 0:
-            raise _NoMatch("non-positive scale")
+        if not c > 0 or _name(a) in _FN_OPS and _name(a) not in ("mul", "div", "add"):
+            return _peel_function(n, r, qk_memo, mods_below)  # a factor on a function of the scores, or a negative one
         r.scale *= c
         r.nodes.append(n)
         mods_below.append("scale")
         return _peel_scores(a, r, qk_memo, mods_below)
+    if nm in _FN_OPS:
+        return _peel_function(n, r, qk_memo, mods_below)
     raise _NoMatch(f"unsupported operation on the scores: {nm}")
 
 
@@ -418,7 +490,7 @@ def _contains_qk(n: Any, memo: Dict[fx.Node, bool]) -> bool:
     memo[n] = False
     if nm == "matmul" and len(n.args) >= 2 and _is_last2_transpose(n.args[1]) is not None:
         r = True
-    elif nm in ("where", "masked_fill", "add", "mul", "div", "tanh", "to", "type_as", "float", "contiguous", "clone"):
+    elif nm in ("where", "masked_fill") or nm in _FN_OPS or nm in _PASS_OPS:
         r = any(_contains_qk(a, memo) for a in n.args if isinstance(a, fx.Node))
     else:
         r = False
@@ -541,7 +613,7 @@ def _merge_differential(gm: fx.GraphModule) -> int:
             continue
         if not all(x.op == "call_function" and x.target is fused_attention for x in (a, b)):
             continue
-        if a.kwargs != b.kwargs or a.kwargs.get("gqa") or a.kwargs.get("diff_lambda") is not None:
+        if a.kwargs != b.kwargs or a.kwargs.get("gqa") or a.kwargs.get("diff_lambda") is not None or a.kwargs.get("score_fn"):
             continue
         if a.args[2] is not b.args[2] or a.args[3] is not b.args[3]:
             continue
@@ -573,6 +645,11 @@ def fuse_attention(gm: fx.GraphModule) -> int:
             gqa, L, S, Hq = _shapes(r)
             kwargs: Dict[str, Any] = dict(scale=float(r.scale), mask_kind=_ffi.MASK_NONE, window=0, prefix=0,
                                           alibi_heads=0, softcap=float(r.softcap), gqa=gqa)
+            # (a score function other than the soft-cap goes with positional masks and dense operands only: document
+            # ids and the in-kernel ALiBi term stay dense then)
+            plain = r.score_fn is None
+            if not plain:
+                kwargs["score_fn"] = r.score_fn
             doc_ids = None
             run_masks: List[fx.Node] = []
             run_invert: List[bool] = []
@@ -598,7 +675,7 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                         const_biases.append(torch.zeros(m.shape, dtype=_val(r.q).dtype, device=m.device)
                                             .masked_fill_(m, _NEG_INF))
                     continue
-                if len(phs) == 1 and kwargs["mask_kind"] == _ffi.MASK_NONE:
+                if plain and len(phs) == 1 and kwargs["mask_kind"] == _ffi.MASK_NONE:
                     kind = _classify_document_mask(node, phs[0], invert, L, S, gm)
                     if kind is not None:
                         kwargs["mask_kind"] = kind
@@ -609,7 +686,7 @@ def fuse_attention(gm: fx.GraphModule) -> int:
             for node in r.biases:
                 b = _try_evaluate(node, gm) if not _placeholders_of(node) else None
                 if isinstance(b, torch.Tensor):
-                    if kwargs["alibi_heads"] == 0 and _is_alibi(b, Hq, L, S):
+                    if plain and kwargs["alibi_heads"] == 0 and _is_alibi(b, Hq, L, S):
                         kwargs["alibi_heads"] = Hq
                     else:
                         const_biases.append(b)

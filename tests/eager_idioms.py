@@ -140,3 +140,28 @@ def returns_weights(query, key, value):
     """Not fusable: the caller wants the attention weights as well."""
     w = torch.softmax(query @ key.transpose(-2, -1) * 0.125, dim=-1)
     return w @ value, w
+
+
+def relu_scores(query, key, value, causal=False):
+    """A score function other than the soft-cap (softcap.py:49 takes any callable): ReLU of the scaled scores."""
+    w = torch.relu(query @ key.transpose(-2, -1) / math.sqrt(query.size(-1)))
+    if causal:
+        w = w.masked_fill(torch.ones(w.size(-2), w.size(-1), dtype=torch.bool, device=w.device).triu(1), float("-inf"))
+    return torch.softmax(w, dim=-1) @ value
+
+
+def sigmoid_scores(query, key, value, bias):
+    w = torch.matmul(query, key.transpose(-2, -1)) * 0.25
+    w = 8.0 * torch.sigmoid(0.5 * w - 1.0) + bias
+    return torch.matmul(F.softmax(w, dim=-1), value)
+
+
+def clamped_scores(query, key, value):
+    w = (query @ key.transpose(-2, -1) * (1 / math.sqrt(query.size(-1)))).clamp(min=-2.0, max=3.0) * 2.0
+    return torch.softmax(w, dim=-1) @ value
+
+
+def squared_scores(query, key, value):
+    w = query @ key.transpose(-2, -1) * 0.125
+    w = -0.5 * w * w + w
+    return torch.softmax(w, dim=-1) @ value

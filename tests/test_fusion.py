@@ -91,6 +91,58 @@ def test_rewrite_recognises(name):
     assert list(calls[0].args[4]) == [] and list(calls[0].args[5]) == [] and calls[0].args[3] is None
 
 
+# name -> (function, number of extra tensor inputs, expected score_fn kind and constants, other expected kwargs)
+FN_CASES = {
+    "relu": (E.relu_scores, 0, (_ffi.SCORE_CLAMP, (1.0, 0.0, 0.0, float("inf"))), dict(mask_kind=_ffi.MASK_NONE)),
+    "relu causal": (functools.partial(E.relu_scores, causal=True), 0, (_ffi.SCORE_CLAMP, (1.0, 0.0, 0.0, float("inf"))),
+                    dict(mask_kind=_ffi.MASK_CAUSAL)),
+    "sigmoid + bias": (E.sigmoid_scores, 1, (_ffi.SCORE_SIGMOID, (0.5, -1.0, 8.0, 0.0)), dict(scale=0.25)),
+    "clamp": (E.clamped_scores, 0, (_ffi.SCORE_CLAMP, (2.0, 0.0, -4.0, 6.0)), dict()),
+    "polynomial": (E.squared_scores, 0, (_ffi.SCORE_POLY, (0.0, 1.0, -0.5, 0.0)), dict(scale=0.125)),
+}
+
+
+def _fn_extra(n, q, dev="cpu"):
+    g = torch.Generator().manual_seed(5)
+    return [torch.randn(q.size(1), q.size(2), q.size(2), generator=g).to(BF).to(dev) for _ in range(n)]
+
+
+@pytest.mark.parametrize("name", sorted(FN_CASES))
+def test_rewrite_recognises_score_functions(name):
+    # a ReLU, sigmoid, clamp or polynomial between the first matmul and the softmax becomes the kernel's score_fn: the
+    # chain is analysed like a caller's score_mod (the scale stays with the kernel's `scale` where it is a plain factor)
+    fn, n_extra, (kind, consts), want = FN_CASES[name]
+    q, k, v = _qkv()
+    gm, calls = _rewrite(fn, q, k, v, *_fn_extra(n_extra, q))
+    assert len(calls) == 1 and not _leftover(gm), gm.graph
+    kw = calls[0].kwargs
+    got_kind, got_consts = kw["score_fn"]
+    scale = kw["scale"]
+    assert got_kind == kind and kw["softcap"] == 0.0
+    # the analysis may leave the scale inside the function (scale 1) or outside: compare the composition on a grid
+    x = torch.linspace(-6, 6, 25, dtype=torch.float64)
+    want_scale = want.get("scale", 32 ** -0.5)
+
+    def apply(kind, c, z):
+        if kind == _ffi.SCORE_SIGMOID:
+            return c[2] * torch.sigmoid(c[0] * z + c[1]) + c[3]
+        if kind == _ffi.SCORE_CLAMP:
+            return torch.clamp(c[0] * z + c[1], min=c[2], max=c[3])
+        return c[0] + c[1] * z + c[2] * z ** 2 + c[3] * z ** 3
+    assert torch.allclose(apply(got_kind, got_consts, x * scale), apply(kind, consts, x * want_scale), atol=1e-9)
+    if "mask_kind" in want:
+        assert kw["mask_kind"] == want["mask_kind"]
+    assert len(calls[0].args[4]) == n_extra and list(calls[0].args[5]) == []
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(FN_CASES))
+def test_rewritten_score_functions_equal_eager_on_gpu(name):
+    fn, n_extra, _, _ = FN_CASES[name]
+    q, k, v = _qkv(N=2, Hq=4, Hkv=4, L=200, E=64, dev="cuda", seed=13)
+    _check_on_gpu(fn, (q, k, v, *_fn_extra(n_extra, q, "cuda")), name)
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("gqa", [False, True])
 def test_rewrite_recognises_document_masks_by_probing(causal, gqa):

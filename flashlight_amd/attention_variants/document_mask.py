@@ -11,7 +11,8 @@ from ._common import grouped_view, run
 
 def attention_pytorch_document_mask(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                     document_id: torch.Tensor, scale=None, enable_gqa=False, *,
-                                    is_causal: bool = False, workspace: "_ffi.DocWorkspace | None" = None) -> torch.Tensor:
+                                    is_causal: bool = False, workspace: "_ffi.DocWorkspace | None" = None,
+                                    dropout_p: float = 0.0) -> torch.Tensor:
     """document_mask.py:6-41: `document_id` is an integer tensor [N, L]; q attends k iff document_id[n, q] ==
     document_id[n, k] (both directions inside a document).  The ids may be any integers in any order; sorted ids let
     the kernel skip whole key tiles.
@@ -21,12 +22,15 @@ def attention_pytorch_document_mask(query: torch.Tensor, key: torch.Tensor, valu
 
     workspace (not in the reference): a `DocumentMaskWorkspace()` handle.  Calls that pass the same handle with the
     same `document_id` tensor and shapes derive the key tiles each query tile visits once instead of on every call, as
-    that baseline builds its block mask once for all layers (run_flex_variants.py:66-90)."""
+    that baseline builds its block mask once for all layers (run_flex_variants.py:66-90).
+
+    dropout_p (not in the reference): dropout on the softmax weights, applied once `honor_dropout(True)` has been
+    called, like the `dropout_p` of the causal, ALiBi and soft-cap variants."""
     if document_id.dim() != 2:
         raise ValueError(f"document_id must be [N, L], got {tuple(document_id.shape)}")
     kind = _ffi.MASK_DOCUMENT_CAUSAL if is_causal else _ffi.MASK_DOCUMENT
     out = run(query, key, value, scale=scale, enable_gqa=enable_gqa, mask_kind=kind, doc_ids=document_id,
-              doc_workspace=workspace)
+              doc_workspace=workspace, dropout_p=dropout_p)
     return grouped_view(out, key, enable_gqa)
 
 

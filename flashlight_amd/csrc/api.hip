@@ -348,9 +348,11 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   if (p->dropout_threshold) {
     if (p->dropout_threshold > 65535u)
       return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
-    if (is_doc(p->mask_kind) || p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
-      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional masks, ALiBi and the soft-cap only (no document mask, "
-                                      "bias, gate, differential attention, dump)");
+    if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
+      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional and document masks, ALiBi and the soft-cap only (no bias, "
+                                      "gate, differential attention, dump)");
+    if (is_doc(p->mask_kind) && (p->alibi_heads > 0 || p->softcap > 0.f))
+      return fail(FL_ERR_UNSUPPORTED, "dropout under a document mask is built without ALiBi and the soft-cap");
   }
   if (p->lse) {
     if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
@@ -791,7 +793,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   uint32_t want = 0;
   if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
   if (is_doc(p->mask_kind)) want |= fl::F_DOC;
-  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() has excluded document masks
+  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() allows a document mask or ALiBi / soft-cap, not both
   if (has_bias) want = fl::F_BIAS;
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)

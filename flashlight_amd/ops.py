@@ -287,7 +287,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         return out[..., :v.size(-1)]
     if dropout_p > 0.0:
         if biases or gate is not None or diff or seq_major_out:
-            raise NotImplementedError("dropout is built for positional masks, the in-kernel ALiBi term and the soft-cap; not "
+            raise NotImplementedError("dropout is built for positional and document masks, the in-kernel ALiBi term and the soft-cap; not "
                                       "for bias operands, the gate or differential attention")
         if dropout_seed is None:
             if torch.compiler.is_compiling():

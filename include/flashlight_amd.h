@@ -120,8 +120,9 @@ typedef struct fl_attn_params {
    * ignore it (attention_variants/causal.py:4-36, alibi.py:13-33, softcap.py:4-53); 0 here does the same.
    * dropout_threshold = round(p * 65536), 1 .. 65535: a weight is dropped when the 16 bits a counter-based hash of
    * (dropout_seed, batch * Hq + head, query, key) gives it are below the threshold.  fl_attn_bwd regenerates the same
-   * decisions from the same fields.  With positional masks, GQA, ALiBi and the soft-cap; not with document masks, bias
-   * operands, gate, differential attention or the dump hook; Dqk = Dv in {64, 128}. */
+   * decisions from the same fields.  With positional masks, GQA, ALiBi and the soft-cap, or with a document mask (then
+   * without ALiBi and the soft-cap); not with bias operands, gate, differential attention or the dump hook;
+   * Dqk = Dv in {64, 128}. */
   uint32_t dropout_threshold;
   uint32_t dropout_seed[2]; /* low, high half of a 64-bit seed */
 

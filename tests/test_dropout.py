@@ -163,7 +163,16 @@ def test_abi_validation_of_dropout_fields():
         p.dropout_threshold = 100
         mutate(p)
         assert rc(p) == 0, _ffi.last_error()
-    for mutate in (lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000)),
+    for kind in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):  # a document mask alone goes with dropout
+        p = good_params()
+        p.dropout_threshold = 100
+        p.mask_kind, p.doc_ids = kind, 0x50000
+        p.workspace, p.workspace_bytes = 0x80000, lib.fl_workspace_bytes(C.byref(p))
+        assert rc(p) == 0, _ffi.last_error()
+    doc = lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000),  # noqa: E731
+                     setattr(p, "workspace", 0x80000), setattr(p, "workspace_bytes", lib.fl_workspace_bytes(C.byref(p))))
+    for mutate in (lambda p: (doc(p), setattr(p, "alibi_heads", 4)),
+                   lambda p: (doc(p), setattr(p, "softcap", 30.0)),
                    lambda p: setattr(p, "diff", 1)):
         p = good_params()
         p.dropout_threshold = 100
@@ -276,6 +285,58 @@ def test_dropout_with_alibi_and_softcap(D, alibi, softcap):
     for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
         scale = max(1.0, want.abs().max().item())
         assert_parity(got.float() / scale, want / scale, f"{what} with dropout and score modifications")
+
+
+def _document_ids(B, L, lengths, shuffle_seed=None):
+    ids = torch.repeat_interleave(torch.arange(len(lengths)), torch.tensor(lengths))[:L]
+    ids = torch.cat([ids, ids.new_full((L - ids.numel(),), len(lengths))])
+    rows = []
+    for b in range(B):
+        row = (ids + 3 * b) * 7 - 11  # any integers, not 0..n
+        if shuffle_seed is not None:  # unsorted ids: same-document positions scattered over the sequence
+            row = row[torch.randperm(L, generator=torch.Generator().manual_seed(shuffle_seed + b))]
+        rows.append(row)
+    return torch.stack(rows).to(torch.int64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("causal,shuffled", [(False, False), (True, False), (False, True)])
+def test_dropout_under_a_document_mask(D, causal, shuffled):
+    B, Hq, Hkv, L = 2, 4, 2, 391
+    q, k, v, dout = _gpu_inputs(B, Hq, Hkv, L, L, D, seed=D + 31 * causal + 5 * shuffled)
+    ids = _document_ids(B, L, [70, 1, 129, 64, 100], shuffle_seed=17 if shuffled else None)
+    p, seed = 0.15, 0x5EED0000DEADBEEF >> 1
+    kind = _ffi.MASK_DOCUMENT_CAUSAL if causal else _ffi.MASK_DOCUMENT
+    kw = dict(mask_kind=kind, doc_ids=ids.to(DEV), dropout_p=p, dropout_seed=seed)
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, **kw)
+    torch.cuda.synchronize()
+    attend = (ids[:, :, None] == ids[:, None, :])[:, None]  # [B, 1, L, L]
+    if causal:
+        attend = attend & (torch.arange(L)[None, :] <= torch.arange(L)[:, None])
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    ref = OD.attention_dropout(qf, kf, vf, OD.keep_mask(seed, B, Hq, L, L, p), p, attend=attend)
+    ref.backward(dout.float().cpu())
+    assert_parity(out, ref, "forward with dropout under a document mask")
+    for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{what} with dropout under a document mask")
+    # the dropped weights are the ones the positional-mask kernels drop for the same seed: one document gives the
+    # unmasked / causal call's result
+    one = torch.zeros(B, L, dtype=torch.int64, device=DEV)
+    a = _ffi.attn_fwd(q, k, v, mask_kind=kind, doc_ids=one, dropout_p=p, dropout_seed=seed)
+    b = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL if causal else _ffi.MASK_NONE, dropout_p=p, dropout_seed=seed)
+    assert_parity(a, b.float().cpu(), "one document against the positional mask")
+    # the variant function takes dropout_p once the switch is on
+    with A.honor_dropout():
+        torch.manual_seed(5)
+        x = A.attention_pytorch_document_mask(q, k, v, ids.to(DEV), enable_gqa=True, is_causal=causal, dropout_p=p)
+        torch.manual_seed(5)
+        y = A.attention_pytorch_document_mask(q, k, v, ids.to(DEV), enable_gqa=True, is_causal=causal, dropout_p=p)
+    z = A.attention_pytorch_document_mask(q, k, v, ids.to(DEV), enable_gqa=True, is_causal=causal, dropout_p=p)
+    assert torch.equal(x, y) and not torch.equal(x, z)
 
 
 @pytest.mark.gpu

@@ -233,7 +233,7 @@ _HEAD_DIMS = (32, 64, 128)
 
 def _pad_head_dims(q, k, v, gate, diff):
     """(q, k, v, gate) with zero columns appended up to a compiled head dim, or None when the head dims are compiled as
-    they are (32, 64, 128 for q, k and v alike; 256 for q and k with values in slabs of 128 columns; the 64/128 and
+    they are (32, 64, 128 for q, k and v alike; 256 and 512 for q and k with values in slabs of 128 columns; the 64/128 and
     128/256 pairs of differential attention) or when no padding would help."""
     dqk, dv = q.shape[-1], v.shape[-1]
     if not diff and dqk == dv and dqk in _HEAD_DIMS:
@@ -248,9 +248,9 @@ def _pad_head_dims(q, k, v, gate, diff):
     elif (dqk, dv) in ((32, 64), (64, 128)):
         return None  # compiled pairs (invariant point attention's channel counts land on them)
     elif dqk > 128 or dv > 128:
-        if dqk > 256:
+        if dqk > 512:
             return None
-        pq, pv = (256 if dqk > 128 else 128), -(-dv // 128) * 128
+        pq, pv = (128 if dqk <= 128 else 256 if dqk <= 256 else 512), -(-dv // 128) * 128
     else:
         pq = pv = next(p for p in _HEAD_DIMS if p >= max(dqk, dv))
     if (pq, pv) == (dqk, dv):
@@ -276,7 +276,8 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     padded = _pad_head_dims(q, k, v, gate, diff)
     if padded is not None:
         # head dims between the compiled ones: zero columns change neither q.k nor the columns of the result that are
-        # kept (the reference's generated kernel takes any head dim up to 256, monkeypatch/fusion/_common.py:4)
+        # kept (the reference's generated kernel takes any head dim up to 256 in one block, monkeypatch/fusion/_common.py:4,
+        # and loops over wider ones, monkeypatch/fusion/reduction_kernel_fusion.py:1102; here up to 512)
         qp, kp, vp, gp = padded
         if scale is None:
             scale = 1.0 / math.sqrt(q.size(-1))

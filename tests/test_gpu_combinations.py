@@ -75,6 +75,44 @@ def test_head_dim_256_row_statistics_come_from_the_first_slab():
     assert (lse.cpu() - ref).abs().max().item() < 2e-2
 
 
+@pytest.mark.parametrize("D,Dv,S", [(512, 128, 1), (512, 512, 333), (320, 320, 200), (384, 64, 1024), (512, 256, 97)])
+def test_head_dims_up_to_512(D, Dv, S):
+    """Head dims above 256 run on the 512-wide instances (one wave per SIMD); widths in between are zero-padded.  The
+    reference's generated kernel loops over the head dim there (monkeypatch/fusion/reduction_kernel_fusion.py:1102)."""
+    q, k, v = qkv(2, 4, 2, S, D, Dv, seed=S + D + Dv)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch(q, k, v, enable_gqa=True), O.attention_vanilla(qf, kf, vf, enable_gqa=True), "vanilla")
+    assert_parity(A.attention_pytorch_causal(q, k, v, enable_gqa=True), O.attention_causal(qf, kf, vf, enable_gqa=True),
+                  "causal")
+    assert_parity(A.attention_pytorch_sliding_window(q, k, v, window_size=33, enable_gqa=True),
+                  O.attention_sliding_window(qf, kf, vf, window_size=33, enable_gqa=True), "sliding")
+    assert_parity(A.attention_pytorch_prefix_lm(q, k, v, prefix_lengths=50, enable_gqa=True),
+                  O.attention_prefix_lm(qf, kf, vf, prefix_lengths=50, enable_gqa=True), "prefix")
+
+
+def test_head_dim_512_score_mods_documents_and_fp16():
+    S = 450
+    q, k, v = qkv(2, 4, 4, S, 512, 256, seed=15, amp=3.0)
+    qf, kf, vf = f32(q, k, v)
+    assert_parity(A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(4)),
+                  O.attention_alibi(qf, kf, vf, score_mod=4), "alibi")
+    assert_parity(A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(20.0)),
+                  O.attention_softcapped(qf, kf, vf, score_mod=20.0), "softcap")
+    assert_parity(A.attention_pytorch_alibi(q, k, v, score_mod=A.generate_alibi_bias_pytorch(4), is_causal=True, softcap=15.0),
+                  O.attention_alibi(qf, kf, vf, score_mod=4, is_causal=True, honor_causal=True, softcap=15.0),
+                  "alibi+softcap+causal")
+    g = torch.Generator().manual_seed(16)
+    ids = torch.sort(torch.randint(0, 5, (2, S), generator=g), dim=1).values
+    for causal in (False, True):
+        assert_parity(A.attention_pytorch_document_mask(q, k, v, ids.to(DEV), is_causal=causal),
+                      O.attention_document_mask(qf, kf, vf, ids, is_causal=causal), f"document causal={causal}")
+    h = tuple(t.to(torch.float16) for t in (q / 3.0, k, v))
+    assert_parity(A.attention_pytorch_causal(*h), O.attention_causal(*f32(*h)), "fp16 causal")
+    with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
+        big = torch.zeros(1, 1, 8, 520, dtype=torch.bfloat16, device=DEV)
+        A.attention_pytorch(big, big, big)
+
+
 def _doc_alibi_oracle(qf, kf, vf, ids, nheads, cap, causal):
     """Eager fp32 composition: cap * tanh(q k^T s / cap) + slope_h (k - q), masked where the ids differ (or k > q)."""
     slopes = alibi_slopes(nheads).float().view(1, nheads, 1, 1)

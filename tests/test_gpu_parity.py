@@ -270,9 +270,9 @@ def test_front_end_errors_on_gpu_tensors():
     q48 = torch.randn(1, 2, 64, 48, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
         _ffi.attn_fwd(q48, q48, q48)  # the C ABI takes compiled head dims only (the front-ends pad others)
-    q320 = torch.randn(1, 2, 64, 320, device=DEV, dtype=torch.bfloat16)
+    q640 = torch.randn(1, 2, 64, 640, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(_ffi.FlashlightError, match="no kernel instance"):
-        A.attention_pytorch(q320, q320, q320)  # beyond 256
+        A.attention_pytorch(q640, q640, q640)  # beyond 512
 
 
 def test_mfma_rate_probe_runs_and_sums_products():

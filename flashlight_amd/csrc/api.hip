@@ -348,11 +348,13 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
   if (p->dropout_threshold) {
     if (p->dropout_threshold > 65535u)
       return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
-    if (p->bias[0] || p->bias[1] || p->gate || p->diff || p->attended_dump)
-      return fail(FL_ERR_UNSUPPORTED, "dropout is built for positional and document masks, ALiBi and the soft-cap only (no bias, "
-                                      "gate, differential attention, dump)");
-    if (is_doc(p->mask_kind) && (p->alibi_heads > 0 || p->softcap > 0.f))
-      return fail(FL_ERR_UNSUPPORTED, "dropout under a document mask is built without ALiBi and the soft-cap");
+    if (p->diff || p->attended_dump)
+      return fail(FL_ERR_UNSUPPORTED, "dropout is not built for differential attention and the dump hook");
+    const bool dense = p->bias[0] || p->bias[1] || p->gate;
+    const bool mods = p->alibi_heads > 0 || p->softcap > 0.f;
+    if ((is_doc(p->mask_kind) && (mods || dense)) || (mods && dense))
+      return fail(FL_ERR_UNSUPPORTED, "dropout is built with one of: ALiBi and / or the soft-cap, a document mask, bias operands "
+                                      "and / or the gate (each under any positional mask), not with two of them");
   }
   if (p->lse) {
     if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
@@ -768,8 +770,8 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
   if (p->score_fn != FL_SCORE_NONE) return fail(FL_ERR_UNSUPPORTED, "backward: score_fn is forward-only");
   const bool has_bias = p->bias[0] || p->bias[1];
-  if (has_bias && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind) || p->dropout_threshold))
-    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands go with positional masks only (no ALiBi, soft-cap, document mask or dropout)");
+  if (has_bias && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind)))
+    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands go with positional masks (and dropout) only: no ALiBi, soft-cap or document mask");
   if (b->dscores && !has_bias) return fail(FL_ERR_ARG, "backward: dscores is only written for calls with bias operands");
   if (b->dscores && reinterpret_cast<uintptr_t>(b->dscores) % 16) return fail(FL_ERR_ALIGN, "backward: dscores must be 16-byte aligned");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
@@ -793,8 +795,8 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   uint32_t want = 0;
   if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
   if (is_doc(p->mask_kind)) want |= fl::F_DOC;
-  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() allows a document mask or ALiBi / soft-cap, not both
   if (has_bias) want = fl::F_BIAS;
+  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() allows one of document mask, ALiBi / soft-cap, bias operands
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)

@@ -120,8 +120,8 @@ typedef struct fl_attn_params {
    * ignore it (attention_variants/causal.py:4-36, alibi.py:13-33, softcap.py:4-53); 0 here does the same.
    * dropout_threshold = round(p * 65536), 1 .. 65535: a weight is dropped when the 16 bits a counter-based hash of
    * (dropout_seed, batch * Hq + head, query, key) gives it are below the threshold.  fl_attn_bwd regenerates the same
-   * decisions from the same fields.  With positional masks, GQA, ALiBi and the soft-cap, or with a document mask (then
-   * without ALiBi and the soft-cap); not with bias operands, gate, differential attention or the dump hook;
+   * decisions from the same fields.  With any positional mask and GQA, together with one of: ALiBi and / or the soft-cap;
+   * a document mask; bias operands and / or the gate.  Not with two of these, differential attention or the dump hook;
    * Dqk = Dv in {64, 128}. */
   uint32_t dropout_threshold;
   uint32_t dropout_seed[2]; /* low, high half of a 64-bit seed */
@@ -193,7 +193,7 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
  * kind, grouped-query heads, ALiBi, the tanh soft-cap (either of them under a document mask at head dims 64 and 128);
  * Dqk == Dv in {32, 64, 128}.  Bias operands (fwd.bias, as in the
- * forward) go with positional masks only, not with ALiBi, a soft-cap, a document mask or dropout.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
+ * forward) go with positional masks and dropout only, not with ALiBi, a soft-cap or a document mask.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
  * (both are compositions of calls that are supported: out * sigmoid(gate); one call per branch and half of the value
  * columns), the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]

@@ -87,7 +87,7 @@ def test_backward_abi_validation():
         (lambda b: setattr(b, "dout", 0xA0008), -7, "dout"),
         (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),
         (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
-                    setattr(b.fwd, "softcap", 30.0)), -4, "positional masks only"),
+                    setattr(b.fwd, "softcap", 30.0)), -4, "positional masks"),
         (lambda b: setattr(b, "dscores", 0xF0000), -5, "dscores"),
         (lambda b: (setattr(b.fwd, "gate", 0x70000), b.fwd.gate_strides.__setitem__(slice(0, 4), list(b.fwd.o_strides))),
          -4, "not supported"),

@@ -171,8 +171,20 @@ def test_abi_validation_of_dropout_fields():
         assert rc(p) == 0, _ffi.last_error()
     doc = lambda p: (setattr(p, "mask_kind", _ffi.MASK_DOCUMENT), setattr(p, "doc_ids", 0x50000),  # noqa: E731
                      setattr(p, "workspace", 0x80000), setattr(p, "workspace_bytes", lib.fl_workspace_bytes(C.byref(p))))
+    def dense(p):
+        p.bias[0], p.bias_batch_div[0] = 0x60000, 1
+        p.bias_strides[0][:] = (0, 0, p.Lk, 1)
+
+    for mutate in (dense, lambda p: (dense(p), setattr(p, "mask_kind", _ffi.MASK_CAUSAL)),
+                   lambda p: (setattr(p, "gate", 0x70000), p.gate_strides.__setitem__(slice(0, 4), list(p.o_strides)))):
+        p = good_params()
+        p.dropout_threshold = 100
+        mutate(p)
+        assert rc(p) == 0, _ffi.last_error()
     for mutate in (lambda p: (doc(p), setattr(p, "alibi_heads", 4)),
                    lambda p: (doc(p), setattr(p, "softcap", 30.0)),
+                   lambda p: (doc(p), dense(p)),
+                   lambda p: (dense(p), setattr(p, "softcap", 30.0)),
                    lambda p: setattr(p, "diff", 1)):
         p = good_params()
         p.dropout_threshold = 100
@@ -193,7 +205,11 @@ def test_front_end_switch_and_refusals():
         A.attention_pytorch_causal(q, q, q, dropout_p=0.5)
     assert "dropout" not in str(e.value)
     with pytest.raises(NotImplementedError, match="dropout"):
-        ops.dispatch(q, q, q, dropout_p=0.1, gate=q)
+        ops.dispatch(q, q, q, dropout_p=0.1, diff=True)
+    with pytest.raises(NotImplementedError, match="dropout"):  # bias operands or the gate: not with ALiBi / soft-cap / ids
+        ops.dispatch(q, q, q, dropout_p=0.1, gate=q, softcap=5.0)
+    with pytest.raises(NotImplementedError, match="dropout"):
+        ops.dispatch(q, q, q, dropout_p=0.1, biases=[(torch.zeros(1, 1, 8, 8), 1)], alibi_heads=2)
     with pytest.raises(ValueError, match="dropout_p"):
         ops.dispatch(q, q, q, dropout_p=1.5)
     with A.honor_dropout():
@@ -340,6 +356,57 @@ def test_dropout_under_a_document_mask(D, causal, shuffled):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("mask_kind", [_ffi.MASK_NONE, _ffi.MASK_CAUSAL])
+def test_dropout_with_bias_operands_and_the_gate(D, mask_kind):
+    """A dense additive term per head (shared by the batch: a relative-position table) and a row-broadcast fp32 term, with
+    dropout: forward, gradients of q, k, v and the score gradient the bias gradients are summed from."""
+    B, Hq, Hkv, L, S = 2, 4, 2, 210, 275
+    q, k, v, dout = _gpu_inputs(B, Hq, Hkv, L, S, D, seed=D + mask_kind)
+    g = torch.Generator().manual_seed(D)
+    table = torch.randn(1, Hq, L, S, generator=g).to(torch.bfloat16).to(DEV)
+    rowb = (torch.randn(B, 1, 1, S, generator=g) * 2).to(DEV)
+    p, seed = 0.2, 0x0123456789ABCDE
+    kw = dict(mask_kind=mask_kind, biases=[(table, 1), (rowb, 1)], dropout_p=p, dropout_seed=seed)
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+    dscores = torch.zeros(B, Hq, L, S, dtype=torch.float32, device=DEV)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, dscores=dscores, **kw)
+    torch.cuda.synchronize()
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    bias = (table.float().cpu() + rowb.cpu()).requires_grad_(True)
+    ref = OD.attention_dropout(qf, kf, vf, OD.keep_mask(seed, B, Hq, L, S, p), p, attend=_attend(mask_kind, L, S), bias=bias)
+    ref.backward(dout.float().cpu())
+    assert_parity(out, ref, "forward with bias operands and dropout")
+    for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad), ("dscores", dscores, bias.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{what} with bias operands and dropout")
+    # the gate multiplies the result, whatever was dropped
+    gate = torch.randn(B, Hq, L, D, generator=g).to(torch.bfloat16).to(DEV)
+    gated = _ffi.attn_fwd(q, k, v, gate=gate, **kw)
+    assert_parity(gated, ref.detach() * torch.sigmoid(gate.float().cpu()), "gate with dropout")
+    plain = _ffi.attn_fwd(q, k, v, gate=gate, mask_kind=mask_kind, dropout_p=p, dropout_seed=seed)
+    ref0 = OD.attention_dropout(qf.detach(), kf.detach(), vf.detach(), OD.keep_mask(seed, B, Hq, L, S, p), p,
+                                attend=_attend(mask_kind, L, S))
+    assert_parity(plain, ref0 * torch.sigmoid(gate.float().cpu()), "gate with dropout, no bias")
+    # through autograd: bias gradients are the score gradient summed over what the operand broadcasts over
+    qg, kg, vg, tg, rg = (t.detach().clone().requires_grad_(True) for t in (q, k, v, table, rowb))
+    o = ops.dispatch(qg, kg, vg, mask_kind=mask_kind, biases=[(tg, 1), (rg, 1)], gate=gate, dropout_p=p, dropout_seed=seed)
+    o.backward(dout)
+    sg = torch.sigmoid(gate.float().cpu())
+    qf2, kf2, vf2 = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    tf, rf = table.float().cpu().requires_grad_(True), rowb.cpu().requires_grad_(True)
+    r2 = OD.attention_dropout(qf2, kf2, vf2, OD.keep_mask(seed, B, Hq, L, S, p), p, attend=_attend(mask_kind, L, S),
+                              bias=tf + rf) * sg
+    r2.backward(dout.float().cpu())
+    assert_parity(o, r2, "autograd forward with bias operands, gate and dropout")
+    for what, got, want in (("dq", qg.grad, qf2.grad), ("dtable", tg.grad, tf.grad), ("drow", rg.grad, rf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"autograd {what} with bias operands, gate and dropout",
+                      max_tol=3e-2)
+
+
+@pytest.mark.gpu
 def test_dropout_fp16_forward_and_determinism():
     q, k, v, _ = _gpu_inputs(1, 2, 2, 192, 192, 128, seed=3)
     q, k, v = (t.to(torch.float16) for t in (q, k, v))
@@ -366,9 +433,12 @@ def test_dropout_through_autograd_and_the_variant_switch():
         b = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
         c = A.attention_pytorch_causal(q, k, v, dropout_p=0.5, enable_gqa=True)
         assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a, base)
-        with pytest.raises(NotImplementedError, match="dropout"):  # a dense score_mod tensor goes through the bias path
-            A.attention_pytorch_alibi(q, k, v, score_mod=lambda L, S: torch.zeros(4, L, S, device=DEV), dropout_p=0.1,
-                                      enable_gqa=True)
+        dense = lambda L, S: torch.zeros(4, L, S, device=DEV)  # noqa: E731  (a dense score_mod tensor: the bias path)
+        torch.manual_seed(11)
+        d = A.attention_pytorch_alibi(q, k, v, score_mod=dense, dropout_p=0.5, enable_gqa=True, is_causal=True)
+        assert torch.equal(d, a)  # a zero bias and the same seed: the same weights are dropped
+        with pytest.raises(NotImplementedError, match="dropout"):  # not together with the soft-cap
+            A.attention_pytorch_alibi(q, k, v, score_mod=dense, dropout_p=0.1, enable_gqa=True, softcap=5.0)
     # autograd: the backward regenerates the forward's decisions from the seed
     qg, kg, vg = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
     out = ops.dispatch(qg, kg, vg, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.3, dropout_seed=2024)

@@ -483,7 +483,7 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   const int64_t worst = std::max(std::max(p->q_strides[2], p->o_strides[2]), p->gate ? p->gate_strides[2] : 0);
   if (((int64_t)p->Lq * worst + 64) * 2 >= ((int64_t)1 << 31)) return false;
   // ... and so are those inside one key tile of 64 rows
-  if ((64 * std::max(p->k_strides[2], p->v_strides[2]) + 32) * 2 >= ((int64_t)1 << 31)) return false;
+  if ((64 * std::max(p->k_strides[2], p->v_strides[2]) + p->Dqk) * 2 >= ((int64_t)1 << 31)) return false;
   // the selector weight 1 / scale must be an ordinary number in the element type (bf16 shares fp32's range; fp16 ends at
   // 65504 and loses precision below 2^-14)
   {

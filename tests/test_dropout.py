@@ -406,6 +406,77 @@ def test_dropout_with_bias_operands_and_the_gate(D, mask_kind):
                       max_tol=3e-2)
 
 
+def _random_dropout_case(seed):
+    import random
+    rnd = random.Random(seed)
+    D = rnd.choice([64, 128])
+    Hkv, G, B = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 4]), rnd.choice([1, 2])
+    L = rnd.choice([1, 33, 64, 100, 129, 200, 257, 384, 450])
+    S = L if rnd.random() < 0.6 else rnd.choice([17, 64, 150, 300])
+    family = rnd.choice(["plain", "mods", "document", "bias"])
+    mask_kind = rnd.choice([_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM])
+    if mask_kind in (_ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM):
+        S = L  # (as in the reference: these masks are defined for equal lengths)
+    if family == "document":
+        S = L
+        mask_kind = rnd.choice([_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL])
+    return dict(seed=seed, D=D, Hkv=Hkv, G=G, B=B, L=L, S=S, family=family, mask_kind=mask_kind,
+                window=rnd.choice([1, 31, 70, 128]), prefix=rnd.choice([1, 32, 50, 129]), p=rnd.choice([0.05, 0.3, 0.7]),
+                alibi=rnd.random() < 0.6, cap=rnd.choice([None, 4.0, 25.0]), ndocs=rnd.choice([1, 3, 7]),
+                fp16=rnd.random() < 0.25)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(500, 540))
+def test_random_dropout_cases(seed):
+    """Seeded draws over the families the dropout kernels are built for (positional masks alone, with ALiBi / soft-cap,
+    document masks, bias operands), ragged and unequal lengths, grouped heads, both element types: forward and
+    gradients against autograd through the oracle with the same seed."""
+    import oracle as O
+    c = _random_dropout_case(seed)
+    B, Hkv, Hq, L, S, D, p = c["B"], c["Hkv"], c["Hkv"] * c["G"], c["L"], c["S"], c["D"], c["p"]
+    dt = torch.float16 if c["fp16"] else torch.bfloat16
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dt).to(DEV)  # noqa: E731
+    q, k, v, dout = mk(B, Hq, L, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, L, D)
+    kw = dict(mask_kind=c["mask_kind"], window=c["window"], prefix=c["prefix"], dropout_p=p, dropout_seed=seed * 0x9E3779B97F4A7 + 1)
+    attend = _attend(c["mask_kind"], L, S, c["window"], c["prefix"])
+    bias, cap, operand = None, None, None
+    if c["family"] == "mods":
+        cap = c["cap"]
+        if c["alibi"] or cap is None:
+            rel = (torch.arange(S)[None, :] - torch.arange(L)[:, None]).float()
+            bias = O.alibi_slopes(Hq)[:, None, None] * rel[None]
+            kw["alibi_heads"] = Hq
+        kw["softcap"] = cap or 0.0
+    elif c["family"] == "document":
+        ids = torch.sort(torch.randint(0, c["ndocs"], (B, L), generator=g), dim=1).values
+        if seed % 3 == 0:
+            ids = ids[:, torch.randperm(L, generator=g)]
+        kw["doc_ids"] = ids.to(DEV)
+        attend = (ids[:, :, None] == ids[:, None, :])[:, None]
+        if c["mask_kind"] == _ffi.MASK_DOCUMENT_CAUSAL:
+            attend = attend & (torch.arange(L)[None, :] <= torch.arange(L)[:, None])
+    elif c["family"] == "bias":
+        operand = torch.randn(1, Hq, L, S, generator=g).to(dt).to(DEV)
+        kw["biases"] = [(operand, 1)]
+        bias = operand.float().cpu()
+    lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
+    dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, **kw)
+    torch.cuda.synchronize()
+    qf, kf, vf = (t.float().cpu().requires_grad_(True) for t in (q, k, v))
+    ref = OD.attention_dropout(qf, kf, vf, OD.keep_mask(kw["dropout_seed"], B, Hq, L, S, p), p, attend=attend, bias=bias,
+                               softcap=cap)
+    ref.backward(dout.float().cpu())
+    # kept weights are scaled by 1 / (1 - p): the tolerances scale with it
+    f = 1.0 / (1.0 - p)
+    assert_parity(out.float() / f, ref / f, f"forward {c}")
+    for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        scale = max(1.0, want.abs().max().item())
+        assert_parity(got.float() / scale, want / scale, f"{what} {c}")
+
+
 @pytest.mark.gpu
 def test_dropout_fp16_forward_and_determinism():
     q, k, v, _ = _gpu_inputs(1, 2, 2, 192, 192, 128, seed=3)

@@ -21,7 +21,10 @@ Masks and biases are recognised by what they compute, not by how they were writt
     bias at run time;
   * a constant bias equal to 2^(-8 (h + 1) / H) * (k - q) is ALiBi and is computed inside the kernel; other biases are
     passed to the kernel's bias operands (fp32 or bf16).
-Regions that do not fit (a softmax whose weights are used elsewhere, dropout with p > 0, ...) are left untouched.
+A training-mode dropout on the softmax weights becomes the kernel's own dropout (same rate, the kernel's random
+stream, a fresh seed per call) where the dropout kernels cover the region: one of ALiBi / soft-cap, a document mask or
+dense operands, head dims 33 .. 128.  Regions that do not fit (a softmax whose weights are used elsewhere, dropout
+outside that coverage, ...) are left untouched.
 """
 from __future__ import annotations
 
@@ -269,12 +272,16 @@ def _kernel_bias(b: torch.Tensor, lead: Tuple[int, ...], heads: Tuple[int, ...],
 def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: Optional[torch.Tensor],
                     biases: Sequence[torch.Tensor], masks: Sequence[torch.Tensor], *, scale: float, mask_kind: int,
                     window: int, prefix: int, alibi_heads: int, softcap: float, gqa: bool,
-                    mask_invert: Sequence[bool] = (), diff_lambda: Optional[float] = None, score_fn=None) -> torch.Tensor:
+                    mask_invert: Sequence[bool] = (), diff_lambda: Optional[float] = None, score_fn=None,
+                    dropout_p: float = 0.0) -> torch.Tensor:
     """Target of the replacement node.  q [*lead, H, L, E] (or [N, Hkv, G, L, E] with `gqa`), k/v likewise with S keys;
     `biases` are added to the scaled scores, `masks` (bool, True = masked unless the matching `mask_invert` entry is
     set) are those the rewrite could not map to a positional or document mask.  Returns what the eager region
     returned: [*q.shape[:-1], Ev].  With `diff_lambda` q and k hold the heads of both softmax branches (first half,
-    second half) and the result is branch 0 minus diff_lambda times branch 1."""
+    second half) and the result is branch 0 minus diff_lambda times branch 1.  `dropout_p` > 0 (a training-mode dropout
+    on the softmax weights in the eager region) drops weights inside the kernel; each call draws its seed from torch's
+    default CPU generator, so `torch.manual_seed` reproduces a run, but the weights dropped are not the ones
+    `torch.nn.functional.dropout` would have dropped for that seed."""
     L, S = q.size(-2), k.size(-2)
     result_shape = (*q.shape[:-1], v.size(-1))
     if gqa:
@@ -307,7 +314,7 @@ def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: 
         kb[-2:] = [(b1.float() + b2.float(), d1)]
     if diff_lambda is None:
         out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
-                           alibi_heads=alibi_heads, softcap=softcap, biases=kb, score_fn=score_fn)
+                           alibi_heads=alibi_heads, softcap=softcap, biases=kb, score_fn=score_fn, dropout_p=dropout_p)
         return out.reshape(result_shape)
     out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                        alibi_heads=alibi_heads, softcap=softcap, biases=kb, diff=True, lambda_full=float(diff_lambda))
@@ -323,6 +330,7 @@ class _Region:
         self.scale = 1.0
         self.softcap = 0.0
         self.score_fn = None                 # (kind, four constants) of fl_attn_params.score_fn
+        self.dropout_p = 0.0                 # rate of a training-mode dropout between the softmax and the second matmul
         self.biases: List[fx.Node] = []
         self.masks: List[Tuple[fx.Node, bool]] = []   # (mask node, invert)
         self.out: Optional[fx.Node] = None
@@ -537,9 +545,13 @@ def _match(softmax: fx.Node) -> _Region:
             cur = u
             continue
         if nm == "dropout":
-            p = _arg(u, 1, "p", 0.5)
-            if p != 0.0:
-                raise _NoMatch("dropout with p > 0")
+            p, training = _arg(u, 1, "p", 0.5), _arg(u, 2, "training", True)
+            if not _is_number(p) or not isinstance(training, bool) or not 0.0 <= float(p) < 1.0:
+                raise _NoMatch("dropout with a rate or mode that is not a constant")
+            if training and float(p) > 0.0:
+                if r.dropout_p:
+                    raise _NoMatch("two dropouts on the softmax weights")
+                r.dropout_p = float(p)
             tail.append(u)
             cur = u
             continue
@@ -613,7 +625,8 @@ def _merge_differential(gm: fx.GraphModule) -> int:
             continue
         if not all(x.op == "call_function" and x.target is fused_attention for x in (a, b)):
             continue
-        if a.kwargs != b.kwargs or a.kwargs.get("gqa") or a.kwargs.get("diff_lambda") is not None or a.kwargs.get("score_fn"):
+        if a.kwargs != b.kwargs or a.kwargs.get("gqa") or a.kwargs.get("diff_lambda") is not None or a.kwargs.get("score_fn") \
+                or a.kwargs.get("dropout_p"):
             continue
         if a.args[2] is not b.args[2] or a.args[3] is not b.args[3]:
             continue
@@ -692,6 +705,14 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                         const_biases.append(b)
                 else:
                     run_biases.append(node)
+            if r.dropout_p:
+                # the dropout kernels cover one family at a time and head dims that are (or pad to) 64 or 128
+                families = [bool(kwargs["alibi_heads"] or r.softcap), doc_ids is not None,
+                            bool(run_masks or const_biases or run_biases)]
+                E, Ev = _val(r.q).size(-1), _val(r.v).size(-1)
+                if sum(families) > 1 or not plain or not (32 < max(E, Ev) <= 128):
+                    raise _NoMatch("dropout together with this combination of score modifications or head dims")
+                kwargs["dropout_p"] = r.dropout_p
         except _NoMatch:
             continue
         bias_nodes: List[fx.Node] = list(run_biases)

@@ -165,3 +165,22 @@ def squared_scores(query, key, value):
     w = query @ key.transpose(-2, -1) * 0.125
     w = -0.5 * w * w + w
     return torch.softmax(w, dim=-1) @ value
+
+
+def causal_with_dropout(query, key, value, p=0.1, training=True):
+    """The usual module code: dropout on the attention weights, active in training mode only."""
+    future = torch.triu(torch.ones(query.size(-2), key.size(-2), device=query.device, dtype=torch.bool), diagonal=1)
+    w = (query @ key.transpose(-2, -1) / math.sqrt(query.size(-1))).masked_fill(future, float("-inf"))
+    w = F.dropout(torch.softmax(w, dim=-1), p=p, training=training)
+    return w @ value
+
+
+def learned_bias_with_dropout(query, key, value, bias, p=0.2):
+    w = torch.softmax(query @ key.transpose(-2, -1) * 0.125 + bias, dim=-1)
+    return torch.nn.functional.dropout(w, p) @ value
+
+
+def documents_with_dropout(query, key, value, document_id, p=0.1):
+    same = document_id.unsqueeze(2) == document_id.unsqueeze(1)
+    w = (query @ key.transpose(-2, -1) / math.sqrt(query.size(-1))).masked_fill(~same.unsqueeze(1), -1e10)
+    return torch.dropout(torch.softmax(w, dim=-1), p, True) @ value

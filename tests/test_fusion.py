@@ -186,6 +186,30 @@ def test_rewrite_differential_and_msa_row():
     assert len(calls) == 1 and not _leftover(gm) and len(calls[0].args[4]) == 2
 
 
+def test_rewrite_maps_training_mode_dropout_to_the_kernel():
+    q, k, v = _qkv(E=64)
+    gm, calls = _rewrite(E.causal_with_dropout, q, k, v)
+    assert len(calls) == 1 and not _leftover(gm) and "dropout" not in {fusion._name(n) for n in gm.graph.nodes}
+    assert calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL
+    # evaluation mode: the dropout is the identity and leaves no trace
+    gm, calls = _rewrite(functools.partial(E.causal_with_dropout, training=False), q, k, v)
+    assert len(calls) == 1 and not calls[0].kwargs.get("dropout_p") and not _leftover(gm)
+    gm, calls = _rewrite(E.learned_bias_with_dropout, q, k, v, torch.randn(4, 48, 48))
+    assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.2 and len(calls[0].args[4]) == 1
+    gm, calls = _rewrite(E.documents_with_dropout, q, k, v, _ids(2, 48))
+    assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_DOCUMENT
+    # outside what the dropout kernels cover the region stays eager: head dim 32; a bias together with a soft-cap
+    q32, k32, v32 = _qkv(E=32)
+    gm, calls = _rewrite(E.causal_with_dropout, q32, k32, v32)
+    assert calls == [] and "dropout" in {fusion._name(n) for n in gm.graph.nodes}
+
+    def capped_bias_dropout(q, k, v, b):
+        w = torch.softmax(20.0 * torch.tanh(q @ k.transpose(-2, -1) * 0.125 / 20.0) + b, dim=-1)
+        return torch.nn.functional.dropout(w, 0.1) @ v
+    gm, calls = _rewrite(capped_bias_dropout, q, k, v, torch.randn(4, 48, 48))
+    assert calls == []
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)
@@ -272,6 +296,58 @@ def test_rewritten_dense_document_differential_and_msa_on_gpu():
     Q, K, V = (torch.randn(1, 3, 104, 2, 32, generator=g).to(BF).to(dev) for _ in range(3))
     mask, pair = torch.randn(1, 3, 1, 1, 104, generator=g).to(BF).to(dev), torch.randn(1, 1, 2, 104, 104, generator=g).to(BF).to(dev)
     _check_on_gpu(lambda Q, K, V, m, p: E.msa_row(Q, K, V, [m, p]), (Q, K, V, mask, pair), "msa row")
+
+
+@pytest.mark.gpu
+def test_rewritten_dropout_regions_on_gpu():
+    """The kernel's random stream is not torch's, so the rewritten function is compared with the kernel called directly
+    for the same seed (itself checked against the oracle in tests/test_dropout.py), and with the eager function through
+    what does not depend on the stream: the kept fraction, and p = 0 in evaluation mode."""
+    from flashlight_amd import ops
+    q, k, v = _qkv(N=2, Hq=4, Hkv=4, L=300, E=64, dev="cuda", seed=21)
+    torch._dynamo.reset()
+    fn = torch.compile(E.causal_with_dropout, backend=fusion.backend, dynamic=False, fullgraph=True)
+    torch.manual_seed(5)
+    a = fn(q, k, v)
+    torch.manual_seed(5)
+    b = fn(q, k, v)
+    c = fn(q, k, v)
+    torch.manual_seed(5)
+    direct = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.1)
+    assert torch.equal(a, b) and not torch.equal(a, c) and torch.equal(a, direct)
+    # with value = 1 every output element is (kept weight mass) / (1 - p): mean 1 over rows with many keys
+    ones = torch.ones_like(v)
+    mass = fn(q * 0, k, ones).float()[:, :, 150:, 0]  # uniform weights over >= 151 keys
+    assert abs(mass.mean().item() - 1.0) < 0.01 and 0.02 < mass.std().item() < 0.06
+    torch._dynamo.reset()
+    ev = torch.compile(functools.partial(E.causal_with_dropout, training=False), backend=fusion.backend, dynamic=False,
+                       fullgraph=True)(q, k, v)
+    assert_parity(ev, E.causal_with_dropout(q.float(), k.float(), v.float(), training=False), "evaluation mode")
+    # gradients flow through the rewritten region (the backward regenerates the forward's decisions)
+    qg = q.detach().clone().requires_grad_(True)
+    torch.manual_seed(9)
+    fn(qg, k, v).float().sum().backward()
+    q2 = q.detach().clone().requires_grad_(True)
+    torch.manual_seed(9)
+    ops.dispatch(q2, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.1).float().sum().backward()
+    assert torch.equal(qg.grad, q2.grad) and qg.grad.abs().max().item() > 0
+    # documents and a learned bias
+    ids = _ids(2, 300, "cuda")
+    torch._dynamo.reset()
+    fd = torch.compile(E.documents_with_dropout, backend=fusion.backend, dynamic=False, fullgraph=True)
+    torch.manual_seed(3)
+    x = fd(q, k, v, ids)
+    torch.manual_seed(3)
+    y = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_DOCUMENT, doc_ids=ids, dropout_p=0.1)
+    assert torch.equal(x, y)
+    bias = torch.randn(4, 300, 300, device="cuda")
+    torch._dynamo.reset()
+    fb = torch.compile(E.learned_bias_with_dropout, backend=fusion.backend, dynamic=False, fullgraph=True)
+    torch.manual_seed(4)
+    x = fb(q, k, v, bias)
+    torch.manual_seed(4)
+    y = ops.dispatch(q, k, v, scale=0.125, biases=[(bias.unsqueeze(0), 1)], dropout_p=0.2)
+    assert torch.equal(x, y)
 
 
 @pytest.mark.gpu

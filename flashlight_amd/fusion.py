@@ -195,7 +195,7 @@ def _classify_document_mask(node: fx.Node, ids_ph: fx.Node, invert: bool, L: int
               torch.randint(-5, 7, (N, L), generator=g),
               torch.zeros(N, L, dtype=torch.int64)]
     q, k = _idx(L, S, dev)
-    verdict = None
+    found = None
     for ids in probes:
         ids = ids.to(device=dev, dtype=ex.dtype)
         try:
@@ -215,10 +215,10 @@ def _classify_document_mask(node: fx.Node, ids_ph: fx.Node, invert: bool, L: int
         got = _ffi.MASK_DOCUMENT if ok_doc else _ffi.MASK_DOCUMENT_CAUSAL if ok_causal else None
         if ok_doc and ok_causal:  # a probe that cannot tell the two apart
             continue
-        if got is None or (verdict is not None and verdict != got):
+        if got is None or (found is not None and found != got):
             return None
-        verdict = got
-    return verdict
+        found = got
+    return found
 
 
 def _is_alibi(b: torch.Tensor, H: int, L: int, S: int) -> bool:

@@ -472,9 +472,13 @@ def test_random_dropout_cases(seed):
     # kept weights are scaled by 1 / (1 - p): the tolerances scale with it
     f = 1.0 / (1.0 - p)
     assert_parity(out.float() / f, ref / f, f"forward {c}")
+    # With a single key the exact score gradient is 0 (dP / (1 - p) - Delta cancels), and what the kernels return is
+    # the rounding of the bf16 forward result inside Delta times q or k: a few 1e-3 on every element, so such a case
+    # is held to the max-abs bound alone.
+    mean_tol = 2e-2 if S == 1 else 2e-3
     for what, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
-        scale = max(1.0, want.abs().max().item())
-        assert_parity(got.float() / scale, want / scale, f"{what} {c}")
+        scale = max(1.0, want.abs().max().item()) * f
+        assert_parity(got.float() / scale, want / scale, f"{what} {c}", mean_tol=mean_tol)
 
 
 @pytest.mark.gpu

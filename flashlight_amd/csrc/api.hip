@@ -693,7 +693,9 @@ int fl_attn_fwd(const fl_attn_params* p, void* stream_) {
   for (int nb = 0; nb < 2; ++nb) {
     if (!p->bias[nb] || p->bias_strides[nb][3] != 1 || reinterpret_cast<uintptr_t>(p->bias[nb]) % 16 != 0) continue;
     if (p->Lk % 8 != 0) continue;
-    if (kp.bias_f32[nb] && p->bias_strides[nb][2] != 0) continue;  // fp32: only a row-broadcast operand is staged
+    // fp32: staged only as the row-broadcast operand (the [rows][keys] tiles hold 16-bit elements, so a second fp32 row
+    // operand takes the direct path)
+    if (kp.bias_f32[nb] && (p->bias_strides[nb][2] != 0 || kp.bias_row >= 0)) continue;
     bool ok = true;
     for (int i = 0; i < 3; ++i) ok = ok && p->bias_strides[nb][i] % 8 == 0;
     // per-lane byte offsets inside one (batch, head) slice are 32-bit

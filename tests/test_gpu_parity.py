@@ -241,6 +241,7 @@ def test_evoformer_bias_staged_and_direct_paths(D):
     # boundary (read directly), each with the sigmoid gate.
     g = torch.Generator().manual_seed(170 + D)
     mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(DEV)
+    mk32 = lambda *s: torch.randn(*s, generator=g).to(DEV)
     B, N, S, H = 1, 3, 104, 2
     Q, K, V, G = mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D), mk(B, N, S, H, D)
     wide = mk(B, 1, H, S, S + 8)
@@ -248,6 +249,11 @@ def test_evoformer_bias_staged_and_direct_paths(D):
         "mask + pair": [mk(B, N, 1, 1, S), mk(B, 1, H, S, S)],
         "two dense": [mk(B, 1, H, S, S), mk(B, N, H, S, S)],
         "two masks": [mk(B, N, 1, 1, S), mk(B, 1, 1, 1, S)],
+        # fp32 rows: the first is staged as the row operand, a second one is read directly (the staged tiles hold
+        # 16-bit elements)
+        "two fp32 masks": [mk32(B, N, 1, 1, S), mk32(B, 1, 1, 1, S)],
+        "mask + fp32 mask": [mk(B, N, 1, 1, S), mk32(B, 1, H, 1, S)],
+        "fp32 mask + pair": [mk32(B, N, 1, 1, S), mk(B, 1, H, S, S)],
         "misaligned rows": [wide[..., 1:S + 1]],
         "padded rows": [wide[..., 8:S + 8]],
     }

@@ -366,7 +366,7 @@ struct FwdTraits {
 #ifdef FL_WPE
   static constexpr int WAVES_PER_EU = FL_WPE;
 #else
-  static constexpr int WAVES_PER_EU = (RW == 32 && DQK <= 256) ? 2 : 1;
+  static constexpr int WAVES_PER_EU = (RW == 32 && DQK <= 256 && !(DQK == 256 && (FEAT_ & F_BIAS))) ? 2 : 1;
 #endif
   // One dense bias operand is staged through LDS like K and V: per ring slot a [BM][BN] bf16 tile, every wave
   // transferring (and later reading) only its own RW rows.

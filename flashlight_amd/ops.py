@@ -235,7 +235,7 @@ def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi
 _HEAD_DIMS = (32, 64, 128)
 
 
-def _pad_head_dims(q, k, v, gate, diff):
+def _pad_head_dims(q, k, v, gate, diff, bias_only=True):
     """(q, k, v, gate) with zero columns appended up to a compiled head dim, or None when the head dims are compiled as
     they are (32, 64, 128 for q, k and v alike; 256 and 512 for q and k with values in slabs of 128 columns; the 64/128 and
     128/256 pairs of differential attention) or when no padding would help."""
@@ -249,8 +249,10 @@ def _pad_head_dims(q, k, v, gate, diff):
             return None
         pq = next(p for p in (64, 128) if p >= dqk)
         pv = 2 * pq
-    elif (dqk, dv) in ((32, 64), (64, 128)):
-        return None  # compiled pairs (invariant point attention's channel counts land on them)
+    elif (dqk, dv) in ((32, 64), (64, 128)) and bias_only:
+        # compiled pairs (invariant point attention's channel counts land on them), with dense bias operands as the only
+        # score modification; anything else goes to the square head dim, whose instances cover every combination
+        return None
     elif dqk > 128 or dv > 128:
         if dqk > 512:
             return None
@@ -277,7 +279,9 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     their pre-pass every time.  `score_fn` = (kind, four constants), see `_ffi.attn_fwd`: forward only."""
     dropout_p = float(dropout_p)
     _ffi.dropout_threshold(dropout_p)  # range check
-    padded = _pad_head_dims(q, k, v, gate, diff)
+    padded = _pad_head_dims(q, k, v, gate, diff,
+                            bias_only=not (alibi_heads or softcap or doc_ids is not None or gate is not None or dropout_p > 0.0
+                                           or score_fn is not None))
     if padded is not None:
         # head dims between the compiled ones: zero columns change neither q.k nor the columns of the result that are
         # kept (the reference's generated kernel takes any head dim up to 256 in one block, monkeypatch/fusion/_common.py:4,

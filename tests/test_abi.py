@@ -55,6 +55,31 @@ def rc(lib, p):
     return lib.fl_attn_validate(C.byref(p))
 
 
+def test_every_combination_of_score_modifications_has_a_kernel(lib):
+    """Mask kind x ALiBi x soft-cap x bias operands x gate, at every compiled head dim and in both element types: the
+    reference's functions compose these freely (attention_variants/*.py are plain PyTorch), so no combination of them
+    may end in "no kernel instance"."""
+    import itertools
+    for (D, Dv), dtype in itertools.product(((32, 32), (64, 64), (128, 128), (256, 128), (512, 128)), (_ffi.FL_BF16, _ffi.FL_F16)):
+        for kind, alibi, cap, bias, gate in itertools.product(
+                (_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM, _ffi.MASK_DOCUMENT,
+                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2), (False, True)):
+            p = good_params(D=D, Dv=Dv)
+            p.dtype = dtype
+            p.mask_kind, p.window, p.prefix = kind, 17, 40
+            p.alibi_heads, p.softcap = alibi, cap
+            for i in range(bias):
+                p.bias[i], p.bias_batch_div[i], p.bias_dtype[i] = 0x60000 + 0x100000 * i, 1, dtype
+                p.bias_strides[i][:] = (0, 0, 304, 1) if i == 0 else (0, 0, 0, 1)
+            if gate:
+                p.gate = 0x70000
+                p.gate_strides[:] = list(p.o_strides)
+            if kind in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):
+                p.doc_ids, p.doc_stride = 0x50000, 300
+                p.workspace, p.workspace_bytes = 0x80000, lib.fl_workspace_bytes(C.byref(p))
+            assert rc(lib, p) == 0, (D, Dv, dtype, kind, alibi, cap, bias, gate, _ffi.last_error())
+
+
 def test_valid_params_pass(lib):
     for D in (32, 64, 128):
         assert rc(lib, good_params(D=D)) == 0, _ffi.last_error()

@@ -165,6 +165,37 @@ def test_document_mask_with_dense_bias_and_gate(D, cap, causal):
     assert_parity(out, ref * torch.sigmoid(gate.float()), f"D={D} cap={cap} causal={causal}")
 
 
+@pytest.mark.parametrize("D,Dv", [(32, 32), (64, 64), (128, 128), (256, 128), (512, 128), (64, 128), (32, 64), (96, 256)])
+@pytest.mark.parametrize("kind", [_ffi.MASK_SLIDING, _ffi.MASK_DOCUMENT_CAUSAL])
+@pytest.mark.parametrize("cap", [None, 12.0])
+def test_all_score_modifications_together_at_every_head_dim(D, Dv, kind, cap):
+    """The in-kernel ALiBi term, the soft-cap (or none), a dense bf16 operand, a row-broadcast fp32 operand and the gate
+    under a sliding window or causal documents: at every compiled head dim, at the rectangular pairs (which go to the
+    square instances for this) and at a padded one."""
+    B, Hq, Hkv, S, window = 2, 4, 2, 290, 77
+    q, k, v = qkv(B, Hq, Hkv, S, D, Dv, seed=D + Dv + kind, amp=2.0)
+    g = torch.Generator().manual_seed(29)
+    ids = torch.sort(torch.randint(0, 4, (B, S), generator=g), dim=1).values
+    dense = (torch.randn(1, Hq, S, S, generator=g) * 1.5).to(torch.bfloat16)
+    row = torch.randn(B, 1, 1, S, generator=g)
+    gate = torch.randn(B, Hq, S, Dv, generator=g).to(torch.bfloat16)
+    doc = kind == _ffi.MASK_DOCUMENT_CAUSAL
+    out = ops.dispatch(q, k, v, mask_kind=kind, window=window, doc_ids=ids.to(DEV) if doc else None, alibi_heads=Hq,
+                       softcap=cap or 0.0, biases=[(dense.to(DEV), B), (row.to(DEV), 1)], gate=gate.to(DEV))
+    slopes = alibi_slopes(Hq).float().view(1, Hq, 1, 1)
+
+    def masked(qi, ki):
+        if doc:
+            return (ids[:, qi.view(-1)].view(B, 1, -1, 1) != ids[:, ki.view(-1)].view(B, 1, 1, -1)) | (ki > qi)
+        return (ki > qi) | (qi - ki > window)
+
+    qf, kf, vf = f32(q, k, v)
+    ref = _softmax_attention(qf, kf.repeat_interleave(Hq // Hkv, 1), vf.repeat_interleave(Hq // Hkv, 1), 1.0 / math.sqrt(D),
+                             masked=masked, softcap=cap,
+                             bias=lambda qi, ki: (slopes * (ki - qi).float(), dense.float()[..., qi.view(-1), :], row))
+    assert_parity(out, ref * torch.sigmoid(gate.float()), f"D={D}/{Dv} kind={kind} cap={cap}")
+
+
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("gqa", [False, True])
 def test_dense_score_mod_with_softcap(D, gqa):

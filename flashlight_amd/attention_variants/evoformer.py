@@ -57,10 +57,10 @@ def attention_reference(q_input: torch.Tensor, k_input: torch.Tensor, v_input: t
         return t.reshape(-1, *t.shape[-3:]).transpose(1, 2)
 
     bl = list(biases)
-    if len(bl) > 2:  # the kernel takes two bias operands; fold the rest into the second one
-        extra = bl[1]
+    if len(bl) > 2:  # the kernel takes two bias operands; fold the rest into the second one, in fp32 (a sum rounded to
+        extra = bl[1].float()  # 16 bits would move the logits by the rounding of their largest term)
         for b in bl[2:]:
-            extra = extra + b
+            extra = extra + b.float()
         bl = [bl[0], extra]
     if S != Sk and bl:
         raise ValueError("biases need equally long query and key sequences")

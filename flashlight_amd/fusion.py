@@ -23,7 +23,7 @@ Masks and biases are recognised by what they compute, not by how they were writt
     passed to the kernel's bias operands (fp32 or bf16).
 A training-mode dropout on the softmax weights becomes the kernel's own dropout (same rate, the kernel's random
 stream, a fresh seed per call) where the dropout kernels cover the region: one of ALiBi / soft-cap, a document mask or
-dense operands, head dims 33 .. 128.  Regions that do not fit (a softmax whose weights are used elsewhere, dropout
+dense operands, head dims up to 128.  Regions that do not fit (a softmax whose weights are used elsewhere, dropout
 outside that coverage, ...) are left untouched.
 """
 from __future__ import annotations
@@ -400,6 +400,20 @@ def _peel_function(n: fx.Node, r: _Region, qk_memo, mods_below: List[str]):
     return _peel_scores(root[0], r, qk_memo, mods_below)
 
 
+def _as_number(x) -> Optional[float]:
+    """x as a float when it is a Python number or a one-element tensor that depends on no graph input (a fill written
+    as `torch.tensor(float("-inf"))` or `torch.full((), -1e10)`), else None."""
+    if _is_number(x):
+        return float(x)
+    if isinstance(x, fx.Node) and not _placeholders_of(x):
+        ex = _val(x)
+        if isinstance(ex, torch.Tensor) and ex.numel() == 1:
+            got = _try_evaluate(x, x.graph.owning_module)
+            if isinstance(got, torch.Tensor) and got.numel() == 1:
+                return float(got.float().item())
+    return None
+
+
 def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
     """Walks from the softmax input up to the q k^T matmul, recording what each step does to the scores."""
     nm = _name(n)
@@ -420,10 +434,11 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
         return
     if nm in ("where",):
         cond, a, b = n.args[0], n.args[1], n.args[2]
-        if isinstance(b, fx.Node) and _is_number(a) and a <= -1e9:
+        fa, fb = _as_number(a), _as_number(b)
+        if isinstance(b, fx.Node) and fb is None and fa is not None and fa <= -1e9:
             r.masks.append((cond, False))
             inner = b
-        elif isinstance(a, fx.Node) and _is_number(b) and b <= -1e9:
+        elif isinstance(a, fx.Node) and fa is None and fb is not None and fb <= -1e9:
             r.masks.append((cond, True))
             inner = a
         else:
@@ -432,8 +447,8 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
         mods_below.append("mask")
         return _peel_scores(inner, r, qk_memo, mods_below)
     if nm == "masked_fill":
-        inner, cond, fill = n.args[0], _arg(n, 1, "mask"), _arg(n, 2, "value")
-        if not (_is_number(fill) and fill <= -1e9):
+        inner, cond, fill = n.args[0], _arg(n, 1, "mask"), _as_number(_arg(n, 2, "value"))
+        if fill is None or not fill <= -1e9:
             raise _NoMatch("masked_fill value is not a large negative number")
         r.masks.append((cond, False))
         r.nodes.append(n)
@@ -706,11 +721,11 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                 else:
                     run_biases.append(node)
             if r.dropout_p:
-                # the dropout kernels cover one family at a time and head dims that are (or pad to) 64 or 128
+                # the dropout kernels cover one family at a time and head dims up to 128 (padded to 64 or 128)
                 families = [bool(kwargs["alibi_heads"] or r.softcap), doc_ids is not None,
                             bool(run_masks or const_biases or run_biases)]
                 E, Ev = _val(r.q).size(-1), _val(r.v).size(-1)
-                if sum(families) > 1 or not plain or not (32 < max(E, Ev) <= 128):
+                if sum(families) > 1 or not plain or max(E, Ev) > 128:
                     raise _NoMatch("dropout together with this combination of score modifications or head dims")
                 kwargs["dropout_p"] = r.dropout_p
         except _NoMatch:

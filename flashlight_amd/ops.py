@@ -235,12 +235,12 @@ def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi
 _HEAD_DIMS = (32, 64, 128)
 
 
-def _pad_head_dims(q, k, v, gate, diff, bias_only=True):
+def _pad_head_dims(q, k, v, gate, diff, bias_only=True, min_dim=32):
     """(q, k, v, gate) with zero columns appended up to a compiled head dim, or None when the head dims are compiled as
     they are (32, 64, 128 for q, k and v alike; 256 and 512 for q and k with values in slabs of 128 columns; the 64/128 and
     128/256 pairs of differential attention) or when no padding would help."""
     dqk, dv = q.shape[-1], v.shape[-1]
-    if not diff and dqk == dv and dqk in _HEAD_DIMS:
+    if not diff and dqk == dv and dqk in _HEAD_DIMS and not (dqk == 32 and min_dim > 32):
         return None  # the common case, decided first: this runs on every call
     if dqk != k.size(-1) or q.dim() != 4 or v.dim() != 4:
         return None  # left to the binding's own checks
@@ -258,7 +258,7 @@ def _pad_head_dims(q, k, v, gate, diff, bias_only=True):
             return None
         pq, pv = (128 if dqk <= 128 else 256 if dqk <= 256 else 512), -(-dv // 128) * 128
     else:
-        pq = pv = next(p for p in _HEAD_DIMS if p >= max(dqk, dv))
+        pq = pv = next(p for p in _HEAD_DIMS if p >= max(dqk, dv, min_dim))
     if (pq, pv) == (dqk, dv):
         return None
     pad = torch.nn.functional.pad
@@ -281,7 +281,9 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     _ffi.dropout_threshold(dropout_p)  # range check
     padded = _pad_head_dims(q, k, v, gate, diff,
                             bias_only=not (alibi_heads or softcap or doc_ids is not None or gate is not None or dropout_p > 0.0
-                                           or score_fn is not None))
+                                           or score_fn is not None),
+                            # (score functions and dropout are compiled from head dim 64 up)
+                            min_dim=64 if (score_fn is not None or dropout_p > 0.0) else 32)
     if padded is not None:
         # head dims between the compiled ones: zero columns change neither q.k nor the columns of the result that are
         # kept (the reference's generated kernel takes any head dim up to 256 in one block, monkeypatch/fusion/_common.py:4,

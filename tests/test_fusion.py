@@ -198,10 +198,21 @@ def test_rewrite_maps_training_mode_dropout_to_the_kernel():
     assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.2 and len(calls[0].args[4]) == 1
     gm, calls = _rewrite(E.documents_with_dropout, q, k, v, _ids(2, 48))
     assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_DOCUMENT
-    # outside what the dropout kernels cover the region stays eager: head dim 32; a bias together with a soft-cap
-    q32, k32, v32 = _qkv(E=32)
-    gm, calls = _rewrite(E.causal_with_dropout, q32, k32, v32)
+    # outside what the dropout kernels cover the region stays eager: head dims above 128; a bias together with a soft-cap
+    q256, k256, v256 = _qkv(E=256)
+    gm, calls = _rewrite(E.causal_with_dropout, q256, k256, v256)
     assert calls == [] and "dropout" in {fusion._name(n) for n in gm.graph.nodes}
+    q32, k32, v32 = _qkv(E=32)  # (head dim 32 is padded to 64 at run time)
+    gm, calls = _rewrite(E.causal_with_dropout, q32, k32, v32)
+    assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.1
+    # a fill written as a one-element constant tensor is a fill like any number
+    def tensor_fill(q, k, v):
+        future = torch.ones(q.size(-2), k.size(-2), dtype=torch.bool).triu(1)
+        s = torch.where(future, torch.tensor(float("-inf")), q @ k.transpose(-2, -1) * 0.125)
+        s = s.masked_fill(future, torch.full((), -1e10))
+        return torch.softmax(s, dim=-1) @ v
+    gm, calls = _rewrite(tensor_fill, q, k, v)
+    assert len(calls) == 1 and not _leftover(gm) and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL
 
     def capped_bias_dropout(q, k, v, b):
         w = torch.softmax(20.0 * torch.tanh(q @ k.transpose(-2, -1) * 0.125 / 20.0) + b, dim=-1)

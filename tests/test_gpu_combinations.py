@@ -254,6 +254,20 @@ def test_score_mod_callables_of_the_softcap_signature(D):
     assert_parity(out, _eager_softcapped(qf, kf, vf, capped_then_shifted, causal=True), "capped_then_shifted")
 
 
+def test_head_dim_32_score_functions_and_dropout_run_on_the_64_wide_kernels():
+    """Score functions other than the soft-cap and dropout are compiled from head dim 64 up; narrower calls are padded."""
+    import oracle.dropout as OD
+    q, k, v = qkv(2, 4, 4, 150, 32, seed=60, amp=3.0)
+    qf, kf, vf = f32(q, k, v)
+    relu = lambda s, b, h, qi, ki: torch.relu(s)  # noqa: E731
+    assert_parity(A.attention_softcapped(q, k, v, score_mod=relu, is_causal=True),
+                  _eager_softcapped(qf, kf, vf, relu, causal=True), "relu at head dim 32")
+    out = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.25, dropout_seed=99)
+    keep = OD.keep_mask(99, 2, 4, 150, 150, 0.25)
+    causal = torch.arange(150)[None, :] <= torch.arange(150)[:, None]
+    assert_parity(out, OD.attention_dropout(qf, kf, vf, keep, 0.25, attend=causal), "dropout at head dim 32")
+
+
 def test_score_mod_the_kernel_cannot_apply_is_refused():
     q, k, v = qkv(1, 2, 2, 64, 64, seed=50)
     for fn in (lambda s, b, h, qi, ki: torch.exp(s),

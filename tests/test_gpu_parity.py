@@ -92,6 +92,41 @@ def assert_script_tolerance(out, ref, what=""):
     assert n_over == 0, f"{what}: worst {excess.max().item():.3f} x bound, {n_over} of {excess.numel()} elements over"
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_sequences_of_65536_through_size_independent_properties(D):
+    """Too long for the CPU oracle: (1) the unmasked result equals the merge, through the row statistics, of four calls
+    that each see a quarter of the keys; (2) a document mask over sorted ids equals separate calls per document, with and
+    without the causal term.  Both sides are 16-bit results of the same kernels on different tilings and list lengths,
+    so the bound is the suite's (max-abs 2e-2, mean-abs 2e-3)."""
+    L, H = 65536, 2
+    g = torch.Generator().manual_seed(65 + D)
+    q, k, v = (torch.randn(1, H, L, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(3))
+    lse = torch.empty(1, H, L, dtype=torch.float32, device=DEV)
+    full = _ffi.attn_fwd(q, k, v, lse=lse).float()
+    parts, stats = [], []
+    for c in range(4):
+        ks = slice(c * L // 4, (c + 1) * L // 4)
+        st = torch.empty(1, H, L, dtype=torch.float32, device=DEV)
+        parts.append(_ffi.attn_fwd(q, k[:, :, ks], v[:, :, ks], lse=st, scale=1.0 / math.sqrt(D)).float())
+        stats.append(st)
+    stats = torch.stack(stats)                                   # log2 of the row sums
+    total = torch.logsumexp(stats * math.log(2.0), dim=0) / math.log(2.0)
+    merged = sum(p * torch.exp2(st - total).unsqueeze(-1) for p, st in zip(parts, stats))
+    assert_parity(full, merged, "65536 keys against four quarters")
+    assert (lse - total).abs().max().item() < 2e-2
+    lengths = [20000, 1, 30001, 15534]
+    ids = torch.repeat_interleave(torch.arange(4), torch.tensor(lengths)).view(1, L).to(DEV)
+    for causal in (False, True):
+        got = A.attention_pytorch_document_mask(q, k, v, ids, is_causal=causal)
+        a = 0
+        for n in lengths:
+            sl = slice(a, a + n)
+            fn = A.attention_pytorch_causal if causal else A.attention_pytorch
+            want = fn(q[:, :, sl], k[:, :, sl], v[:, :, sl], scale=1.0 / math.sqrt(D))
+            assert_parity(got[:, :, sl], want, f"document of {n} positions at {a}, causal={causal}")
+            a += n
+
+
 def test_reference_script_vanilla_and_causal():   # tests/test_vanilla.py:21-36, tests/test_causal.py:21-36
     q, k, v = qkv(2, 1, 1, 16384, 128, seed=1, lo_hi=(-9, 9))
     assert_script_tolerance(A.attention_pytorch(q, k, v), O.attention_vanilla(*f32(q, k, v), q_block=1024), "vanilla")

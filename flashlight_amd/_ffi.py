@@ -426,9 +426,9 @@ def attn_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tenso
     `grads` = (dq, dk, dv) receives the results when given.  `static_scratch` goes through `fl_attn_bwd_static`: nothing
     is allocated here beyond the results, the library's own static device array serves as scratch (calls that may
     overlap on one GPU must not both use it).
-    `biases` are the forward's bias operands (positional masks only); `dscores`, a zero-filled contiguous float32
-    [B, Hq, Lq, Lk] tensor, then receives the gradient with respect to the scores, from which the caller sums the
-    gradient of each operand over the axes it broadcasts over."""
+    `biases` are the forward's bias operands; `dscores`, a zero-filled contiguous float32 [B, Hq, Lq, Lk] tensor, then
+    receives the gradient with respect to the scores, from which the caller sums the gradient of each operand over the
+    axes it broadcasts over (not under a soft-cap)."""
     lib = load_library()
     for name, t in (("query", q), ("key", k), ("value", v), ("out", out), ("dout", dout)):
         _require_gpu_half(name, t, q if isinstance(q, torch.Tensor) and q.dtype in _HALF_TYPES else None)

@@ -772,8 +772,10 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
   if (p->score_fn != FL_SCORE_NONE) return fail(FL_ERR_UNSUPPORTED, "backward: score_fn is forward-only");
   const bool has_bias = p->bias[0] || p->bias[1];
-  if (has_bias && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind)))
-    return fail(FL_ERR_UNSUPPORTED, "backward: bias operands go with positional masks (and dropout) only: no ALiBi, soft-cap or document mask");
+  if (has_bias && p->dropout_threshold && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind)))
+    return fail(FL_ERR_UNSUPPORTED, "backward: dropout with bias operands goes with positional masks only (no ALiBi, soft-cap or document mask)");
+  if (b->dscores && p->softcap > 0.f)
+    return fail(FL_ERR_UNSUPPORTED, "backward: dscores is not produced under a soft-cap (gradients of bias operands added after the cap)");
   if (b->dscores && !has_bias) return fail(FL_ERR_ARG, "backward: dscores is only written for calls with bias operands");
   if (b->dscores && reinterpret_cast<uintptr_t>(b->dscores) % 16) return fail(FL_ERR_ALIGN, "backward: dscores must be 16-byte aligned");
   if (p->Dqk != p->Dv) return fail(FL_ERR_UNSUPPORTED, "backward needs Dqk == Dv (got %d, %d)", p->Dqk, p->Dv);
@@ -797,15 +799,15 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   uint32_t want = 0;
   if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
   if (is_doc(p->mask_kind)) want |= fl::F_DOC;
-  if (has_bias) want = fl::F_BIAS;
+  if (has_bias) want |= fl::F_BIAS;
   if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() allows one of document mask, ALiBi / soft-cap, bias operands
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)
       in = &fl::kBwdInstances[i];
   if (!in)
-    return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d with features 0x%x (compiled: 64 and 128; 32 "
-                "without score modification or with bias operands)", p->Dqk, want);
+    return fail(FL_ERR_UNSUPPORTED, "backward: no kernel for head dim %d with features 0x%x (compiled: 32, 64 and 128; dropout at 64 "
+                "and 128)", p->Dqk, want);
   if (out) *out = in;
   g_err[0] = 0;
   return 0;

@@ -122,7 +122,7 @@ void bwd_kernel(const BParams p) {
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC, kBias = FEAT & F_BIAS;
   constexpr bool kDQ = ROLE == ROLE_DQ;
-  static_assert(!kBias || !(kAlibi || kSoftcap || kDoc), "bias operands go with positional masks (and dropout) only");
+  static_assert(!kBias || !((kAlibi || kSoftcap || kDoc) && (FEAT & F_DROPOUT)), "dropout with bias operands goes with positional masks only");
   using E = typename T::Elem;  // pointers in BParams are typed bf16_t whatever E is: 16 opaque bits
   typedef E ex8 __attribute__((ext_vector_type(8)));
   typedef E ex4 __attribute__((ext_vector_type(4)));
@@ -535,7 +535,8 @@ void bwd_kernel(const BParams p) {
               }
               dsf[2 * sb + i / 8][i % 8] = (E)ds;
               if constexpr (kBias && kDQ) {
-                // the gradient with respect to the score (no soft-cap goes with a bias: d(score) / d(qk * scale) = 1)
+                // the gradient with respect to the score; with the soft-cap switched on ds carries d(cap) / d(qk * scale)
+                // besides, which is not part of it: the host refuses dscores then
                 const int key = sbase + 8 * g + e;
                 if (p.dscores != nullptr && opos < p.Lq && key < p.Lk)
                   p.dscores[(((int64_t)batch * p.Hq + ohead) * p.Lq + opos) * p.Lk + key] = ds;

@@ -120,7 +120,8 @@ attn_fwd_lse.register_autograd(_backward, setup_context=_setup_context)
 @torch.library.custom_op("flashlight_amd::attn_fwd_bias_lse", mutates_args=())
 def attn_fwd_bias_lse(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, mask_kind: int, window: int,
                       prefix: int, bias0: Optional[torch.Tensor], bias0_div: int, bias1: Optional[torch.Tensor],
-                      bias1_div: int, dropout_p: float = 0.0, dropout_seed: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
+                      bias1_div: int, dropout_p: float = 0.0, dropout_seed: int = 0, doc_ids: Optional[torch.Tensor] = None,
+                      alibi_heads: int = 0, softcap: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
     """The forward with bias operands for calls that will be differentiated (the reference's Evoformer function and its
     dense `score_mod` tensors, attention_variants/evoformer.py:24-27, alibi.py:26-30; the reference itself has no
     backward): result and row statistics, like `attn_fwd_lse`.  An operator of its own, so that `torch.compile` traces
@@ -129,13 +130,14 @@ def attn_fwd_bias_lse(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: 
     lse = torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
     biases = [(b, d) for b, d in ((bias0, bias0_div), (bias1, bias1_div)) if b is not None]
     _ffi.attn_fwd(q, k, v, scale=scale if scale > 0 else None, mask_kind=mask_kind, window=window, prefix=prefix,
-                  biases=biases, out=out, lse=lse, dropout_p=dropout_p, dropout_seed=dropout_seed)
+                  biases=biases, out=out, lse=lse, dropout_p=dropout_p, dropout_seed=dropout_seed, doc_ids=doc_ids,
+                  alibi_heads=alibi_heads, softcap=softcap)
     return out, lse
 
 
 @attn_fwd_bias_lse.register_fake
 def _attn_fwd_bias_lse_fake(q, k, v, scale, mask_kind, window, prefix, bias0, bias0_div, bias1, bias1_div, dropout_p=0.0,
-                            dropout_seed=0):
+                            dropout_seed=0, doc_ids=None, alibi_heads=0, softcap=0.0):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("query, key and value must be 4-D [batch, heads, seq, dim]")
     return _alloc_out(q, v, False, False), torch.empty((q.size(0), q.size(1), q.size(2)), dtype=torch.float32, device=q.device)
@@ -145,8 +147,9 @@ def _attn_fwd_bias_lse_fake(q, k, v, scale, mask_kind, window, prefix, bias0, bi
 def attn_bwd_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
                   dout: torch.Tensor, scale: float, mask_kind: int, window: int, prefix: int,
                   bias0: Optional[torch.Tensor], bias0_div: int, bias1: Optional[torch.Tensor], bias1_div: int,
-                  want_dscores: bool, dropout_p: float = 0.0,
-                  dropout_seed: int = 0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                  want_dscores: bool, dropout_p: float = 0.0, dropout_seed: int = 0,
+                  doc_ids: Optional[torch.Tensor] = None, alibi_heads: int = 0,
+                  softcap: float = 0.0) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dq, dk, dv, dscores) of `attn_fwd_bias_lse`: dscores, float32 [B, Hq, Lq, Lk], is the gradient with respect to
     whatever was added to q k^T scale (empty when `want_dscores` is false: no bias operand asks for a gradient)."""
     biases = [(b, d) for b, d in ((bias0, bias0_div), (bias1, bias1_div)) if b is not None]
@@ -154,13 +157,14 @@ def attn_bwd_bias(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.
     dscores = torch.zeros(shape, dtype=torch.float32, device=q.device)
     dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, scale=scale if scale > 0 else None, mask_kind=mask_kind,
                                window=window, prefix=prefix, biases=biases, dscores=dscores if want_dscores else None,
-                               dropout_p=dropout_p, dropout_seed=dropout_seed)
+                               dropout_p=dropout_p, dropout_seed=dropout_seed, doc_ids=doc_ids, alibi_heads=alibi_heads,
+                               softcap=softcap)
     return dq, dk, dv, dscores
 
 
 @attn_bwd_bias.register_fake
 def _attn_bwd_bias_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefix, bias0, bias0_div, bias1, bias1_div,
-                        want_dscores, dropout_p=0.0, dropout_seed=0):
+                        want_dscores, dropout_p=0.0, dropout_seed=0, doc_ids=None, alibi_heads=0, softcap=0.0):
     c = torch.contiguous_format
     shape = (q.size(0), q.size(1), q.size(2), k.size(2)) if want_dscores else (0,)
     return (torch.empty_like(q, memory_format=c), torch.empty_like(k, memory_format=c), torch.empty_like(v, memory_format=c),
@@ -168,20 +172,21 @@ def _attn_bwd_bias_fake(q, k, v, out, lse, dout, scale, mask_kind, window, prefi
 
 
 def _bias_setup_context(ctx, inputs, output):
-    q, k, v, scale, mask_kind, window, prefix, bias0, div0, bias1, div1, dropout_p, dropout_seed = inputs
+    q, k, v, scale, mask_kind, window, prefix, bias0, div0, bias1, div1, dropout_p, dropout_seed, doc_ids, alibi_heads, \
+        softcap = inputs
     out, lse = output
-    ctx.save_for_backward(q, k, v, out, lse, bias0, bias1)
-    ctx.args = (scale, mask_kind, window, prefix, div0, div1, dropout_p, dropout_seed)
+    ctx.save_for_backward(q, k, v, out, lse, bias0, bias1, doc_ids)
+    ctx.args = (scale, mask_kind, window, prefix, div0, div1, dropout_p, dropout_seed, alibi_heads, softcap)
 
 
 def _bias_backward(ctx, dout, dlse):
     """The gradient of a bias operand is the score gradient summed over the batch entries and axes the operand
     broadcasts over."""
-    q, k, v, out, lse, bias0, bias1 = ctx.saved_tensors
-    scale, mask_kind, window, prefix, div0, div1, dropout_p, dropout_seed = ctx.args
+    q, k, v, out, lse, bias0, bias1, doc_ids = ctx.saved_tensors
+    scale, mask_kind, window, prefix, div0, div1, dropout_p, dropout_seed, alibi_heads, softcap = ctx.args
     want = [b is not None and ctx.needs_input_grad[7 + 2 * i] for i, b in enumerate((bias0, bias1))]
     dq, dk, dv, dscores = attn_bwd_bias(q, k, v, out, lse, dout.to(q.dtype), scale, mask_kind, window, prefix, bias0, div0,
-                                        bias1, div1, any(want), dropout_p, dropout_seed)
+                                        bias1, div1, any(want), dropout_p, dropout_seed, doc_ids, alibi_heads, softcap)
     dbs = []
     for b, d, w in ((bias0, div0, want[0]), (bias1, div1, want[1])):
         if not w:
@@ -192,7 +197,7 @@ def _bias_backward(ctx, dout, dlse):
         if axes:
             g = g.sum(axes, keepdim=True)
         dbs.append(g.to(b.dtype))
-    return dq, dk, dv, None, None, None, None, dbs[0], None, dbs[1], None, None, None
+    return dq, dk, dv, None, None, None, None, dbs[0], None, dbs[1], None, None, None, None, None, None
 
 
 attn_fwd_bias_lse.register_autograd(_bias_backward, setup_context=_bias_setup_context)
@@ -217,13 +222,13 @@ def _differentiable(q, k, v, *, scale, mask_kind, window, prefix, doc_ids, alibi
                                     for c in range(0, v.size(3), d)], dim=-1))
         out = (parts[0] - lambda_full * parts[1]).to(q.dtype)
     elif biases:
-        if alibi_heads or softcap or doc_ids is not None:
-            raise NotImplementedError("gradients with bias operands are built for positional masks without ALiBi, soft-cap "
-                                      "or document ids")
+        if softcap and any(b.requires_grad for b, _ in biases):
+            raise NotImplementedError("gradients of bias operands are not built under a soft-cap (gradients of q, k and v "
+                                      "are: pass the operands detached)")
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
         out, _ = attn_fwd_bias_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
                                    int(prefix), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), dropout_p,
-                                   int(dropout_seed))
+                                   int(dropout_seed), doc_ids, int(alibi_heads), float(softcap))
     else:
         out, _ = attn_fwd_lse(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window),
                               int(prefix), doc_ids, int(alibi_heads), float(softcap), dropout_p, int(dropout_seed))

@@ -191,9 +191,9 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * softmax attention, recomputing the weights from the forward's row statistics.
  * `fwd` describes the forward call whose gradients are wanted: same q, k, v, sizes, scale, mask and score
  * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
- * kind, grouped-query heads, ALiBi, the tanh soft-cap (either of them under a document mask at head dims 64 and 128);
- * Dqk == Dv in {32, 64, 128}.  Bias operands (fwd.bias, as in the
- * forward) go with positional masks and dropout only, not with ALiBi, a soft-cap or a document mask.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
+ * kind, grouped-query heads, ALiBi, the tanh soft-cap and bias operands (fwd.bias, as in the forward) in any
+ * combination; Dqk == Dv in {32, 64, 128}.  Dropout (head dims 64 and 128) goes with one of ALiBi / soft-cap, a document
+ * mask or bias operands, the last under positional masks only.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
  * (both are compositions of calls that are supported: out * sigmoid(gate); one call per branch and half of the value
  * columns), the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]
@@ -213,7 +213,8 @@ typedef struct fl_attn_bwd_params {
    * loss with respect to the score of every (query, key) pair, i.e. with respect to whatever was added to q k^T * scale:
    * the gradient of a bias operand is this array summed over the axes (and batch entries) the operand broadcasts
    * over.  Only key tiles that some query of the workgroup attends are written (zeros where a pair is masked inside
-   * them): clear the array before the call. */
+   * them): clear the array before the call.  Not under a soft-cap (the bias is added after the cap, and the kernels
+   * keep only the gradient with respect to the capped product there). */
   float* dscores;
   int32_t reserved[6]; /* must be 0 */
 } fl_attn_bwd_params;

@@ -3,6 +3,7 @@ checker is autograd through the CPU oracle's eager functions, which `test_oracle
 pins against central differences in float64 (a wrong formula in the oracle, or in autograd's use of it, fails there).
 GPU tests compare the HIP kernels' gradients, through the C ABI, with those."""
 import ctypes as C
+import math
 
 import pytest
 import torch
@@ -87,7 +88,9 @@ def test_backward_abi_validation():
         (lambda b: setattr(b, "dout", 0xA0008), -7, "dout"),
         (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),
         (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
-                    setattr(b.fwd, "softcap", 30.0)), -4, "positional masks"),
+                    setattr(b.fwd, "softcap", 30.0), setattr(b, "dscores", 0xF0000)), -4, "soft-cap"),
+        (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
+                    setattr(b.fwd, "alibi_heads", 4), setattr(b.fwd, "dropout_threshold", 100)), -4, "dropout"),
         (lambda b: setattr(b, "dscores", 0xF0000), -5, "dscores"),
         (lambda b: (setattr(b.fwd, "gate", 0x70000), b.fwd.gate_strides.__setitem__(slice(0, 4), list(b.fwd.o_strides))),
          -4, "not supported"),
@@ -114,6 +117,37 @@ def test_backward_abi_validation():
     b = params(D=64, Dv=128)
     b.fwd.diff = 0
     assert rc(b) == -4
+
+
+def test_every_combination_of_score_modifications_has_a_backward_kernel():
+    """Mask kind x ALiBi x soft-cap x bias operands at head dims 32, 64 and 128, both element types (the gate and
+    differential attention are compositions around these calls)."""
+    import itertools
+    lib = _ffi.load_library()
+    for D, dtype in itertools.product((32, 64, 128), (_ffi.FL_BF16, _ffi.FL_F16)):
+        for kind, alibi, cap, bias in itertools.product(
+                (_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM, _ffi.MASK_DOCUMENT,
+                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2)):
+            b = _ffi.FlAttnBwdParams()
+            b.fwd = good_params(D=D)
+            f = b.fwd
+            f.dtype, f.mask_kind, f.window, f.prefix, f.alibi_heads, f.softcap = dtype, kind, 17, 40, alibi, cap
+            for i in range(bias):
+                f.bias[i], f.bias_batch_div[i], f.bias_dtype[i] = 0x60000 + 0x100000 * i, 1, dtype
+                f.bias_strides[i][:] = (0, 0, 304, 1) if i == 0 else (0, 0, 0, 1)
+            if kind in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):
+                f.doc_ids, f.doc_stride = 0x50000, 300
+                f.workspace, f.workspace_bytes = 0x80000, lib.fl_workspace_bytes(C.byref(f))
+            L, Hq, Hkv = f.Lq, f.Hq, f.Hkv
+            f.lse = 0x90000
+            b.dout, b.dq, b.dk, b.dv, b.delta = 0xA0000, 0xB0000, 0xC0000, 0xD0000, 0xE0000
+            b.dout_strides[:] = (Hq * L * D, L * D, D, 1)
+            b.dq_strides[:] = (Hq * L * D, L * D, D, 1)
+            b.dk_strides[:] = (Hkv * L * D, L * D, D, 1)
+            b.dv_strides[:] = (Hkv * L * D, L * D, D, 1)
+            if bias and not cap:
+                b.dscores = 0xF0000
+            assert lib.fl_attn_bwd_validate(C.byref(b)) == 0, (D, dtype, kind, alibi, cap, bias, _ffi.last_error())
 
 
 # ---- the kernels ---------------------------------------------------------------------------------------------------------------
@@ -376,6 +410,63 @@ def test_gradients_differential_attention(causal):
         res.append([out.detach()] + [t.grad for t in ts])
     torch.cuda.synchronize()
     _compare((f"diffattn causal={causal}", ("out", "dq", "dk", "dv")), res[0], res[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("kind", ["alibi", "softcap", "document", "document+alibi+softcap"])
+def test_gradients_bias_operands_with_other_score_modifications(D, kind):
+    """Bias operands together with the in-kernel ALiBi term, the soft-cap and document ids: gradients of q, k, v always,
+    of the operands too unless a soft-cap is on (the dense score_mod of alibi.py:26-30 with `softcap=`, and what the
+    graph rewrite composes)."""
+    from flashlight_amd import ops
+    from oracle.attention import _softmax_attention, alibi_slopes
+    B, Hq, Hkv, L = 2, 4, 2, 210
+    q, k, v, dout = _inputs(B, Hq, Hkv, L, D, seed=400 + D)
+    g = torch.Generator().manual_seed(D)
+    table = torch.randn(1, Hq, L, L, generator=g)
+    row = torch.randn(B, 1, 1, L, generator=g)
+    ids = torch.sort(torch.randint(0, 4, (B, L), generator=g), dim=1).values
+    alibi, cap, doc = "alibi" in kind, (9.0 if "softcap" in kind else None), "document" in kind
+    bias_grads = cap is None
+    # the kernels
+    qq, kk, vv = (t.detach().to(DEV).requires_grad_(True) for t in (q, k, v))
+    tb, rb = table.to(torch.bfloat16).to(DEV).requires_grad_(bias_grads), row.to(DEV).requires_grad_(bias_grads)
+    out = ops.dispatch(qq, kk, vv, mask_kind=_ffi.MASK_DOCUMENT_CAUSAL if doc else _ffi.MASK_CAUSAL,
+                       doc_ids=ids.to(DEV) if doc else None, alibi_heads=Hq if alibi else 0, softcap=cap or 0.0,
+                       biases=[(tb, B), (rb, 1)])
+    out.backward(dout.to(DEV))
+    # the oracle
+    qf, kf, vf = (t.detach().float().cpu().requires_grad_(True) for t in (q, k, v))
+    tf, rf = table.to(torch.bfloat16).float().requires_grad_(True), row.clone().requires_grad_(True)
+    slopes = alibi_slopes(Hq).float().view(1, Hq, 1, 1)
+
+    def masked(qi, ki):
+        m = ki > qi
+        return (m | (ids[:, qi.view(-1)].view(B, 1, -1, 1) != ids[:, ki.view(-1)].view(B, 1, 1, -1))) if doc else m
+
+    def bias(qi, ki):
+        return ([slopes * (ki - qi).float()] if alibi else []) + [tf[..., qi.view(-1), :], rf]
+
+    ref = _softmax_attention(qf, kf.repeat_interleave(Hq // Hkv, 1), vf.repeat_interleave(Hq // Hkv, 1), 1.0 / math.sqrt(D),
+                             masked=masked, bias=bias, softcap=cap)
+    ref.backward(dout.float().cpu())
+    names, got, want = ["out", "dq", "dk", "dv"], [out.detach(), qq.grad, kk.grad, vv.grad], [ref.detach(), qf.grad, kf.grad, vf.grad]
+    if bias_grads:
+        names += ["dtable", "drow"]
+        got += [tb.grad, rb.grad]
+        want += [tf.grad, rf.grad]
+    else:
+        with pytest.raises(NotImplementedError, match="soft-cap"):
+            ops.dispatch(qq, kk, vv, mask_kind=_ffi.MASK_CAUSAL, softcap=cap, biases=[(tb.detach().requires_grad_(True), B)])
+    torch.cuda.synchronize()
+    for what, g_, w_ in zip(names, got, want):
+        assert g_ is not None and tuple(g_.shape) == tuple(w_.shape), what
+        scale = max(1.0, w_.abs().max().item())
+        # (a bias gradient is a sum of score gradients over everything the operand broadcasts over: the bound grows with
+        # the square root of the number of summands)
+        fan = math.sqrt(B) if what == "dtable" else math.sqrt(Hq * L / 8) if what == "drow" else 1.0
+        assert_parity(g_.float() / scale, w_.float() / scale, f"{kind} D={D}: {what}", max_tol=2e-2 * fan, mean_tol=2e-3 * fan)
 
 
 @pytest.mark.gpu

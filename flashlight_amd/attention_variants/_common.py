@@ -41,9 +41,9 @@ class honor_dropout:
     softcap.py:4-53), and so do this package's by default.  `honor_dropout(True)` (also usable as a context manager:
     `with honor_dropout(): ...`) makes them apply it: softmax weights are dropped with probability `dropout_p` and the
     kept ones scaled by 1 / (1 - p), as torch.nn.functional.dropout would.  Seeds come from torch's default CPU
-    generator.  The kernels have dropout for positional masks with the in-kernel ALiBi term and the soft-cap, for
-    document masks, and for dense bias operands (a `score_mod` tensor) without a soft-cap: the causal, ALiBi, soft-cap
-    and document-mask variants take it; a dense `score_mod` tensor together with a soft-cap and dropout_p > 0 raises."""
+    generator.  The kernels have dropout for every mask kind with the in-kernel ALiBi term, the soft-cap and dense bias
+    operands (a `score_mod` tensor) in any combination, at head dims up to 128: the causal, ALiBi, soft-cap and
+    document-mask variants take it."""
 
     def __init__(self, enabled: bool = True):
         global _honor_dropout

@@ -350,11 +350,6 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
       return fail(FL_ERR_ARG, "dropout_threshold must be at most 65535 (rate 65535/65536), got %u", p->dropout_threshold);
     if (p->diff || p->attended_dump)
       return fail(FL_ERR_UNSUPPORTED, "dropout is not built for differential attention and the dump hook");
-    const bool dense = p->bias[0] || p->bias[1] || p->gate;
-    const bool mods = p->alibi_heads > 0 || p->softcap > 0.f;
-    if ((is_doc(p->mask_kind) && (mods || dense)) || (mods && dense))
-      return fail(FL_ERR_UNSUPPORTED, "dropout is built with one of: ALiBi and / or the soft-cap, a document mask, bias operands "
-                                      "and / or the gate (each under any positional mask), not with two of them");
   }
   if (p->lse) {
     if (reinterpret_cast<uintptr_t>(p->lse) % 4) return fail(FL_ERR_ALIGN, "lse must be 4-byte aligned");
@@ -772,8 +767,6 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
     return fail(FL_ERR_UNSUPPORTED, "backward: gate, differential attention and the dump hook are not supported");
   if (p->score_fn != FL_SCORE_NONE) return fail(FL_ERR_UNSUPPORTED, "backward: score_fn is forward-only");
   const bool has_bias = p->bias[0] || p->bias[1];
-  if (has_bias && p->dropout_threshold && (p->alibi_heads > 0 || p->softcap > 0.f || is_doc(p->mask_kind)))
-    return fail(FL_ERR_UNSUPPORTED, "backward: dropout with bias operands goes with positional masks only (no ALiBi, soft-cap or document mask)");
   if (b->dscores && p->softcap > 0.f)
     return fail(FL_ERR_UNSUPPORTED, "backward: dscores is not produced under a soft-cap (gradients of bias operands added after the cap)");
   if (b->dscores && !has_bias) return fail(FL_ERR_ARG, "backward: dscores is only written for calls with bias operands");
@@ -800,7 +793,7 @@ static int validate_bwd(const fl_attn_bwd_params* b, const fl::BwdInstance** out
   if (p->alibi_heads > 0 || p->softcap > 0.f) want = fl::F_ALIBI | fl::F_SOFTCAP;
   if (is_doc(p->mask_kind)) want |= fl::F_DOC;
   if (has_bias) want |= fl::F_BIAS;
-  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // validate() allows one of document mask, ALiBi / soft-cap, bias operands
+  if (p->dropout_threshold) want |= fl::F_DROPOUT;  // (head dims 64 and 128)
   const fl::BwdInstance* in = nullptr;
   for (int i = 0; i < fl::kNumBwdInstances; ++i)
     if (fl::kBwdInstances[i].d == p->Dqk && fl::kBwdInstances[i].feat == want && fl::kBwdInstances[i].dtype == p->dtype)

@@ -44,9 +44,8 @@ hipError_t launch_delta(const BParams& bp, hipStream_t stream) {
 // (D, FEAT) pairs with compiled backward kernels.  FEAT 3 = ALiBi and/or soft-cap (either may be off at run time),
 // 4 = bias operands, 8 = document ids in the element predicate, 11 = document ids with ALiBi and/or a soft-cap,
 // 7, 12, 15 = bias operands with ALiBi / soft-cap, with document ids, with both,
-// 128 = dropout, 131 = dropout with ALiBi and/or a soft-cap, 132 = dropout with bias operands,
-// 136 = dropout with document ids.
-#define FL_BWD_LIST(X) X(32, 0) X(32, 3) X(32, 4) X(32, 7) X(32, 8) X(32, 11) X(32, 12) X(32, 15) X(64, 0) X(64, 3) X(64, 4) X(64, 7) X(64, 8) X(64, 11) X(64, 12) X(64, 15) X(64, 128) X(64, 131) X(64, 132) X(64, 136) X(128, 0) X(128, 3) X(128, 4) X(128, 7) X(128, 8) X(128, 11) X(128, 12) X(128, 15) X(128, 128) X(128, 131) X(128, 132) X(128, 136)
+// 128 + any of these = the same with dropout (head dims 64 and 128).
+#define FL_BWD_LIST(X) X(32, 0) X(32, 3) X(32, 4) X(32, 7) X(32, 8) X(32, 11) X(32, 12) X(32, 15) X(64, 0) X(64, 3) X(64, 4) X(64, 7) X(64, 8) X(64, 11) X(64, 12) X(64, 15) X(64, 128) X(64, 131) X(64, 132) X(64, 135) X(64, 136) X(64, 139) X(64, 140) X(64, 143) X(128, 0) X(128, 3) X(128, 4) X(128, 7) X(128, 8) X(128, 11) X(128, 12) X(128, 15) X(128, 128) X(128, 131) X(128, 132) X(128, 135) X(128, 136) X(128, 139) X(128, 140) X(128, 143)
 
 // Every (D, FEAT) pair is compiled for bf16 and for fp16 elements (suffix _bf16 / _f16).
 #define FL_BWD_DECL_(D, FEAT, SFX)                                            \

@@ -122,7 +122,6 @@ void bwd_kernel(const BParams p) {
   constexpr uint32_t FEAT = T::FEAT;
   constexpr bool kAlibi = FEAT & F_ALIBI, kSoftcap = FEAT & F_SOFTCAP, kDoc = FEAT & F_DOC, kBias = FEAT & F_BIAS;
   constexpr bool kDQ = ROLE == ROLE_DQ;
-  static_assert(!kBias || !((kAlibi || kSoftcap || kDoc) && (FEAT & F_DROPOUT)), "dropout with bias operands goes with positional masks only");
   using E = typename T::Elem;  // pointers in BParams are typed bf16_t whatever E is: 16 opaque bits
   typedef E ex8 __attribute__((ext_vector_type(8)));
   typedef E ex4 __attribute__((ext_vector_type(4)));

@@ -22,8 +22,8 @@ Masks and biases are recognised by what they compute, not by how they were writt
   * a constant bias equal to 2^(-8 (h + 1) / H) * (k - q) is ALiBi and is computed inside the kernel; other biases are
     passed to the kernel's bias operands (fp32 or bf16).
 A training-mode dropout on the softmax weights becomes the kernel's own dropout (same rate, the kernel's random
-stream, a fresh seed per call) where the dropout kernels cover the region: one of ALiBi / soft-cap, a document mask or
-dense operands, head dims up to 128.  Regions that do not fit (a softmax whose weights are used elsewhere, dropout
+stream, a fresh seed per call) where the dropout kernels cover the region: head dims up to 128, no score function
+other than the soft-cap.  Regions that do not fit (a softmax whose weights are used elsewhere, dropout
 outside that coverage, ...) are left untouched.
 """
 from __future__ import annotations
@@ -721,11 +721,10 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                 else:
                     run_biases.append(node)
             if r.dropout_p:
-                # the dropout kernels cover one family at a time and head dims up to 128 (padded to 64 or 128)
-                families = [bool(kwargs["alibi_heads"] or r.softcap), doc_ids is not None,
-                            bool(run_masks or const_biases or run_biases)]
+                # the dropout kernels cover head dims up to 128 (padded to 64 or 128) and every score modification but the
+                # score functions
                 E, Ev = _val(r.q).size(-1), _val(r.v).size(-1)
-                if sum(families) > 1 or not plain or max(E, Ev) > 128:
+                if not plain or max(E, Ev) > 128:
                     raise _NoMatch("dropout together with this combination of score modifications or head dims")
                 kwargs["dropout_p"] = r.dropout_p
         except _NoMatch:

@@ -304,9 +304,6 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     if dropout_p > 0.0:
         if diff or seq_major_out:
             raise NotImplementedError("dropout is not built for differential attention and sequence-major results")
-        if (biases or gate is not None) and (alibi_heads or softcap or doc_ids is not None):
-            raise NotImplementedError("dropout with bias operands or the gate is built without the in-kernel ALiBi term, the "
-                                      "soft-cap and document ids")
         if dropout_seed is None:
             if torch.compiler.is_compiling():
                 raise NotImplementedError("dropout under torch.compile needs an explicit dropout_seed (a seed drawn "

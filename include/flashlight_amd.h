@@ -120,9 +120,8 @@ typedef struct fl_attn_params {
    * ignore it (attention_variants/causal.py:4-36, alibi.py:13-33, softcap.py:4-53); 0 here does the same.
    * dropout_threshold = round(p * 65536), 1 .. 65535: a weight is dropped when the 16 bits a counter-based hash of
    * (dropout_seed, batch * Hq + head, query, key) gives it are below the threshold.  fl_attn_bwd regenerates the same
-   * decisions from the same fields.  With any positional mask and GQA, together with one of: ALiBi and / or the soft-cap;
-   * a document mask; bias operands and / or the gate.  Not with two of these, differential attention or the dump hook;
-   * Dqk = Dv in {64, 128}. */
+   * decisions from the same fields.  With every mask kind, GQA, ALiBi, the soft-cap, bias operands and the gate, in any
+   * combination; not with differential attention, score_fn or the dump hook; Dqk = Dv in {64, 128}. */
   uint32_t dropout_threshold;
   uint32_t dropout_seed[2]; /* low, high half of a 64-bit seed */
 
@@ -192,8 +191,8 @@ int fl_attn_plan(const fl_attn_params* p, int64_t out[8]);
  * `fwd` describes the forward call whose gradients are wanted: same q, k, v, sizes, scale, mask and score
  * modification; fwd.o is the forward's output and fwd.lse the row statistics that call wrote.  Supported: every mask
  * kind, grouped-query heads, ALiBi, the tanh soft-cap and bias operands (fwd.bias, as in the forward) in any
- * combination; Dqk == Dv in {32, 64, 128}.  Dropout (head dims 64 and 128) goes with one of ALiBi / soft-cap, a document
- * mask or bias operands, the last under positional masks only.  Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
+ * combination, with or without dropout (dropout: head dims 64 and 128); Dqk == Dv in {32, 64, 128}.
+ * Not supported (FL_ERR_UNSUPPORTED): gate, differential attention
  * (both are compositions of calls that are supported: out * sigmoid(gate); one call per branch and half of the value
  * columns), the attended_dump hook.
  * dout [B, Hq, Lq, Dv] is the gradient of the output; dq [B, Hq, Lq, Dqk], dk [B, Hkv, Lk, Dqk], dv [B, Hkv, Lk, Dv]

@@ -56,16 +56,18 @@ def rc(lib, p):
 
 
 def test_every_combination_of_score_modifications_has_a_kernel(lib):
-    """Mask kind x ALiBi x soft-cap x bias operands x gate, at every compiled head dim and in both element types: the
+    """Mask kind x ALiBi x soft-cap x bias operands x gate (x dropout at head dims 64 and 128), at every compiled head
+    dim and in both element types: the
     reference's functions compose these freely (attention_variants/*.py are plain PyTorch), so no combination of them
     may end in "no kernel instance"."""
     import itertools
     for (D, Dv), dtype in itertools.product(((32, 32), (64, 64), (128, 128), (256, 128), (512, 128)), (_ffi.FL_BF16, _ffi.FL_F16)):
-        for kind, alibi, cap, bias, gate in itertools.product(
+        for kind, alibi, cap, bias, gate, drop in itertools.product(
                 (_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM, _ffi.MASK_DOCUMENT,
-                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2), (False, True)):
+                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2), (False, True), (0, 6554) if D in (64, 128) else (0,)):
             p = good_params(D=D, Dv=Dv)
             p.dtype = dtype
+            p.dropout_threshold = drop  # (dropout kernels exist at head dims 64 and 128)
             p.mask_kind, p.window, p.prefix = kind, 17, 40
             p.alibi_heads, p.softcap = alibi, cap
             for i in range(bias):
@@ -77,7 +79,7 @@ def test_every_combination_of_score_modifications_has_a_kernel(lib):
             if kind in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):
                 p.doc_ids, p.doc_stride = 0x50000, 300
                 p.workspace, p.workspace_bytes = 0x80000, lib.fl_workspace_bytes(C.byref(p))
-            assert rc(lib, p) == 0, (D, Dv, dtype, kind, alibi, cap, bias, gate, _ffi.last_error())
+            assert rc(lib, p) == 0, (D, Dv, dtype, kind, alibi, cap, bias, gate, drop, _ffi.last_error())
 
 
 def test_valid_params_pass(lib):

@@ -89,8 +89,6 @@ def test_backward_abi_validation():
         (lambda b: b.dk_strides.__setitem__(2, 62), -7, "dk"),
         (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
                     setattr(b.fwd, "softcap", 30.0), setattr(b, "dscores", 0xF0000)), -4, "soft-cap"),
-        (lambda b: (b.fwd.bias.__setitem__(0, 0x60000), b.fwd.bias_batch_div.__setitem__(0, 1),
-                    setattr(b.fwd, "alibi_heads", 4), setattr(b.fwd, "dropout_threshold", 100)), -4, "dropout"),
         (lambda b: setattr(b, "dscores", 0xF0000), -5, "dscores"),
         (lambda b: (setattr(b.fwd, "gate", 0x70000), b.fwd.gate_strides.__setitem__(slice(0, 4), list(b.fwd.o_strides))),
          -4, "not supported"),
@@ -120,18 +118,19 @@ def test_backward_abi_validation():
 
 
 def test_every_combination_of_score_modifications_has_a_backward_kernel():
-    """Mask kind x ALiBi x soft-cap x bias operands at head dims 32, 64 and 128, both element types (the gate and
-    differential attention are compositions around these calls)."""
+    """Mask kind x ALiBi x soft-cap x bias operands (x dropout from head dim 64 up) at head dims 32, 64 and 128, both
+    element types (the gate and differential attention are compositions around these calls)."""
     import itertools
     lib = _ffi.load_library()
     for D, dtype in itertools.product((32, 64, 128), (_ffi.FL_BF16, _ffi.FL_F16)):
-        for kind, alibi, cap, bias in itertools.product(
+        for kind, alibi, cap, bias, drop in itertools.product(
                 (_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM, _ffi.MASK_DOCUMENT,
-                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2)):
+                 _ffi.MASK_DOCUMENT_CAUSAL), (0, 4), (0.0, 30.0), (0, 1, 2), (0, 6554) if D > 32 else (0,)):
             b = _ffi.FlAttnBwdParams()
             b.fwd = good_params(D=D)
             f = b.fwd
             f.dtype, f.mask_kind, f.window, f.prefix, f.alibi_heads, f.softcap = dtype, kind, 17, 40, alibi, cap
+            f.dropout_threshold = drop
             for i in range(bias):
                 f.bias[i], f.bias_batch_div[i], f.bias_dtype[i] = 0x60000 + 0x100000 * i, 1, dtype
                 f.bias_strides[i][:] = (0, 0, 304, 1) if i == 0 else (0, 0, 0, 1)
@@ -147,7 +146,7 @@ def test_every_combination_of_score_modifications_has_a_backward_kernel():
             b.dv_strides[:] = (Hkv * L * D, L * D, D, 1)
             if bias and not cap:
                 b.dscores = 0xF0000
-            assert lib.fl_attn_bwd_validate(C.byref(b)) == 0, (D, dtype, kind, alibi, cap, bias, _ffi.last_error())
+            assert lib.fl_attn_bwd_validate(C.byref(b)) == 0, (D, dtype, kind, alibi, cap, bias, drop, _ffi.last_error())
 
 
 # ---- the kernels ---------------------------------------------------------------------------------------------------------------

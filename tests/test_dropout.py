@@ -181,15 +181,21 @@ def test_abi_validation_of_dropout_fields():
         p.dropout_threshold = 100
         mutate(p)
         assert rc(p) == 0, _ffi.last_error()
-    for mutate in (lambda p: (doc(p), setattr(p, "alibi_heads", 4)),
-                   lambda p: (doc(p), setattr(p, "softcap", 30.0)),
-                   lambda p: (doc(p), dense(p)),
-                   lambda p: (dense(p), setattr(p, "softcap", 30.0)),
-                   lambda p: setattr(p, "diff", 1)):
+    # ... and so does every combination of them (the workspace size follows the kernel chosen: ids last)
+    for mutate in (lambda p: (setattr(p, "alibi_heads", 4), doc(p)),
+                   lambda p: (setattr(p, "softcap", 30.0), doc(p)),
+                   lambda p: (dense(p), doc(p)),
+                   lambda p: (dense(p), setattr(p, "softcap", 30.0))):
         p = good_params()
         p.dropout_threshold = 100
         mutate(p)
-        assert rc(p) == -4 and "dropout" in _ffi.last_error(), _ffi.last_error()
+        assert rc(p) == 0, _ffi.last_error()
+    for mutate in (lambda p: setattr(p, "diff", 1),
+                   lambda p: (setattr(p, "score_fn", _ffi.SCORE_CLAMP), p.score_fn_params.__setitem__(slice(0, 4), [1.0, 0.0, -1.0, 1.0]))):
+        p = good_params()
+        p.dropout_threshold = 100
+        mutate(p)
+        assert rc(p) == -4, _ffi.last_error()
     p = good_params(D=32)  # no dropout kernel at head dim 32
     p.dropout_threshold = 100
     assert rc(p) == -4, _ffi.last_error()
@@ -206,10 +212,8 @@ def test_front_end_switch_and_refusals():
     assert "dropout" not in str(e.value)
     with pytest.raises(NotImplementedError, match="dropout"):
         ops.dispatch(q, q, q, dropout_p=0.1, diff=True)
-    with pytest.raises(NotImplementedError, match="dropout"):  # bias operands or the gate: not with ALiBi / soft-cap / ids
-        ops.dispatch(q, q, q, dropout_p=0.1, gate=q, softcap=5.0)
-    with pytest.raises(NotImplementedError, match="dropout"):
-        ops.dispatch(q, q, q, dropout_p=0.1, biases=[(torch.zeros(1, 1, 8, 8), 1)], alibi_heads=2)
+    with pytest.raises(NotImplementedError, match="dropout"):  # score functions take no dropout
+        ops.dispatch(q, q, q, dropout_p=0.1, score_fn=(_ffi.SCORE_CLAMP, (1.0, 0.0, -1.0, 1.0)))
     with pytest.raises(ValueError, match="dropout_p"):
         ops.dispatch(q, q, q, dropout_p=1.5)
     with A.honor_dropout():
@@ -413,13 +417,16 @@ def _random_dropout_case(seed):
     Hkv, G, B = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 4]), rnd.choice([1, 2])
     L = rnd.choice([1, 33, 64, 100, 129, 200, 257, 384, 450])
     S = L if rnd.random() < 0.6 else rnd.choice([17, 64, 150, 300])
-    family = rnd.choice(["plain", "mods", "document", "bias"])
+    family = rnd.choice(["plain", "mods", "document", "bias", "all", "all"])
     mask_kind = rnd.choice([_ffi.MASK_NONE, _ffi.MASK_CAUSAL, _ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM])
+    if family == "all" and rnd.random() < 0.5:
+        mask_kind = rnd.choice([_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL])
     if mask_kind in (_ffi.MASK_SLIDING, _ffi.MASK_PREFIX_LM):
         S = L  # (as in the reference: these masks are defined for equal lengths)
     if family == "document":
-        S = L
         mask_kind = rnd.choice([_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL])
+    if mask_kind in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):
+        S = L
     return dict(seed=seed, D=D, Hkv=Hkv, G=G, B=B, L=L, S=S, family=family, mask_kind=mask_kind,
                 window=rnd.choice([1, 31, 70, 128]), prefix=rnd.choice([1, 32, 50, 129]), p=rnd.choice([0.05, 0.3, 0.7]),
                 alibi=rnd.random() < 0.6, cap=rnd.choice([None, 4.0, 25.0]), ndocs=rnd.choice([1, 3, 7]),
@@ -427,11 +434,11 @@ def _random_dropout_case(seed):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed", range(500, 540))
+@pytest.mark.parametrize("seed", range(500, 580))
 def test_random_dropout_cases(seed):
-    """Seeded draws over the families the dropout kernels are built for (positional masks alone, with ALiBi / soft-cap,
-    document masks, bias operands), ragged and unequal lengths, grouped heads, both element types: forward and
-    gradients against autograd through the oracle with the same seed."""
+    """Seeded draws over what the dropout kernels cover (every mask kind; ALiBi, soft-cap, bias operands, alone and all
+    together), ragged and unequal lengths, grouped heads, both element types: forward and gradients against autograd
+    through the oracle with the same seed."""
     import oracle as O
     c = _random_dropout_case(seed)
     B, Hkv, Hq, L, S, D, p = c["B"], c["Hkv"], c["Hkv"] * c["G"], c["L"], c["S"], c["D"], c["p"]
@@ -442,14 +449,15 @@ def test_random_dropout_cases(seed):
     kw = dict(mask_kind=c["mask_kind"], window=c["window"], prefix=c["prefix"], dropout_p=p, dropout_seed=seed * 0x9E3779B97F4A7 + 1)
     attend = _attend(c["mask_kind"], L, S, c["window"], c["prefix"])
     bias, cap, operand = None, None, None
-    if c["family"] == "mods":
+    fam = c["family"]
+    if fam in ("mods", "all"):
         cap = c["cap"]
         if c["alibi"] or cap is None:
             rel = (torch.arange(S)[None, :] - torch.arange(L)[:, None]).float()
             bias = O.alibi_slopes(Hq)[:, None, None] * rel[None]
             kw["alibi_heads"] = Hq
         kw["softcap"] = cap or 0.0
-    elif c["family"] == "document":
+    if c["mask_kind"] in (_ffi.MASK_DOCUMENT, _ffi.MASK_DOCUMENT_CAUSAL):
         ids = torch.sort(torch.randint(0, c["ndocs"], (B, L), generator=g), dim=1).values
         if seed % 3 == 0:
             ids = ids[:, torch.randperm(L, generator=g)]
@@ -457,10 +465,10 @@ def test_random_dropout_cases(seed):
         attend = (ids[:, :, None] == ids[:, None, :])[:, None]
         if c["mask_kind"] == _ffi.MASK_DOCUMENT_CAUSAL:
             attend = attend & (torch.arange(L)[None, :] <= torch.arange(L)[:, None])
-    elif c["family"] == "bias":
+    if fam in ("bias", "all"):
         operand = torch.randn(1, Hq, L, S, generator=g).to(dt).to(DEV)
         kw["biases"] = [(operand, 1)]
-        bias = operand.float().cpu()
+        bias = operand.float().cpu() if bias is None else bias + operand.float().cpu()
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=DEV)
     out = _ffi.attn_fwd(q, k, v, lse=lse, **kw)
     dq, dk, dv = _ffi.attn_bwd(q, k, v, out, lse, dout, **kw)
@@ -512,8 +520,8 @@ def test_dropout_through_autograd_and_the_variant_switch():
         torch.manual_seed(11)
         d = A.attention_pytorch_alibi(q, k, v, score_mod=dense, dropout_p=0.5, enable_gqa=True, is_causal=True)
         assert torch.equal(d, a)  # a zero bias and the same seed: the same weights are dropped
-        with pytest.raises(NotImplementedError, match="dropout"):  # not together with the soft-cap
-            A.attention_pytorch_alibi(q, k, v, score_mod=dense, dropout_p=0.1, enable_gqa=True, softcap=5.0)
+        e = A.attention_pytorch_alibi(q, k, v, score_mod=dense, dropout_p=0.5, enable_gqa=True, softcap=5.0)
+        assert torch.isfinite(e).all() and not torch.equal(e, a)  # with a soft-cap too
     # autograd: the backward regenerates the forward's decisions from the seed
     qg, kg, vg = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
     out = ops.dispatch(qg, kg, vg, mask_kind=_ffi.MASK_CAUSAL, dropout_p=0.3, dropout_seed=2024)

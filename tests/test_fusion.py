@@ -198,7 +198,7 @@ def test_rewrite_maps_training_mode_dropout_to_the_kernel():
     assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.2 and len(calls[0].args[4]) == 1
     gm, calls = _rewrite(E.documents_with_dropout, q, k, v, _ids(2, 48))
     assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_DOCUMENT
-    # outside what the dropout kernels cover the region stays eager: head dims above 128; a bias together with a soft-cap
+    # outside what the dropout kernels cover the region stays eager: head dims above 128, score functions
     q256, k256, v256 = _qkv(E=256)
     gm, calls = _rewrite(E.causal_with_dropout, q256, k256, v256)
     assert calls == [] and "dropout" in {fusion._name(n) for n in gm.graph.nodes}
@@ -218,6 +218,11 @@ def test_rewrite_maps_training_mode_dropout_to_the_kernel():
         w = torch.softmax(20.0 * torch.tanh(q @ k.transpose(-2, -1) * 0.125 / 20.0) + b, dim=-1)
         return torch.nn.functional.dropout(w, 0.1) @ v
     gm, calls = _rewrite(capped_bias_dropout, q, k, v, torch.randn(4, 48, 48))
+    assert len(calls) == 1 and calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["softcap"] == 20.0
+
+    def relu_dropout(q, k, v):  # score functions have no dropout kernels: left eager
+        return torch.nn.functional.dropout(torch.softmax(torch.relu(q @ k.transpose(-2, -1) * 0.125), dim=-1), 0.1) @ v
+    gm, calls = _rewrite(relu_dropout, q, k, v)
     assert calls == []
 
 

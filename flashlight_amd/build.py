@@ -148,7 +148,25 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
     tmp = PROBE_LIB_PATH.with_suffix(".so.tmp")
     _compile(([cc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", str(probe_obj), "-o", str(tmp)], tmp))
     os.replace(tmp, PROBE_LIB_PATH)
+    build_c_host()
     return LIB_PATH
+
+
+C_HOST_SRC = PKG_DIR.parent / "tests" / "c_host" / "attn_host.c"
+C_HOST_BIN = C_HOST_SRC.with_suffix("")
+
+
+def build_c_host() -> Path | None:
+    """The plain-C host program of the test suite (tests/c_host/attn_host.c): C99, gcc, linked against the library just
+    built and the HIP runtime.  Skipped when the source is not there (a copy of the package alone)."""
+    if not C_HOST_SRC.exists() or LIB_PATH.parent != PKG_DIR:
+        return None
+    rocm = Path(hipcc()).resolve().parent.parent
+    cmd = [shutil.which("gcc") or "gcc", "-std=c99", "-O1", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__",
+           f"-I{rocm / 'include'}", f"-I{INCLUDE}", str(C_HOST_SRC), "-o", str(C_HOST_BIN), f"-L{PKG_DIR}", "-lflashlight_amd",
+           f"-L{rocm / 'lib'}", "-lamdhip64", "-lm", "-Wl,-rpath,$ORIGIN/../../flashlight_amd", f"-Wl,-rpath,{rocm / 'lib'}"]
+    _compile((cmd, C_HOST_BIN))
+    return C_HOST_BIN
 
 
 if __name__ == "__main__":

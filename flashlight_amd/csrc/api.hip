@@ -443,8 +443,9 @@ int validate(const fl_attn_params* p, const fl::Instance** out, bool for_bwd = f
 }
 
 // Whether *p (already validated) is a call the shared-bias streaming forward covers: head dim 32, no mask or other
-// score modification, exactly one dense 16-bit bias operand that several consecutive batch entries share, 256 / 320 /
-// 384 keys.  Fills the kernel's parameters and launch shape.
+// score modification, one dense 16-bit bias operand that several consecutive batch entries share (and optionally one
+// row of keys per batch entry), a key count the kernel is compiled for (pairbias_has_shape).  Fills the kernel's
+// parameters and launch shape.
 bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
   static const bool disabled = std::getenv("FL_NO_PAIRBIAS") != nullptr;  // A/B knob: the general kernel instead
   if (disabled) return false;
@@ -458,7 +459,7 @@ bool plan_pairbias(const fl_attn_params* p, fl::PParams* out, int* grid) {
     if (!p->bias[i]) continue;
     const int64_t* st = p->bias_strides[i];
     if (p->bias_dtype[i] != p->dtype || st[3] != 1) return false;
-    if (p->bias_batch_div[i] >= 2 && st[1] != 0 && st[2] != 0 && pi < 0) pi = i;
+    if (p->bias_batch_div[i] >= 2 && (st[1] != 0 || p->Hq == 1) && st[2] != 0 && pi < 0) pi = i;  // (one head: no head stride)
     else if (p->bias_batch_div[i] == 1 && st[1] == 0 && st[2] == 0 && ri < 0) ri = i;
     else return false;
   }

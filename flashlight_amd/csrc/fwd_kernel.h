@@ -1036,11 +1036,17 @@ void fwd_kernel(const KParams p) {
       if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-          const float m_new = __builtin_fmaxf(m_run[qb], mx[qb]);
+          // Before the first update the reference is 0 (see softmax_p), and tiles may already have been accumulated
+          // against it without this function being called (the reference-free path).  The reference then never moves
+          // below 0: a tile whose every key carries a huge finite negative term (an additive padding mask such as
+          // -1e9 over a ragged last tile) would otherwise pull it down there and scale the accumulated weights up
+          // past the largest float.  With nothing accumulated yet the tile's own maximum is taken, whatever it is.
+          const bool fresh = m_run[qb] == -INFINITY;
+          const float floor_ = (fresh && xhalf_sum(l_run[qb]) > 0.f) ? 0.f : m_run[qb];
+          const float m_new = __builtin_fmaxf(floor_, mx[qb]);
           const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // row fully masked so far
-          // before the first update the reference is 0 (see softmax_p); the clamp keeps 0 * inf out of accumulators
-          // whose contents have underflowed to nothing
-          const float m_old = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
+          // (the clamp keeps 0 * inf out of accumulators whose contents have underflowed to nothing)
+          const float m_old = fresh ? 0.f : m_run[qb];
           const float alpha = __builtin_fminf(fast_exp2((m_old - m_use) * c2), 0x1p126f);
           m_run[qb] = m_new;
           l_run[qb] *= alpha;

@@ -268,6 +268,32 @@ def test_head_dim_32_score_functions_and_dropout_run_on_the_64_wide_kernels():
     assert_parity(out, OD.attention_dropout(qf, kf, vf, keep, 0.25, attend=causal), "dropout at head dim 32")
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("fill", [-1e9, -30000.0, float("-inf")])
+def test_additive_padding_mask_over_a_ragged_last_tile(D, dtype, fill):
+    """Key padding written as an additive term (a large finite negative number, as model code does, or -inf) that covers
+    the whole ragged last tile of every sequence: the softmax reference must not follow such a tile down (it once did
+    when nothing had moved it yet, and scaled what was accumulated past the largest float: NaN)."""
+    B, Hq, Hkv = 3, 4, 2
+    for S, valid in ((100, (90, 37, 96)), (200, (150, 190, 64)), (333, (320, 100, 288))):
+        q, k, v = (t.to(dtype) for t in qkv(B, Hq, Hkv, S, D, seed=S + D))
+        pad = torch.zeros(B, 1, 1, S)
+        for b, n in enumerate(valid):
+            pad[b, ..., n:] = fill
+        for operand in (pad, pad.to(dtype)):  # fp32, and the element type (fp16 turns -1e9 into -inf)
+            out = ops.dispatch(q, k, v, biases=[(operand.to(DEV), 1)])
+            qf, kf, vf = f32(q, k, v)
+            ref = _softmax_attention(qf, kf.repeat_interleave(Hq // Hkv, 1), vf.repeat_interleave(Hq // Hkv, 1),
+                                     1.0 / math.sqrt(D), bias=lambda qi, ki: operand.float())
+            assert_parity(out, ref, f"D={D} S={S} {dtype} fill={fill} operand {operand.dtype}")
+            # the same under the causal mask (the first tile of early rows is then the masked diagonal one)
+            out = ops.dispatch(q, k, v, mask_kind=_ffi.MASK_CAUSAL, biases=[(operand.to(DEV), 1)])
+            ref = _softmax_attention(qf, kf.repeat_interleave(Hq // Hkv, 1), vf.repeat_interleave(Hq // Hkv, 1),
+                                     1.0 / math.sqrt(D), masked=lambda qi, ki: ki > qi, bias=lambda qi, ki: operand.float())
+            assert_parity(out, ref, f"causal D={D} S={S} {dtype} fill={fill} operand {operand.dtype}")
+
+
 def test_score_mod_the_kernel_cannot_apply_is_refused():
     q, k, v = qkv(1, 2, 2, 64, 64, seed=50)
     for fn in (lambda s, b, h, qi, ki: torch.exp(s),

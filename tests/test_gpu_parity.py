@@ -624,6 +624,10 @@ def test_config0_shape_causal():
     (1, 2, 256, 8, False, torch.bfloat16, False),    # two rows: chunks of one entry
     (1, 21, 320, 2, False, torch.bfloat16, False),   # five tiles per entry without a gate
     (1, 40, 384, 4, False, torch.float16, False),    # six tiles per entry without a gate, fp16
+    (2, 11, 128, 4, True, torch.bfloat16, False),    # two tiles per entry: the ring runs three entries ahead
+    (1, 23, 128, 2, False, torch.float16, True),
+    (1, 17, 192, 8, True, torch.bfloat16, True),     # three tiles per entry
+    (3, 6, 192, 1, False, torch.bfloat16, False),
 ])
 def test_shared_bias_streaming_kernel(B, N, S, H, gate, dtype, inf):
     g = torch.Generator().manual_seed(31)
@@ -676,6 +680,11 @@ def test_shared_bias_streaming_kernel_half_masked_lanes(dtype, drop):
     (32, 1, 13, 384, 8, True, torch.bfloat16, "1e9", None),      # head dim 32 with mask bias, pair bias and gate
     (32, 2, 7, 256, 4, False, torch.bfloat16, "inf", None),
     (32, 1, 10, 320, 2, True, torch.float16, "randn", None),
+    (32, 2, 9, 128, 4, True, torch.bfloat16, "inf", None),       # 128 and 192 keys, both head dims
+    (32, 1, 14, 192, 2, False, torch.float16, "1e9", 0.2),
+    (64, 1, 12, 128, 4, False, torch.bfloat16, "1e9", None),
+    (64, 2, 7, 192, 2, False, torch.bfloat16, "randn", 0.1),
+    (64, 1, 3, 192, 8, False, torch.float16, "inf", None),
 ])
 def test_shared_bias_streaming_kernel_with_a_row_bias(D, B, N, S, H, gate, dtype, mask, scale):
     # two operands: a row of keys per batch entry (the reference's mask bias [B, N, 1, 1, S]) and the shared pair bias

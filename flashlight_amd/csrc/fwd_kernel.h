@@ -1034,6 +1034,9 @@ void fwd_kernel(const KParams p) {
       for (int qb = 0; qb < QB; ++qb)
         grow = grow | ((mx[qb] - m_run[qb]) * c2 > kTau);  // m_run = -inf before the first tile: always true
       if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+        // (in the units of the scores: s * c2 is in log2 units; worked out here, on the rare path, so that it does not
+        // hold a register through the loop)
+        const float ref_floor = kBias ? -32768.0f * fast_rcp(c2) : 0.f;
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
           // Before the first update the reference is 0 (see softmax_p), and tiles may already have been accumulated
@@ -1043,7 +1046,14 @@ void fwd_kernel(const KParams p) {
           // past the largest float.  With nothing accumulated yet the tile's own maximum is taken, whatever it is.
           const bool fresh = m_run[qb] == -INFINITY;
           const float floor_ = (fresh && xhalf_sum(l_run[qb]) > 0.f) ? 0.f : m_run[qb];
-          const float m_new = __builtin_fmaxf(floor_, mx[qb]);
+          // Nor does it go below -2^15 log2 units: scores further down are additive masks written as finite numbers
+          // (-1e9, the element type's most negative value), all of whose weights are zero against any real score.
+          // Taken as the reference they would be subtracted from themselves with the rounding of their own magnitude
+          // (2^+-64 instead of 1 at -1e9, inf - inf at -3e38); held against this floor their weights are plain zeros.
+          // (a row that is fully masked so far takes the floor as its reference too: whatever comes next is above it).
+          // Only bias operands bring such numbers: the other kernels keep the plain maximum.
+          float m_new = __builtin_fmaxf(floor_, mx[qb]);
+          if constexpr (kBias) m_new = __builtin_fmaxf(m_new, ref_floor);
           const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // row fully masked so far
           // (the clamp keeps 0 * inf out of accumulators whose contents have underflowed to nothing)
           const float m_old = fresh ? 0.f : m_run[qb];

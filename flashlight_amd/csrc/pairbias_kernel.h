@@ -330,6 +330,9 @@ void pairbias_kernel(const PParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) m = __builtin_fmaxf(m, s[i]);
       m = xhalf_max(m) * c2;
+      // (a block whose every key carries a finite mask value such as -1e9 must not become the reference: subtracted
+      // from itself it leaves the rounding of its own magnitude in the exponent; against this floor its weights are 0)
+      m = (m == -INFINITY) ? m : __builtin_fmaxf(m, -32768.0f);
       const float ref_new = (m == -INFINITY) ? ref : __builtin_fmaxf(ref, m);
       // (when nothing has been accumulated yet the old reference carries no weight: take the block's own maximum.  The
       // two lanes of a query hold different keys and so different partial sums; the decision takes their total, so

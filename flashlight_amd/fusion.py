@@ -11,7 +11,8 @@ What a region may contain, from the first matmul to the second:
   q @ k.transpose(-2, -1)  [* scale | / scale]  [cap * tanh(x / cap)]  {+ bias | masked_fill / where(mask, fill, x)}*
   -> softmax(dim=-1) [-> type_as / to] -> @ v
 with q/k/v of any rank >= 3 (leading axes are batch; `query.view(N, Hkv, G, L, E)` with `key.unsqueeze(2)` is
-grouped-query attention) and masks/biases broadcastable to the scores.
+grouped-query attention, and so is a key / value whose heads were repeated to match the query's: `repeat_kv`,
+`repeat_interleave`) and masks/biases broadcastable to the scores.
 
 Masks and biases are recognised by what they compute, not by how they were written:
   * a mask that depends on no graph input is evaluated once at compile time and compared with the closed forms of the
@@ -600,6 +601,49 @@ def _shapes(r: _Region):
     return gqa, L, S, Hq
 
 
+def _unrepeated_kv(n: Any) -> Optional[Tuple[fx.Node, int]]:
+    """(x, g) when n is x [N, Hkv, S, E] with every head repeated g times along the head axis, consecutively:
+    `x[:, :, None].expand(N, Hkv, g, S, E).reshape(N, Hkv * g, S, E)` (the `repeat_kv` of model code), the same with
+    `unsqueeze(2)`, or `x.repeat_interleave(g, dim=1)`.  The kernel groups query heads over key / value heads by itself
+    (query head h reads head h // g), so the repeated copy need not be made."""
+    if not isinstance(n, fx.Node):
+        return None
+    nm = _name(n)
+    if nm == "repeat_interleave":
+        x, g = n.args[0], _arg(n, 1, "repeats")
+        dim = _arg(n, 2, "dim")
+        if isinstance(x, fx.Node) and isinstance(g, int) and g >= 1 and _val(x).dim() == 4 and dim in (1, -3):
+            return x, g
+        return None
+    if nm not in ("reshape", "view") or not isinstance(n.args[0], fx.Node):
+        return None
+    ex, out = n.args[0], _val(n)
+    if _name(ex) != "expand" or out.dim() != 4 or not isinstance(ex.args[0], fx.Node):
+        return None
+    un, e5 = ex.args[0], _val(ex)
+    if e5.dim() != 5 or _val(un).dim() != 5 or _val(un).size(2) != 1:
+        return None
+    if _name(un) == "unsqueeze":
+        if _arg(un, 1, "dim") not in (2, -3):
+            return None
+        x = un.args[0]
+    elif un.op == "call_function" and un.target is operator.getitem:
+        x, idx = un.args
+        full = slice(None, None, None)
+        if not isinstance(idx, tuple) or [i for i in idx if i is not Ellipsis][:3] != [full, full, None] or \
+                any(i is not None and i != full for i in idx):
+            return None
+    else:
+        return None
+    if not isinstance(x, fx.Node):
+        return None
+    xs, g = _val(x), e5.size(2)
+    if xs.dim() != 4 or tuple(e5.shape) != (xs.size(0), xs.size(1), g, xs.size(2), xs.size(3)) or \
+            tuple(out.shape) != (xs.size(0), xs.size(1) * g, xs.size(2), xs.size(3)):
+        return None
+    return x, g
+
+
 def _head_half(n: Any) -> Optional[Tuple[fx.Node, int]]:
     """(x, 0) when n is the first half of x's heads (axis 1), (x, 1) for the second half: x[:, :h], x[:, h:] or
     torch.chunk(x, 2, dim=1)[i]."""
@@ -671,6 +715,12 @@ def fuse_attention(gm: fx.GraphModule) -> int:
         try:
             r = _match(sm)
             gqa, L, S, Hq = _shapes(r)
+            if not gqa and _val(r.q).dim() == 4:
+                # key / value heads that were repeated to match the query heads: hand the kernel the originals
+                uk, uv = _unrepeated_kv(r.k), _unrepeated_kv(r.v)
+                if uk is not None and uv is not None and uk[1] == uv[1] and _val(uk[0]).size(1) == _val(uv[0]).size(1) \
+                        and _val(uk[0]).size(1) * uk[1] == Hq:
+                    r.k, r.v = uk[0], uv[0]
             kwargs: Dict[str, Any] = dict(scale=float(r.scale), mask_kind=_ffi.MASK_NONE, window=0, prefix=0,
                                           alibi_heads=0, softcap=float(r.softcap), gqa=gqa)
             # (a score function other than the soft-cap goes with positional masks and dense operands only: document

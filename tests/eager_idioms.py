@@ -184,3 +184,40 @@ def documents_with_dropout(query, key, value, document_id, p=0.1):
     same = document_id.unsqueeze(2) == document_id.unsqueeze(1)
     w = (query @ key.transpose(-2, -1) / math.sqrt(query.size(-1))).masked_fill(~same.unsqueeze(1), -1e10)
     return torch.dropout(torch.softmax(w, dim=-1), p, True) @ value
+
+
+def _repeat_kv(hidden_states, n_rep):
+    """Key / value heads repeated to match the query heads, as model code does before an eager attention."""
+    batch, num_key_value_heads, slen, head_dim = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    hidden_states = hidden_states[:, :, None, :, :].expand(batch, num_key_value_heads, n_rep, slen, head_dim)
+    return hidden_states.reshape(batch, num_key_value_heads * n_rep, slen, head_dim)
+
+
+def decoder_layer_attention(query, key, value, attention_mask, dropout=0.0, training=False):
+    """The eager attention of a decoder layer as transformer libraries write it: repeated key / value heads, an additive
+    mask [B, 1, L, S] holding the dtype's most negative number, softmax in fp32 cast back, dropout, and the result
+    transposed to [B, L, H, E]."""
+    n_rep = query.size(1) // key.size(1)
+    key_states, value_states = _repeat_kv(key, n_rep), _repeat_kv(value, n_rep)
+    attn_weights = torch.matmul(query, key_states.transpose(2, 3)) * query.size(-1) ** -0.5
+    causal_mask = attention_mask[:, :, :, : key_states.shape[-2]]
+    attn_weights = attn_weights + causal_mask
+    attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query.dtype)
+    attn_weights = F.dropout(attn_weights, p=dropout, training=training)
+    attn_output = torch.matmul(attn_weights, value_states)
+    return attn_output.transpose(1, 2).contiguous()
+
+
+def decoder_layer_attention_softcapped(query, key, value, attention_mask, softcap=50.0):
+    """The same with the logit soft-cap written as three statements and the heads repeated with repeat_interleave."""
+    n_rep = query.size(1) // key.size(1)
+    key, value = key.repeat_interleave(n_rep, dim=1), torch.repeat_interleave(value, n_rep, dim=1)
+    attn_weights = torch.matmul(query, key.transpose(2, 3)) * query.size(-1) ** -0.5
+    attn_weights = attn_weights / softcap
+    attn_weights = torch.tanh(attn_weights)
+    attn_weights = attn_weights * softcap
+    attn_weights = attn_weights + attention_mask
+    attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query.dtype)
+    return torch.matmul(attn_weights, value)

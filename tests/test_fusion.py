@@ -226,6 +226,34 @@ def test_rewrite_maps_training_mode_dropout_to_the_kernel():
     assert calls == []
 
 
+def _decoder_mask(B, L, dtype, dev="cpu", pad=(5, 0)):
+    """[B, 1, L, L]: causal, and the first pad[b] keys of batch entry b padded (left padding), as the dtype's minimum."""
+    m = torch.zeros(B, 1, L, L, dtype=dtype, device=dev)
+    m.masked_fill_(torch.ones(L, L, dtype=torch.bool, device=dev).triu(1), torch.finfo(dtype).min)
+    for b, n in enumerate(pad[:B]):
+        m[b, :, :, :n] = torch.finfo(dtype).min
+    return m
+
+
+def test_rewrite_recognises_decoder_layer_attention_with_repeated_heads():
+    q, k, v = _qkv(Hq=8, Hkv=2, E=64)
+    mask = _decoder_mask(2, 48, BF)
+    for fn in (E.decoder_layer_attention, E.decoder_layer_attention_softcapped):
+        gm, calls = _rewrite(fn, q, k, v, mask)
+        names = {fusion._name(n) for n in gm.graph.nodes}
+        assert len(calls) == 1 and not _leftover(gm) and not names & {"expand", "reshape", "repeat_interleave"}, names
+        # key and value reach the kernel with their own two heads
+        assert fusion._val(calls[0].args[1]).size(1) == 2 and fusion._val(calls[0].args[2]).size(1) == 2
+        assert len(calls[0].args[4]) == 1  # the additive mask, as a run-time bias operand
+    assert calls[0].kwargs["softcap"] == 50.0
+    # heads repeated in another order (the whole block of heads tiled) are not grouped-query attention: kept as they are
+    def tiled(q, k, v):
+        kk, vv = k.repeat(1, 4, 1, 1), v.repeat(1, 4, 1, 1)
+        return torch.softmax(q @ kk.transpose(-2, -1) * 0.125, dim=-1) @ vv
+    gm, calls = _rewrite(tiled, q, k, v)
+    assert len(calls) == 1 and fusion._val(calls[0].args[1]).size(1) == 8
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)
@@ -364,6 +392,36 @@ def test_rewritten_dropout_regions_on_gpu():
     torch.manual_seed(4)
     y = ops.dispatch(q, k, v, scale=0.125, biases=[(bias.unsqueeze(0), 1)], dropout_p=0.2)
     assert torch.equal(x, y)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rewritten_decoder_layer_attention_on_gpu(dtype):
+    g = torch.Generator().manual_seed(77)
+    B, Hq, Hkv, L, D = 2, 8, 2, 230, 64
+    q, k, v = (torch.randn(B, h, L, D, generator=g).to(dtype).to("cuda") for h in (Hq, Hkv, Hkv))
+    mask = _decoder_mask(B, L, dtype, "cuda", pad=(37, 0))
+    for fn in (E.decoder_layer_attention, E.decoder_layer_attention_softcapped):
+        torch._dynamo.reset()
+        got = torch.compile(fn, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, mask)
+        want = fn(q.float(), k.float(), v.float(), mask.float())
+        assert got.shape == want.shape and got.dtype == dtype and torch.isfinite(got).all()
+        # the first 37 query positions of batch entry 0 are padding themselves: every key they may see is padded, eager
+        # averages over all keys there (the fills are equal) and the kernels return zeros; such rows are not compared
+        rows = slice(37, None)
+        a, b = (x if x.size(1) == L else x.transpose(1, 2) for x in (got, want))  # [B, L, H, E] either way
+        assert_parity(a[0, rows], b[0, rows], fn.__name__ + ", padded entry")
+        assert_parity(a[1], b[1], fn.__name__ + ", full entry")
+    # training mode: the kernel's dropout, reproducible from torch's seed
+    import functools
+    torch._dynamo.reset()
+    tr = torch.compile(functools.partial(E.decoder_layer_attention, dropout=0.1, training=True), backend=fusion.backend,
+                       dynamic=False, fullgraph=True)
+    torch.manual_seed(3)
+    a = tr(q, k, v, mask)
+    torch.manual_seed(3)
+    b = tr(q, k, v, mask)
+    assert torch.equal(a, b) and torch.isfinite(a).all() and not torch.equal(a, got)
 
 
 @pytest.mark.gpu

@@ -7,7 +7,9 @@ keep their own eager functions: `torch.compile(fn, backend=flashlight_amd.fusion
 function with Dynamo, finds every region of that shape in the FX graph and replaces it by a call into the hand-written
 kernel (`flashlight_amd::attn_fwd`); whatever else the function does keeps running as ordinary eager PyTorch.
 
-What a region may contain, from the first matmul to the second:
+A call of `torch.nn.functional.scaled_dot_product_attention` in the captured function is a region by itself (mask,
+dropout_p, is_causal, scale, enable_gqa as PyTorch defines them).  What a written-out region may contain, from the first
+matmul to the second:
   q @ k.transpose(-2, -1)  [* scale | / scale]  [cap * tanh(x / cap)]  {+ bias | masked_fill / where(mask, fill, x)}*
   -> softmax(dim=-1) [-> type_as / to] -> @ v
 with q/k/v of any rank >= 3 (leading axes are batch; `query.view(N, Hkv, G, L, E)` with `key.unsqueeze(2)` is
@@ -335,6 +337,7 @@ class _Region:
         self.biases: List[fx.Node] = []
         self.masks: List[Tuple[fx.Node, bool]] = []   # (mask node, invert)
         self.out: Optional[fx.Node] = None
+        self.causal = False                  # scaled_dot_product_attention(is_causal=True)
 
 
 _PASS_OPS = ("to", "type_as", "float", "contiguous", "clone")
@@ -588,6 +591,35 @@ def _match(softmax: fx.Node) -> _Region:
     return r
 
 
+def _match_sdpa(n: fx.Node) -> _Region:
+    """torch.nn.functional.scaled_dot_product_attention(query, key, value, attn_mask=None, dropout_p=0.0,
+    is_causal=False, scale=None, enable_gqa=False) as a region of its own: a boolean attn_mask is True where a key
+    takes part, any other is added to the scaled scores; dropout_p applies whenever it is not 0."""
+    q, k, v = (_arg(n, i, name) for i, name in enumerate(("query", "key", "value")))
+    mask, p, causal = _arg(n, 3, "attn_mask"), _arg(n, 4, "dropout_p", 0.0), _arg(n, 5, "is_causal", False)
+    scale, gqa = _arg(n, 6, "scale"), _arg(n, 7, "enable_gqa", False)
+    if not all(isinstance(x, fx.Node) for x in (q, k, v)) or not isinstance(causal, bool) or not isinstance(gqa, bool):
+        raise _NoMatch("scaled_dot_product_attention with operands or flags that are not constants of the graph")
+    if not (_is_number(p) and 0.0 <= float(p) < 1.0) or not (scale is None or (_is_number(scale) and scale > 0)):
+        raise _NoMatch("scaled_dot_product_attention with a dropout rate or scale that is not a constant")
+    qs, ks, vs = _val(q), _val(k), _val(v)
+    if qs.dim() != 4 or ks.dim() != 4 or vs.dim() != 4 or qs.size(1) % ks.size(1) or ks.size(1) != vs.size(1) or \
+            (qs.size(1) != ks.size(1) and not gqa):
+        raise _NoMatch("scaled_dot_product_attention operands are not [N, H, L, E] with grouped heads")
+    r = _Region()
+    r.q, r.k, r.v, r.out, r.nodes = q, k, v, n, [n]
+    r.scale = float(scale) if scale is not None else 1.0 / math.sqrt(qs.size(-1))
+    r.dropout_p, r.causal = float(p), causal
+    if mask is not None:
+        if not isinstance(mask, fx.Node) or (causal and mask is not None):
+            raise _NoMatch("scaled_dot_product_attention with both a mask and is_causal")
+        if _val(mask).dtype == torch.bool:
+            r.masks.append((mask, True))
+        else:
+            r.biases.append(mask)
+    return r
+
+
 def _shapes(r: _Region):
     q, k, v = _val(r.q), _val(r.k), _val(r.v)
     if q.dim() < 3 or k.dim() < 3 or v.dim() < 3:
@@ -597,6 +629,8 @@ def _shapes(r: _Region):
     L, S = q.size(-2), k.size(-2)
     if v.size(-2) != S or q.size(-1) != k.size(-1):
         raise _NoMatch("inconsistent operand shapes")
+    if q.size(-1) > 512:
+        raise _NoMatch("head dims above 512 have no kernel")
     Hq = q.size(1) * q.size(2) if gqa else (q.size(-3) if q.dim() >= 4 else 1)
     return gqa, L, S, Hq
 
@@ -711,9 +745,9 @@ def fuse_attention(gm: fx.GraphModule) -> int:
     """Rewrites every attention region of `gm` (a Dynamo-captured graph with example values on its nodes) in place.
     Returns the number of regions replaced."""
     replaced = 0
-    for sm in [n for n in gm.graph.nodes if _name(n) == "softmax"]:
+    for sm in [n for n in gm.graph.nodes if _name(n) in ("softmax", "scaled_dot_product_attention")]:
         try:
-            r = _match(sm)
+            r = _match(sm) if _name(sm) == "softmax" else _match_sdpa(sm)
             gqa, L, S, Hq = _shapes(r)
             if not gqa and _val(r.q).dim() == 4:
                 # key / value heads that were repeated to match the query heads: hand the kernel the originals
@@ -721,8 +755,8 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                 if uk is not None and uv is not None and uk[1] == uv[1] and _val(uk[0]).size(1) == _val(uv[0]).size(1) \
                         and _val(uk[0]).size(1) * uk[1] == Hq:
                     r.k, r.v = uk[0], uv[0]
-            kwargs: Dict[str, Any] = dict(scale=float(r.scale), mask_kind=_ffi.MASK_NONE, window=0, prefix=0,
-                                          alibi_heads=0, softcap=float(r.softcap), gqa=gqa)
+            kwargs: Dict[str, Any] = dict(scale=float(r.scale), mask_kind=_ffi.MASK_CAUSAL if r.causal else _ffi.MASK_NONE,
+                                          window=0, prefix=0, alibi_heads=0, softcap=float(r.softcap), gqa=gqa)
             # (a score function other than the soft-cap goes with positional masks and dense operands only: document
             # ids and the in-kernel ALiBi term stay dense then)
             plain = r.score_fn is None

@@ -254,6 +254,36 @@ def test_rewrite_recognises_decoder_layer_attention_with_repeated_heads():
     assert len(calls) == 1 and fusion._val(calls[0].args[1]).size(1) == 8
 
 
+def test_rewrite_maps_scaled_dot_product_attention_calls():
+    import torch.nn.functional as F
+    q, k, v = _qkv(Hq=8, Hkv=2, E=64)
+    keep, add = torch.rand(2, 1, 48, 48) > 0.2, torch.randn(2, 8, 48, 48)
+    gm, calls = _rewrite(lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True), q, k, v)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL and calls[0].kwargs["scale"] == 0.125
+    assert "scaled_dot_product_attention" not in {fusion._name(n) for n in gm.graph.nodes}
+    # a boolean mask is True where a key takes part; heads repeated by the caller are grouped again
+    gm, calls = _rewrite(lambda q, k, v, m: F.scaled_dot_product_attention(q, k.repeat_interleave(4, 1), v.repeat_interleave(4, 1),
+                                                                        attn_mask=m), q, k, v, keep)
+    assert len(calls) == 1 and calls[0].kwargs["mask_invert"] == (True,) and fusion._val(calls[0].args[1]).size(1) == 2
+    # a float mask is a bias; dropout_p and scale carry over
+    gm, calls = _rewrite(lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m, dropout_p=0.1, scale=0.2,
+                                                                        enable_gqa=True), q, k, v, add)
+    assert len(calls) == 1 and len(calls[0].args[4]) == 1 and calls[0].kwargs["dropout_p"] == 0.1 and calls[0].kwargs["scale"] == 0.2
+    # a constant lower-triangular mask is the causal mask
+    gm, calls = _rewrite(lambda q, k, v: F.scaled_dot_product_attention(q, k, v, enable_gqa=True,
+                                                                     attn_mask=torch.ones(48, 48, dtype=torch.bool).tril()), q, k, v)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL and not calls[0].args[4] and not calls[0].args[5]
+    # left alone: head dims without a kernel, dropout beyond head dim 128
+    big = torch.randn(1, 2, 16, 640, dtype=BF)
+    gm, calls = _rewrite(lambda q: F.scaled_dot_product_attention(q, q, q), big)
+    assert calls == []
+    wide = torch.randn(1, 2, 16, 256, dtype=BF)
+    gm, calls = _rewrite(lambda q: F.scaled_dot_product_attention(q, q, q, dropout_p=0.1), wide)
+    assert calls == []
+    gm, calls = _rewrite(lambda q: F.scaled_dot_product_attention(q, q, q), wide)
+    assert len(calls) == 1
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)
@@ -422,6 +452,29 @@ def test_rewritten_decoder_layer_attention_on_gpu(dtype):
     torch.manual_seed(3)
     b = tr(q, k, v, mask)
     assert torch.equal(a, b) and torch.isfinite(a).all() and not torch.equal(a, got)
+
+
+@pytest.mark.gpu
+def test_rewritten_scaled_dot_product_attention_on_gpu():
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(91)
+    B, Hq, Hkv, L, S, D = 2, 8, 2, 200, 264, 128
+    q = torch.randn(B, Hq, L, D, generator=g).to(BF).to("cuda")
+    k, v = (torch.randn(B, Hkv, S, D, generator=g).to(BF).to("cuda") for _ in range(2))
+    keep = (torch.rand(B, 1, L, S, generator=g) > 0.3).to("cuda")
+    keep[..., 0] = True
+    add = torch.randn(1, Hq, L, S, generator=g).to("cuda")
+    cases = {
+        "plain gqa": (lambda q, k, v: F.scaled_dot_product_attention(q, k, v, enable_gqa=True), ()),
+        "causal, unequal lengths": (lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True), ()),
+        "boolean mask": (lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m, enable_gqa=True), (keep,)),
+        "float mask, scale": (lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m, scale=0.05, enable_gqa=True), (add,)),
+    }
+    for name, (fn, extra) in cases.items():
+        torch._dynamo.reset()
+        got = torch.compile(fn, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, *extra)
+        want = fn(q.float().cpu(), k.float().cpu(), v.float().cpu(), *(e.cpu() for e in extra))
+        assert_parity(got, want, name)
 
 
 @pytest.mark.gpu

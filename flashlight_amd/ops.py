@@ -284,6 +284,13 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
     their pre-pass every time.  `score_fn` = (kind, four constants), see `_ffi.attn_fwd`: forward only."""
     dropout_p = float(dropout_p)
     _ffi.dropout_threshold(dropout_p)  # range check
+    if q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and q.is_cuda and (q.numel() == 0 or k.size(2) == 0):
+        # no batch entries, heads or queries: an empty result; queries but no keys: zeros (a softmax over nothing times no
+        # values), as the eager functions give.  Nothing to launch; the zeros still hang on the operands for autograd.
+        out = _alloc_out(q, v, diff, seq_major_out).zero_()
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+            out = out + (q.sum() + k.sum() + v.sum()).to(out.dtype) * 0
+        return out
     padded = _pad_head_dims(q, k, v, gate, diff,
                             bias_only=not (alibi_heads or softcap or doc_ids is not None or gate is not None or dropout_p > 0.0
                                            or score_fn is not None),

@@ -298,6 +298,20 @@ def test_evoformer_bias_staged_and_direct_paths(D):
         assert_parity(out, ref, f"D={D} {name}")
 
 
+def test_empty_problems_return_what_eager_returns():
+    """No queries, no batch entries or no heads: an empty tensor; queries without keys: zeros.  Gradients are zeros."""
+    mk = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)  # noqa: E731
+    assert A.attention_pytorch_causal(mk(2, 4, 0, 64), mk(2, 4, 0, 64), mk(2, 4, 0, 64)).shape == (2, 4, 0, 64)
+    assert A.attention_pytorch(mk(0, 4, 16, 64), mk(0, 4, 16, 64), mk(0, 4, 16, 64)).shape == (0, 4, 16, 64)
+    q = torch.randn(2, 4, 16, 64, device=DEV).to(torch.bfloat16).requires_grad_(True)
+    k = mk(2, 4, 0, 64).requires_grad_(True)
+    out = A.attention_pytorch(q, k, mk(2, 4, 0, 128))
+    ref = torch.softmax(q.float() @ k.float().transpose(-1, -2), -1) @ torch.zeros(2, 4, 0, 128, device=DEV)
+    assert out.shape == ref.shape == (2, 4, 16, 128) and torch.equal(out.float(), ref)
+    out.sum().backward()
+    assert q.grad is not None and not q.grad.any() and k.grad.shape == (2, 4, 0, 64)
+
+
 def test_front_end_errors_on_gpu_tensors():
     q, k, v = qkv(1, 4, 2, 64, 64)
     with pytest.raises(ValueError, match="enable_gqa"):

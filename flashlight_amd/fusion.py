@@ -292,8 +292,10 @@ def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: 
         q4 = q.reshape(q.size(0), -1, L, q.size(-1))
         k4, v4 = k.squeeze(2), v.squeeze(2)
     else:
-        if q.dim() == 3:
+        if q.dim() == 3:  # [N, L, E]: one head; operands with a batch axis of their own get the head axis too
             q = q.unsqueeze(1)
+            biases = [b.unsqueeze(-3) if b.dim() == 3 else b for b in biases]
+            masks = [m.unsqueeze(-3) if m.dim() == 3 else m for m in masks]
         lead, heads = tuple(q.shape[:-3]), (q.size(-3),)
 
         def like_q(t):  # key/value with missing or size-1 leading axes broadcast like matmul operands do
@@ -322,6 +324,54 @@ def fused_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, doc_ids: 
     out = ops.dispatch(q4, k4, v4, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                        alibi_heads=alibi_heads, softcap=softcap, biases=kb, diff=True, lambda_full=float(diff_lambda))
     return out.reshape(*result_shape[:-3], result_shape[-3] // 2, *result_shape[-2:])
+
+
+def fused_multi_head_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, *, num_heads: int,
+                               in_proj_weight, in_proj_bias, q_proj_weight, k_proj_weight, v_proj_weight,
+                               out_proj_weight, out_proj_bias, dropout_p: float, key_padding_mask, attn_mask,
+                               is_causal: bool):
+    """Target of the node that replaces a call of torch.nn.functional.multi_head_attention_forward (what
+    torch.nn.MultiheadAttention and the Transformer layers built on it call; Dynamo keeps it as one node, so its
+    scaled_dot_product_attention is not visible to the rewrite).  query [L, N, E], key / value [S, N, *] (or without
+    the batch axis); the three input projections and the output projection run as torch linears, the attention
+    between them on the fused kernel with the heads read in place.  Masks follow that function's conventions: a
+    boolean `attn_mask` ([L, S] or [N * H, L, S]) or `key_padding_mask` ([N, S]) is True where a key is NOT attended,
+    any other dtype is added to the scores; `is_causal` says that `attn_mask` is the causal mask, and is taken at
+    its word only when there is no padding mask, as that function does.  Returns (result [L, N, E], None)."""
+    import torch.nn.functional as F
+    batched = query.dim() == 3
+    if not batched:
+        query, key, value = query.unsqueeze(1), key.unsqueeze(1), value.unsqueeze(1)
+        if key_padding_mask is not None:
+            key_padding_mask = key_padding_mask.unsqueeze(0)
+    (L, N, E), S, H = query.shape, key.size(0), num_heads
+    if is_causal and attn_mask is None:
+        raise RuntimeError("is_causal needs the causal attn_mask it speaks of")
+    if q_proj_weight is None:
+        wq, wk, wv = in_proj_weight.chunk(3)
+    else:
+        wq, wk, wv = q_proj_weight, k_proj_weight, v_proj_weight
+    bq, bk, bv = in_proj_bias.chunk(3) if in_proj_bias is not None else (None, None, None)
+    if q_proj_weight is None and key is query and value is query:
+        q, k, v = F.linear(query, in_proj_weight, in_proj_bias).chunk(3, dim=-1)   # self-attention: one product
+    else:
+        q, k, v = F.linear(query, wq, bq), F.linear(key, wk, bk), F.linear(value, wv, bv)
+    hd = E // H
+    q, k, v = (t.reshape(t.size(0), N, H, hd).permute(1, 2, 0, 3) for t in (q, k, v))   # [N, H, L | S, hd], in place
+    biases, masks = [], []
+    kind = _ffi.MASK_NONE
+    if is_causal and key_padding_mask is None:
+        kind = _ffi.MASK_CAUSAL
+    elif attn_mask is not None:
+        am = attn_mask if attn_mask.dim() == 2 else attn_mask.reshape(N, H, L, S)
+        (masks if am.dtype == torch.bool else biases).append(am)
+    if key_padding_mask is not None:
+        kp = key_padding_mask.reshape(N, 1, 1, S)
+        (masks if kp.dtype == torch.bool else biases).append(kp)
+    out = fused_attention(q, k, v, None, biases, masks, scale=1.0 / math.sqrt(hd), mask_kind=kind, window=0, prefix=0,
+                          alibi_heads=0, softcap=0.0, gqa=False, dropout_p=dropout_p)
+    out = F.linear(out.permute(2, 0, 1, 3).reshape(L * N, E), out_proj_weight, out_proj_bias).reshape(L, N, E)
+    return (out if batched else out.squeeze(1)), None
 
 
 # ---- matching ----------------------------------------------------------------------------------------------------------------
@@ -603,9 +653,12 @@ def _match_sdpa(n: fx.Node) -> _Region:
     if not (_is_number(p) and 0.0 <= float(p) < 1.0) or not (scale is None or (_is_number(scale) and scale > 0)):
         raise _NoMatch("scaled_dot_product_attention with a dropout rate or scale that is not a constant")
     qs, ks, vs = _val(q), _val(k), _val(v)
-    if qs.dim() != 4 or ks.dim() != 4 or vs.dim() != 4 or qs.size(1) % ks.size(1) or ks.size(1) != vs.size(1) or \
+    if qs.dim() == 3 and ks.dim() == 3 and vs.dim() == 3:
+        if not qs.size(0) == ks.size(0) == vs.size(0):
+            raise _NoMatch("scaled_dot_product_attention operands [N, L, E] with different batch sizes")
+    elif qs.dim() != 4 or ks.dim() != 4 or vs.dim() != 4 or qs.size(1) % ks.size(1) or ks.size(1) != vs.size(1) or \
             (qs.size(1) != ks.size(1) and not gqa):
-        raise _NoMatch("scaled_dot_product_attention operands are not [N, H, L, E] with grouped heads")
+        raise _NoMatch("scaled_dot_product_attention operands are not [N, H, L, E] with grouped heads (or [N, L, E])")
     r = _Region()
     r.q, r.k, r.v, r.out, r.nodes = q, k, v, n, [n]
     r.scale = float(scale) if scale is not None else 1.0 / math.sqrt(qs.size(-1))
@@ -741,10 +794,64 @@ def _merge_differential(gm: fx.GraphModule) -> int:
     return merged
 
 
+_MHA_PARAMS = ("query", "key", "value", "embed_dim_to_check", "num_heads", "in_proj_weight", "in_proj_bias", "bias_k",
+               "bias_v", "add_zero_attn", "dropout_p", "out_proj_weight", "out_proj_bias", "training", "key_padding_mask",
+               "need_weights", "attn_mask", "use_separate_proj_weight", "q_proj_weight", "k_proj_weight", "v_proj_weight",
+               "static_k", "static_v", "average_attn_weights", "is_causal")
+_MHA_DEFAULTS = dict(training=True, key_padding_mask=None, need_weights=True, attn_mask=None, use_separate_proj_weight=False,
+                     q_proj_weight=None, k_proj_weight=None, v_proj_weight=None, static_k=None, static_v=None,
+                     average_attn_weights=True, is_causal=False)
+
+
+def _rewrite_multi_head_attention(gm: fx.GraphModule) -> int:
+    """Calls of torch.nn.functional.multi_head_attention_forward that return no weights and use neither bias_k / bias_v,
+    add_zero_attn nor static keys become `fused_multi_head_attention`; others are left as they are.  Head dims above
+    128 are left alone in training mode (no backward kernel there) and with dropout."""
+    import torch.nn.functional as F
+    replaced = 0
+    for n in [x for x in gm.graph.nodes if x.op == "call_function" and x.target is F.multi_head_attention_forward]:
+        a = dict(_MHA_DEFAULTS)
+        a.update(zip(_MHA_PARAMS, n.args))
+        a.update(n.kwargs)
+        if any(name not in a for name in _MHA_PARAMS[:13]):
+            continue
+        if a["need_weights"] is not False or a["bias_k"] is not None or a["bias_v"] is not None or a["add_zero_attn"] is not False \
+                or a["static_k"] is not None or a["static_v"] is not None:
+            continue
+        if not isinstance(a["num_heads"], int) or not _is_number(a["dropout_p"]) or not isinstance(a["training"], bool) \
+                or not isinstance(a["is_causal"], bool) or not isinstance(a["use_separate_proj_weight"], bool):
+            continue
+        if not all(isinstance(a[x], fx.Node) for x in ("query", "key", "value", "out_proj_weight")):
+            continue
+        qv = _val(a["query"])
+        if qv.dim() not in (2, 3) or qv.size(-1) % a["num_heads"] or qv.dtype not in (torch.bfloat16, torch.float16):
+            continue
+        hd = qv.size(-1) // a["num_heads"]
+        p = float(a["dropout_p"]) if a["training"] else 0.0
+        if hd > 512 or (hd > 128 and (a["training"] or p > 0.0)) or not 0.0 <= p < 1.0:
+            continue
+        sep = a["use_separate_proj_weight"]
+        if (sep and any(a[x] is None for x in ("q_proj_weight", "k_proj_weight", "v_proj_weight"))) or \
+                (not sep and a["in_proj_weight"] is None):
+            continue
+        kwargs = dict(num_heads=a["num_heads"], in_proj_weight=None if sep else a["in_proj_weight"],
+                      in_proj_bias=a["in_proj_bias"], q_proj_weight=a["q_proj_weight"] if sep else None,
+                      k_proj_weight=a["k_proj_weight"] if sep else None, v_proj_weight=a["v_proj_weight"] if sep else None,
+                      out_proj_weight=a["out_proj_weight"], out_proj_bias=a["out_proj_bias"], dropout_p=p,
+                      key_padding_mask=a["key_padding_mask"], attn_mask=a["attn_mask"], is_causal=a["is_causal"])
+        with gm.graph.inserting_before(n):
+            new = gm.graph.call_function(fused_multi_head_attention, (a["query"], a["key"], a["value"]), kwargs)
+        new.meta.update(n.meta)
+        n.replace_all_uses_with(new)
+        gm.graph.erase_node(n)
+        replaced += 1
+    return replaced
+
+
 def fuse_attention(gm: fx.GraphModule) -> int:
     """Rewrites every attention region of `gm` (a Dynamo-captured graph with example values on its nodes) in place.
     Returns the number of regions replaced."""
-    replaced = 0
+    replaced = _rewrite_multi_head_attention(gm)
     for sm in [n for n in gm.graph.nodes if _name(n) in ("softmax", "scaled_dot_product_attention")]:
         try:
             r = _match(sm) if _name(sm) == "softmax" else _match_sdpa(sm)

@@ -273,6 +273,10 @@ def test_rewrite_maps_scaled_dot_product_attention_calls():
     gm, calls = _rewrite(lambda q, k, v: F.scaled_dot_product_attention(q, k, v, enable_gqa=True,
                                                                      attn_mask=torch.ones(48, 48, dtype=torch.bool).tril()), q, k, v)
     assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL and not calls[0].args[4] and not calls[0].args[5]
+    # operands without a head axis, [N, L, E], are one head
+    q3 = torch.randn(3, 48, 64, dtype=BF)
+    gm, calls = _rewrite(lambda q, m: F.scaled_dot_product_attention(q, q, q, attn_mask=m), q3, torch.randn(3, 48, 48))
+    assert len(calls) == 1 and len(calls[0].args[4]) == 1
     # left alone: head dims without a kernel, dropout beyond head dim 128
     big = torch.randn(1, 2, 16, 640, dtype=BF)
     gm, calls = _rewrite(lambda q: F.scaled_dot_product_attention(q, q, q), big)
@@ -475,6 +479,19 @@ def test_rewritten_scaled_dot_product_attention_on_gpu():
         got = torch.compile(fn, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, *extra)
         want = fn(q.float().cpu(), k.float().cpu(), v.float().cpu(), *(e.cpu() for e in extra))
         assert_parity(got, want, name)
+    # [N, L, E] operands (no head axis) with a mask / bias that has a batch axis of its own, as a call and spelled out
+    q3, k3, v3 = q[:, 0], k[:, 0], v[:, 0]
+    keep3, add3 = keep[:, 0], torch.randn(B, L, S, generator=g).to("cuda")
+    cases3 = {
+        "3-D, boolean mask": (lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m), keep3),
+        "3-D, float mask": (lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m), add3),
+        "3-D, spelled out": (lambda q, k, v, m: torch.softmax(q @ k.transpose(-2, -1) * 0.08 + m, dim=-1) @ v, add3),
+    }
+    for name, (fn, m) in cases3.items():
+        torch._dynamo.reset()
+        got = torch.compile(fn, backend=fusion.backend, dynamic=False, fullgraph=True)(q3, k3, v3, m)
+        assert got.shape == (B, L, D)
+        assert_parity(got, fn(q3.float().cpu(), k3.float().cpu(), v3.float().cpu(), m.cpu()), name)
 
 
 @pytest.mark.gpu
@@ -493,3 +510,118 @@ def test_a_fully_masked_row_comes_out_as_zeros():
     torch._dynamo.reset()
     got = torch.compile(E.learned_bias, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, bias, pad)
     assert_parity(got, E.learned_bias(q.float(), k.float(), v.float(), bias, pad), "five keys left")
+
+
+def test_rewrite_takes_multi_head_attention_modules():
+    """torch.nn.MultiheadAttention calls torch.nn.functional.multi_head_attention_forward, which Dynamo keeps as one
+    node: the rewrite replaces that node when no weights are returned, and leaves it alone otherwise."""
+    import torch.nn as nn
+    x = torch.randn(2, 40, 128, dtype=BF)
+    pad = torch.zeros(2, 40, dtype=torch.bool)
+
+    def targets(mod, *args, **kwargs):
+        got = []
+
+        def be(gm, example_inputs):
+            fusion.fuse_attention(gm)
+            got.extend(n.target for n in gm.graph.nodes if n.op == "call_function")
+
+            def run(*a):
+                raise _Done
+            return run
+
+        class _Done(Exception):
+            pass
+
+        torch._dynamo.reset()
+        with pytest.raises(_Done):
+            torch.compile(mod, backend=be, dynamic=False)(*args, **kwargs)
+        return got
+
+    mha = nn.MultiheadAttention(128, 4, batch_first=True).to(BF).train()
+    got = targets(mha, x, x, x, need_weights=False, key_padding_mask=pad)
+    assert fusion.fused_multi_head_attention in got and torch.nn.functional.multi_head_attention_forward not in got
+    got = targets(mha, x, x, x, need_weights=True)
+    assert fusion.fused_multi_head_attention not in got and torch.nn.functional.multi_head_attention_forward in got
+    layer = nn.TransformerEncoderLayer(128, 4, 256, dropout=0.1, batch_first=True).to(BF).train()
+    got = targets(layer, x, src_key_padding_mask=pad)
+    assert fusion.fused_multi_head_attention in got
+    # head dim 256 in training mode has no backward kernel: left alone; in evaluation mode it is taken
+    wide = nn.MultiheadAttention(512, 2, batch_first=True).to(BF)
+    xw = torch.randn(2, 40, 512, dtype=BF)
+    assert fusion.fused_multi_head_attention not in targets(wide.train(), xw, xw, xw, need_weights=False)
+    assert fusion.fused_multi_head_attention in targets(wide.eval(), xw, xw, xw, need_weights=False)
+    # bias_k / bias_v and add_zero_attn append keys: left alone
+    odd = nn.MultiheadAttention(128, 4, batch_first=True, add_bias_kv=True).to(BF).train()
+    assert fusion.fused_multi_head_attention not in targets(odd, x, x, x, need_weights=False)
+
+
+@pytest.mark.gpu
+def test_multi_head_attention_modules_on_gpu():
+    """torch.nn.MultiheadAttention and Transformer layers through the rewrite: the module in bf16 on the GPU against a
+    copy of it in fp32 on the CPU; results, and for the attention module the gradients of every parameter."""
+    import copy
+    import torch.nn as nn
+    from flashlight_amd import ops
+    torch.manual_seed(0)
+    B, L, E, H = 2, 200, 256, 4
+    x = torch.randn(B, L, E).to(BF)
+    pad = torch.zeros(B, L, dtype=torch.bool)
+    pad[0, 150:] = True
+    pad[1, 77:] = True
+    causal = nn.Transformer.generate_square_subsequent_mask(L)
+    launches = [0]
+    real = ops.dispatch
+
+    def counting(*a, **k):
+        launches[0] += 1
+        return real(*a, **k)
+
+    def check(name, mod, args, kwargs, n_launches, grads=True, tol=(2e-2, 2e-3)):
+        ref = copy.deepcopy(mod).float().train()
+        m = mod.to(BF).to("cuda").train()
+        dev = lambda t: t.to("cuda") if torch.is_tensor(t) else t
+        launches[0] = 0
+        torch._dynamo.reset()
+        ops.dispatch = counting
+        try:
+            got = torch.compile(m, backend=fusion.backend, dynamic=False)(*map(dev, args), **{k: dev(v) for k, v in kwargs.items()})
+        finally:
+            ops.dispatch = real
+        want = ref(*(a.float() if torch.is_tensor(a) and a.is_floating_point() else a for a in args), **kwargs)
+        got, want = (t[0] if isinstance(t, tuple) else t for t in (got, want))
+        assert launches[0] == n_launches, name
+        assert_parity(got, want, name, max_tol=tol[0] * max(1.0, want.abs().max().item()), mean_tol=tol[1] * max(1.0, want.abs().max().item()))
+        if not grads:
+            return
+        w = torch.randn(want.shape, generator=torch.Generator().manual_seed(5))
+        (want * w).sum().backward()
+        (got.float() * w.to("cuda")).sum().backward()
+        for (pn, p32), (_, p16) in zip(ref.named_parameters(), m.named_parameters()):
+            assert (p32.grad is None) == (p16.grad is None), f"{name}: {pn}"
+            if p32.grad is not None:
+                err = (p16.grad.float().cpu() - p32.grad).abs().max().item()
+                assert err <= 2e-2 * p32.grad.abs().max().item() + 1e-4, f"{name}: gradient of {pn} off by {err}"
+
+    mha = lambda **kw: nn.MultiheadAttention(E, H, **kw)
+    nw = dict(need_weights=False)
+    xt = x.transpose(0, 1)
+    check("self-attention", mha(batch_first=True), (x, x, x), nw, 1)
+    check("padding mask", mha(batch_first=True), (x, x, x), dict(nw, key_padding_mask=pad), 1)
+    check("causal mask tensor", mha(batch_first=True), (x, x, x), dict(nw, attn_mask=causal), 1)
+    check("causal hint", mha(batch_first=True), (x, x, x), dict(nw, attn_mask=causal, is_causal=True), 1)
+    check("sequence first", mha(), (xt, xt, xt), nw, 1)
+    check("unbatched", mha(), (x[0], x[0], x[0]), dict(nw, key_padding_mask=pad[0]), 1)
+    check("key / value widths of their own", mha(batch_first=True, kdim=128, vdim=64), (x, x[:, :120, :128], x[:, :120, :64]), nw, 1)
+    check("float masks", mha(batch_first=True), (x, x, x),
+          dict(nw, attn_mask=torch.randn(L, L), key_padding_mask=torch.zeros(B, L).masked_fill(pad, float("-inf"))), 1)
+    check("a mask per head", mha(batch_first=True), (x, x, x), dict(nw, attn_mask=torch.randn(B * H, L, L)), 1)
+    check("head dim 16", nn.MultiheadAttention(E, 16, batch_first=True), (x, x, x), dict(nw, key_padding_mask=pad), 2)  # padded: 2 calls
+    check("returns weights: left alone", mha(batch_first=True), (x, x, x), dict(need_weights=True), 0)
+    # whole layers: bf16 rounding of the feed-forward part dominates, so results only
+    check("encoder layer", nn.TransformerEncoderLayer(E, H, 512, dropout=0.0, batch_first=True), (x,),
+          dict(src_key_padding_mask=pad), 1, grads=False)
+    check("decoder layer", nn.TransformerDecoderLayer(E, H, 512, dropout=0.0, batch_first=True), (x, x[:, :120]),
+          dict(tgt_mask=causal, tgt_is_causal=True, memory_key_padding_mask=pad[:, :120]), 2, grads=False)
+    check("three encoder layers", nn.TransformerEncoder(nn.TransformerEncoderLayer(E, H, 512, dropout=0.0, batch_first=True), 3,
+                                                        enable_nested_tensor=False), (x,), dict(src_key_padding_mask=pad), 3, grads=False)

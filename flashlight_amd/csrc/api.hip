@@ -206,6 +206,62 @@ int static_scratch_ptr(void** out) {
   return 0;
 }
 
+// Guard of the static scratch: one event per device, recorded behind every eager fl_attn_bwd_static call.  A call on
+// another stream while that event has not completed would share the array with kernels still running: it is refused
+// instead.  Calls on the stream of the previous call are ordered behind it and pass; calls under stream capture are
+// neither checked nor recorded (a graph's replays are the caller's to order).
+struct ScratchGuard {
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool armed = false;
+};
+ScratchGuard g_scratch_guard[kMaxDevices];
+
+bool stream_is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st == hipStreamCaptureStatusActive;
+}
+
+// 0 when the scratch of the current device may be used by a call on `s`.
+int static_scratch_acquire(hipStream_t s, int* dev_out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(FL_ERR_UNSUPPORTED, "no current device the library tracks");
+  *dev_out = dev;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchGuard& g = g_scratch_guard[dev];
+  if (!g.done) {
+    e = hipEventCreateWithFlags(&g.done, hipEventDisableTiming);
+    if (e != hipSuccess) return fail((int)e, "hipEventCreateWithFlags failed: %s", hipGetErrorString(e));
+  }
+  if (g.armed && g.last != s) {
+    e = hipEventQuery(g.done);
+    if (e == hipErrorNotReady) {
+      (void)hipGetLastError();
+      return fail(FL_ERR_WORKSPACE,
+                  "fl_attn_bwd_static: the static scratch of this GPU is still in use by a call on another stream; queue "
+                  "such calls on one stream, wait for the earlier one, or use fl_attn_bwd with buffers of your own");
+    }
+    if (e != hipSuccess) return fail((int)e, "hipEventQuery failed: %s", hipGetErrorString(e));
+  }
+  return 0;
+}
+
+void static_scratch_release(hipStream_t s, int dev) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchGuard& g = g_scratch_guard[dev];
+  if (g.done && hipEventRecord(g.done, s) == hipSuccess) {
+    g.last = s;
+    g.armed = true;
+  } else {
+    (void)hipGetLastError();
+  }
+}
+
 bool is_doc(int kind) { return kind == FL_MASK_DOCUMENT || kind == FL_MASK_DOCUMENT_CAUSAL; }
 
 uint32_t wanted_features(const fl_attn_params* p) {
@@ -911,7 +967,16 @@ int fl_attn_bwd_static(const fl_attn_bwd_params* b, void* stream) {
   c.delta = static_cast<float*>(ptr);
   c.fwd.workspace = table_bytes ? static_cast<unsigned char*>(ptr) + delta_bytes : nullptr;
   c.fwd.workspace_bytes = table_bytes;
-  return fl_attn_bwd(&c, stream);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool capturing = stream_is_capturing(s);
+  int dev = -1;
+  if (!capturing) {
+    rc = static_scratch_acquire(s, &dev);
+    if (rc) return rc;
+  }
+  rc = fl_attn_bwd(&c, stream);
+  if (!capturing && dev >= 0) static_scratch_release(s, dev);
+  return rc;
 }
 
 }  // extern "C"

@@ -233,10 +233,13 @@ int fl_attn_bwd(const fl_attn_bwd_params* p, void* stream);
  * a static device array inside the library (FL_STATIC_SCRATCH_BYTES per GPU, held until the process ends), whose
  * address is looked up once per device on the first call made with that device current.  A call that needs more
  * (4 bytes per query row of every head, rounded up to 256, plus fl_bwd_workspace_bytes()) returns FL_ERR_WORKSPACE and
- * launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine.  All calls on one GPU share the
- * array: two such calls that may overlap on that GPU (different streams, or different threads) race; calls queued on
- * one stream are ordered and safe.  Nothing in the array needs clearing between calls: each call rewrites what it
- * reads. */
+ * launches nothing.  Calls no hipMalloc / hipFree and no allocating library routine (one event per GPU is created on the
+ * first call there).  All calls on one GPU share the array, so two such calls that overlap on that GPU would race:
+ * calls queued on one stream are ordered and safe; a call on another stream while the previous call's kernels are
+ * still running returns FL_ERR_WORKSPACE and launches nothing (queue them on one stream, or wait for the first).  Calls
+ * made under stream capture are outside this check, and so are the replays of the graphs they build: ordering those
+ * against other users of the array is the caller's.  Nothing in the array needs clearing between calls: each call
+ * rewrites what it reads. */
 #define FL_STATIC_SCRATCH_BYTES (8u << 20)
 int fl_attn_bwd_static(const fl_attn_bwd_params* p, void* stream);
 /* FL_STATIC_SCRATCH_BYTES of the loaded library. */

@@ -42,6 +42,37 @@ def test_static_scratch_matches_the_allocating_entry_point_twice_in_a_row():
                 assert torch.equal(a, b), (name, B, H, S, D, kind)
 
 
+@pytest.mark.gpu
+def test_static_scratch_refuses_a_call_that_would_overlap_on_another_stream():
+    """All calls on a GPU share the static array.  A call on a second stream while the first call's kernels are still
+    running is refused (FL_ERR_WORKSPACE) instead of racing; the same stream, or the other stream once the first call
+    has finished, passes and gives the same gradients."""
+    B, H, S, D = 8, 16, 4096, 128   # a backward of a few milliseconds, 2 MiB of row sums
+    g = torch.Generator().manual_seed(3)
+    q, k, v, dout = (torch.randn(B, H, S, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=DEV)
+    out = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, lse=lse)
+    want = _ffi.attn_bwd(q, k, v, out, lse, dout, mask_kind=_ffi.MASK_CAUSAL)
+    g1, g2 = (tuple(torch.empty_like(t) for t in (q, k, v)) for _ in range(2))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    call = lambda grads: _ffi.attn_bwd(q, k, v, out, lse, dout, mask_kind=_ffi.MASK_CAUSAL, static_scratch=True, grads=grads)
+    with torch.cuda.stream(s1):
+        call(g1)
+    with torch.cuda.stream(s2):
+        with pytest.raises(_ffi.FlashlightError, match="still in use") as err:
+            call(g2)
+    assert err.value.code == -6
+    with torch.cuda.stream(s1):     # behind the first call on its own stream: ordered, accepted
+        call(g1)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s2):     # the first stream has drained
+        call(g2)
+    torch.cuda.synchronize()
+    for name, a, b, c in zip(("dq", "dk", "dv"), g1, g2, want):
+        assert torch.equal(a, c) and torch.equal(b, c), name
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     lib = _ffi.load_library()
     b = _ffi.FlAttnBwdParams()

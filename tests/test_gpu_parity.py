@@ -763,3 +763,35 @@ def test_document_mask_prepared_workspace_skips_the_prepass_and_matches():
     assert torch.equal(out, A.attention_pytorch_document_mask(q, k, v, ids, is_causal=True))
     ref = O.attention_document_mask(*f32(q, k, v), ids, is_causal=True)
     assert_parity(out, ref, "prepared workspace")
+
+
+@pytest.mark.gpu
+def test_operands_of_more_than_two_to_the_31_elements():
+    """[16, 64, 16384, 128] in bf16 is 4 GiB per operand: element offsets pass 2^31 and byte offsets 2^32.  Slices of the
+    forward's and the backward's results against runs on the slices alone, which launch the same kernels: bit-equal."""
+    from flashlight_amd import _ffi
+    B, H, L, D = 16, 64, 16384, 128
+
+    def fill(seed):
+        t = torch.empty(B, H, L, D, dtype=torch.bfloat16, device="cuda")
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        flat, step = t.view(-1), 1 << 28
+        for i in range(0, flat.numel(), step):
+            flat[i:i + step].copy_(torch.randn(step, generator=gen, device="cuda"))
+        return t
+    q, k, v, do = (fill(s) for s in (1, 2, 3, 4))
+    assert q.numel() == 1 << 31
+    lse = torch.empty(B, H, L, dtype=torch.float32, device="cuda")
+    out = _ffi.attn_fwd(q, k, v, mask_kind=_ffi.MASK_CAUSAL, lse=lse)
+    grads = _ffi.attn_bwd(q, k, v, out, lse, do, mask_kind=_ffi.MASK_CAUSAL)
+    for b, h in ((0, 0), (8, 0), (15, 63)):
+        one = lambda t: t[b:b + 1, h:h + 1].contiguous()
+        lse1 = torch.empty(1, 1, L, dtype=torch.float32, device="cuda")
+        out1 = _ffi.attn_fwd(one(q), one(k), one(v), mask_kind=_ffi.MASK_CAUSAL, lse=lse1)
+        grads1 = _ffi.attn_bwd(one(q), one(k), one(v), out1, lse1, one(do), mask_kind=_ffi.MASK_CAUSAL)
+        assert torch.equal(out[b, h], out1[0, 0]) and torch.equal(lse[b, h], lse1[0, 0]), (b, h)
+        for name, a, c in zip(("dq", "dk", "dv"), grads, grads1):
+            assert torch.equal(a[b, h], c[0, 0]), (name, b, h)
+    assert torch.isfinite(out[15, 63].float()).all() and out[15, 63].float().abs().max() > 0
+    del q, k, v, do, out, grads, lse
+    torch.cuda.empty_cache()

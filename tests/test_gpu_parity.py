@@ -795,3 +795,65 @@ def test_operands_of_more_than_two_to_the_31_elements():
     assert torch.isfinite(out[15, 63].float()).all() and out[15, 63].float().abs().max() > 0
     del q, k, v, do, out, grads, lse
     torch.cuda.empty_cache()
+
+
+@pytest.mark.gpu
+def test_calls_from_several_threads_on_streams_of_their_own():
+    """The library is re-entrant: no state is shared between calls but a thread-local error text and the lazily set kernel
+    attributes.  Eight threads, each on its own stream, run different variants (document masks with their pre-pass and
+    workspace, a staged bias, a refused call in between, whose message must be the thread's own) 20 times over; every
+    result must be bit-equal to the same call made alone."""
+    import threading
+    g = torch.Generator().manual_seed(77)
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g).to(torch.bfloat16).to("cuda")
+
+    ids = torch.sort(torch.randint(0, 5, (2, 777), generator=g), dim=1).values.to("cuda")
+    jobs = [
+        ("vanilla", lambda: _ffi.attn_fwd(*qkv128)),
+        ("causal", lambda: _ffi.attn_fwd(*qkv128, mask_kind=_ffi.MASK_CAUSAL)),
+        ("sliding", lambda: _ffi.attn_fwd(*qkv64, mask_kind=_ffi.MASK_SLIDING, window=100)),
+        ("document", lambda: _ffi.attn_fwd(*qkv64, mask_kind=_ffi.MASK_DOCUMENT_CAUSAL, doc_ids=ids)),
+        ("alibi + soft-cap", lambda: _ffi.attn_fwd(*qkv128, alibi_heads=4, softcap=20.0, mask_kind=_ffi.MASK_CAUSAL)),
+        ("bias", lambda: _ffi.attn_fwd(*qkv64, biases=[(bias, 1)])),
+        ("prefix", lambda: _ffi.attn_fwd(*qkv64, mask_kind=_ffi.MASK_PREFIX_LM, prefix=300)),
+        ("document, not causal", lambda: _ffi.attn_fwd(*qkv64, mask_kind=_ffi.MASK_DOCUMENT, doc_ids=ids)),
+    ]
+    qkv128 = (rnd(2, 4, 777, 128), rnd(2, 2, 777, 128), rnd(2, 2, 777, 128))
+    qkv64 = (rnd(2, 4, 777, 64), rnd(2, 4, 777, 64), rnd(2, 4, 777, 64))
+    bias = rnd(2, 4, 777, 784)[..., :777]
+    alone = [fn().clone() for _, fn in jobs]
+    torch.cuda.synchronize()
+    errors = []
+    start = threading.Barrier(len(jobs))
+
+    def worker(i):
+        name, fn = jobs[i]
+        try:
+            stream = torch.cuda.Stream()
+            start.wait()
+            with torch.cuda.stream(stream):
+                for it in range(20):
+                    out = fn()
+                    if it % 5 == i % 5:   # a refused call: the message is this thread's
+                        try:
+                            _ffi.attn_fwd(qkv64[0], qkv64[1], qkv64[2], mask_kind=_ffi.MASK_SLIDING, window=-(i + 1))
+                            errors.append((name, "a negative window was accepted"))
+                        except _ffi.FlashlightError as e:
+                            if "window" not in str(e):
+                                errors.append((name, f"foreign error text: {e}"))
+                    stream.synchronize()
+                    if not torch.equal(out, alone[i]):
+                        errors.append((name, f"iteration {it} differs from the call made alone"))
+                        return
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append((name, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not any(t.is_alive() for t in threads), "a worker did not finish"
+    assert errors == [], errors

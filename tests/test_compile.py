@@ -148,3 +148,57 @@ def test_compiled_gradients_with_bias_gate_and_differential_attention():
             assert (a.float() - b.float()).abs().max().item() <= 2e-2 * scale, f"{name}: output {i}"
     torch.library.opcheck(torch.ops.flashlight_amd.attn_fwd_bias_lse.default,
                           (mk(2, 2, 64, 32), mk(2, 2, 64, 32), mk(2, 2, 64, 32), -1.0, 0, 0, 0, mk(1, 2, 64, 64), 2, None, 1))
+
+
+@pytest.mark.gpu
+def test_variants_under_the_default_backend():
+    """`torch.compile(dynamic=False)(fn)` with no backend named (Inductor) is how the reference's scripts call these
+    functions (tests/test_causal.py:33, benchmarks/run_flex_variants.py:118-124): the operator goes through as an
+    external kernel, forward and backward."""
+    g = torch.Generator().manual_seed(0)
+    B, Hq, Hkv, S, D = 2, 8, 2, 300, 64
+    q, k, v = (torch.randn(B, h, S, D, generator=g).to(BF) for h in (Hq, Hkv, Hkv))
+    ids = torch.sort(torch.randint(0, 4, (B, S), generator=g), dim=1).values
+    f = lambda t: t.float()
+    dev = lambda *ts: tuple(t.to("cuda") for t in ts)
+    cases = {
+        "vanilla": (lambda q, k, v: A.attention_pytorch(q, k, v, enable_gqa=True),
+                    lambda: O.attention_vanilla(f(q), f(k), f(v), enable_gqa=True)),
+        "sliding": (lambda q, k, v: A.attention_pytorch_sliding_window(q, k, v, window_size=50, enable_gqa=True),
+                    lambda: O.attention_sliding_window(f(q), f(k), f(v), window_size=50, enable_gqa=True)),
+        "softcap": (lambda q, k, v: A.attention_softcapped(q, k, v, score_mod=A.generate_tanh_softcap(30.0), enable_gqa=True),
+                    lambda: O.attention_softcapped(f(q), f(k), f(v), score_mod=30.0, enable_gqa=True)),
+        "document": (lambda q, k, v: A.attention_pytorch_document_mask(q, k, v, ids.to("cuda"), enable_gqa=True),
+                     lambda: O.attention_document_mask(f(q), f(k), f(v), ids, enable_gqa=True)),
+    }
+    for name, (fn, ref) in cases.items():
+        torch._dynamo.reset()
+        got = torch.compile(fn, dynamic=False, fullgraph=True)(*dev(q, k, v))
+        want = ref()
+        assert_parity(got.reshape(want.shape), want, name)
+    # a training step: causal, gradients against autograd through the oracle
+    torch._dynamo.reset()
+    leaves = [t.requires_grad_(True) for t in dev(q, k, v)]
+    out = torch.compile(lambda q, k, v: A.attention_pytorch_causal(q, k, v, enable_gqa=True), dynamic=False, fullgraph=True)(*leaves)
+    w = torch.randn(out.shape, generator=g)
+    (out.float() * w.to("cuda")).sum().backward()
+    refs = [f(t).requires_grad_(True) for t in (q, k, v)]
+    want = O.attention_causal(*refs, enable_gqa=True)
+    (want * w.reshape(want.shape)).sum().backward()
+    assert_parity(out.reshape(want.shape), want, "causal")
+    for name, a, b in zip(("dq", "dk", "dv"), leaves, refs):
+        scale = max(1.0, b.grad.abs().max().item())
+        assert_parity(a.grad / scale, b.grad / scale, name)
+    # the two variants with layouts of their own
+    torch._dynamo.reset()
+    qd, kd = (torch.randn(2, 8, 200, 64, generator=g).to(BF) for _ in range(2))
+    vd = torch.randn(2, 4, 200, 128, generator=g).to(BF)
+    got = torch.compile(lambda q, k, v: A.diffattn(q, k, v, lambda_full=0.8), dynamic=False, fullgraph=True)(*dev(qd, kd, vd))
+    want = O.diff_attention(f(qd), f(kd), f(vd), lambda_full=0.8)
+    assert_parity(got.reshape(want.shape), want, "diffattn")
+    torch._dynamo.reset()
+    Q, K, V = (torch.randn(1, 8, 96, 4, 32, generator=g).to(BF) for _ in range(3))
+    mb, pb = torch.randn(1, 8, 1, 1, 96, generator=g).to(BF), torch.randn(1, 1, 4, 96, 96, generator=g).to(BF)
+    got = torch.compile(lambda Q, K, V, a, b: A.attention_reference(Q, K, V, [a, b]), dynamic=False, fullgraph=True)(*dev(Q, K, V, mb, pb))
+    want = O.attention_evoformer(f(Q), f(K), f(V), [f(mb), f(pb)])
+    assert_parity(got.reshape(want.shape), want, "evoformer")

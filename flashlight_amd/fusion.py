@@ -950,4 +950,19 @@ def backend(gm: fx.GraphModule, example_inputs):
     return gm.forward
 
 
+def backend_inductor(gm: fx.GraphModule, example_inputs):
+    """`backend="flashlight_amd_inductor"`: the same rewrite, then the rest of the graph goes to Inductor (the reference's
+    setting: its fused attention is one kernel inside an Inductor-compiled graph), which traces through the replacement
+    nodes down to the registered operators and keeps those as external kernels.  A graph in which a region drops
+    weights is not handed on (the seed of each call is drawn when the node runs; a tracer would freeze one into the
+    compiled code): it runs like `backend="flashlight_amd"`."""
+    fuse_attention(gm)
+    for n in gm.graph.nodes:
+        if n.op == "call_function" and n.target in (fused_attention, fused_multi_head_attention) and n.kwargs.get("dropout_p", 0.0):
+            return gm.forward
+    from torch._inductor.compile_fx import compile_fx
+    return compile_fx(gm, example_inputs)
+
+
 torch._dynamo.register_backend(compiler_fn=backend, name="flashlight_amd")
+torch._dynamo.register_backend(compiler_fn=backend_inductor, name="flashlight_amd_inductor")

@@ -271,6 +271,13 @@ def _pad_head_dims(q, k, v, gate, diff, bias_only=True, min_dim=32):
             None if gate is None else pad(gate, (0, pv - dv)))
 
 
+def _being_traced(*tensors) -> bool:
+    """True while Dynamo captures the caller, and while a tracer (AOTAutograd / make_fx under a compiler backend) runs
+    it on stand-in tensors: fake, functional or proxy tensors are subclasses and hold no memory to launch on, so such
+    calls go through the registered operators, which every tracer records as one node."""
+    return torch.compiler.is_compiling() or any(type(t) is not torch.Tensor for t in tensors if t is not None)
+
+
 def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=0, doc_ids=None, alibi_heads=0,
              softcap=0.0, biases=(), gate=None, diff=False, lambda_full=0.0, seq_major_out=False, dropout_p=0.0,
              dropout_seed=None, doc_workspace=None, score_fn=None) -> torch.Tensor:
@@ -312,7 +319,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         if diff or seq_major_out:
             raise NotImplementedError("dropout is not built for differential attention and sequence-major results")
         if dropout_seed is None:
-            if torch.compiler.is_compiling():
+            if _being_traced(q, k, v):
                 raise NotImplementedError("dropout under torch.compile needs an explicit dropout_seed (a seed drawn "
                                           "while tracing would be frozen into the graph)")
             dropout_seed = int(torch.randint(0, 2 ** 63 - 1, (1,), dtype=torch.int64).item())
@@ -322,12 +329,12 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         t is not None and t.requires_grad for t in (q, k, v, gate, *(b for b, _ in biases)))
     if score_fn is not None and (wants_grad or dropout_p > 0.0):
         raise NotImplementedError("score functions other than the tanh soft-cap are forward-only and take no dropout")
-    if wants_grad or (dropout_p > 0.0 and torch.compiler.is_compiling()):
+    if wants_grad or (dropout_p > 0.0 and _being_traced(q, k, v)):
         # (the result comes back in [B, H, L, Dv] memory order whatever seq_major_out asks for)
         return _differentiable(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                                alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
                                lambda_full=lambda_full, dropout_p=dropout_p, dropout_seed=dropout_seed)
-    if torch.compiler.is_compiling():
+    if _being_traced(q, k, v):
         bl = list(biases) + [(None, 1)] * (2 - len(biases))
         fn_kind, fn_c = (int(score_fn[0]), [float(c) for c in score_fn[1]]) if score_fn is not None else (0, [0.0] * 4)
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),

@@ -3,6 +3,7 @@
 tests/test_causal.py:14-17,33).  The CPU tests check what the rewrite recognises; the GPU tests check that the
 rewritten function returns what the eager one returns."""
 import functools
+import math
 
 import pytest
 import torch
@@ -625,3 +626,92 @@ def test_multi_head_attention_modules_on_gpu():
           dict(tgt_mask=causal, tgt_is_causal=True, memory_key_padding_mask=pad[:, :120]), 2, grads=False)
     check("three encoder layers", nn.TransformerEncoder(nn.TransformerEncoderLayer(E, H, 512, dropout=0.0, batch_first=True), 3,
                                                         enable_nested_tensor=False), (x,), dict(src_key_padding_mask=pad), 3, grads=False)
+
+
+def test_inductor_backend_keeps_graphs_with_dropout_out_of_the_tracer(monkeypatch):
+    """`backend="flashlight_amd_inductor"` hands the rewritten graph to Inductor, except when a region drops weights:
+    its seed is drawn per call, which a tracer would freeze."""
+    import torch._inductor.compile_fx as cfx
+    handed = []
+    monkeypatch.setattr(cfx, "compile_fx", lambda gm, ex: handed.append(gm) or gm.forward)
+    q, k, v = _qkv()
+
+    def capture(fn, *args):
+        got = []
+
+        class _Done(Exception):
+            pass
+
+        def be(gm, example_inputs):
+            got.append(fusion.backend_inductor(gm, example_inputs))
+
+            def run(*a):
+                raise _Done
+            return run
+
+        torch._dynamo.reset()
+        with pytest.raises(_Done):
+            torch.compile(fn, backend=be, dynamic=False, fullgraph=True)(*args)
+        return got[0]
+
+    capture(E.causal_triu, q, k, v)
+    assert len(handed) == 1
+    drop = lambda q, k, v: torch.nn.functional.dropout(torch.softmax(q @ k.transpose(-2, -1) * 0.1, dim=-1), 0.1, True) @ v
+    capture(drop, q, k, v)
+    assert len(handed) == 1
+    assert "flashlight_amd_inductor" in torch._dynamo.list_backends(exclude_tags=())
+
+
+@pytest.mark.gpu
+def test_rewrite_followed_by_inductor_on_gpu():
+    """A pre-norm transformer block (eager attention spelled out, causal) and a torch.nn encoder layer under
+    `backend="flashlight_amd_inductor"`: the attention on the fused kernel, everything else compiled by Inductor; results
+    and parameter gradients against the same module in fp32 on the CPU."""
+    import copy
+    import torch.nn as nn
+
+    class Block(nn.Module):
+        def __init__(self, E=256, H=4):
+            super().__init__()
+            self.H = H
+            self.qkv, self.o = nn.Linear(E, 3 * E), nn.Linear(E, E)
+            self.n1, self.n2 = nn.LayerNorm(E), nn.LayerNorm(E)
+            self.f1, self.f2 = nn.Linear(E, 2 * E), nn.Linear(2 * E, E)
+
+        def forward(self, x):
+            B, L, E = x.shape
+            q, k, v = self.qkv(self.n1(x)).view(B, L, 3, self.H, E // self.H).permute(2, 0, 3, 1, 4)
+            s = q @ k.transpose(-2, -1) / math.sqrt(E // self.H)
+            s = s.masked_fill(torch.ones(L, L, dtype=torch.bool, device=x.device).triu(1), float("-inf"))
+            a = torch.softmax(s, dim=-1) @ v
+            x = x + self.o(a.transpose(1, 2).reshape(B, L, E))
+            return x + self.f2(torch.tanh(self.f1(self.n2(x))))
+
+    torch.manual_seed(0)
+    x = torch.randn(2, 200, 256).to(BF)
+    pad = torch.zeros(2, 200, dtype=torch.bool)
+    pad[1, 120:] = True
+    for name, mod, kwargs in (("block", Block(), {}),
+                              ("encoder layer", nn.TransformerEncoderLayer(256, 4, 512, dropout=0.0, batch_first=True, activation=torch.tanh),
+                               dict(src_key_padding_mask=pad))):
+        ref = copy.deepcopy(mod).float().train()
+        m = mod.to(BF).to("cuda").train()
+        torch._dynamo.reset()
+        regions = []
+        real = fusion.fuse_attention
+        fusion.fuse_attention = lambda gm: regions.append(real(gm)) or regions[-1]
+        try:
+            got = torch.compile(m, backend="flashlight_amd_inductor", dynamic=False)(x.to("cuda"), **{k: v.to("cuda") for k, v in kwargs.items()})
+        finally:
+            fusion.fuse_attention = real
+        assert sum(regions) == 1, name   # (after the rewrite nothing but the fused kernel computes the attention)
+        want = ref(x.float(), **kwargs)
+        top = max(1.0, want.abs().max().item())
+        assert_parity(got, want, name, max_tol=3e-2 * top, mean_tol=3e-3 * top)
+        w = torch.randn(want.shape, generator=torch.Generator().manual_seed(5))
+        (want * w).sum().backward()
+        (got.float() * w.to("cuda")).sum().backward()
+        for (pn, p32), (_, p16) in zip(ref.named_parameters(), m.named_parameters()):
+            assert p16.grad is not None, f"{name}: {pn}"
+            err = (p16.grad.float().cpu() - p32.grad).abs().max().item()
+            assert err <= 4e-2 * p32.grad.abs().max().item() + 1e-3, f"{name}: gradient of {pn} off by {err}"

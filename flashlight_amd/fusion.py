@@ -390,7 +390,7 @@ class _Region:
         self.causal = False                  # scaled_dot_product_attention(is_causal=True)
 
 
-_PASS_OPS = ("to", "type_as", "float", "contiguous", "clone")
+_PASS_OPS = ("to", "type", "type_as", "float", "bfloat16", "half", "contiguous", "clone")
 _FN_OPS = ("relu", "sigmoid", "tanh", "clamp", "clip", "clamp_min", "clamp_max", "pow", "square", "neg", "sub", "rsub",
            "mul", "div", "add")
 
@@ -609,7 +609,7 @@ def _match(softmax: fx.Node) -> _Region:
             raise _NoMatch("the softmax weights have more than one consumer")
         (u,) = cur.users
         nm = _name(u)
-        if nm in ("to", "type_as", "float", "contiguous") and u.args[0] is cur:
+        if nm in _PASS_OPS and u.args and u.args[0] is cur:
             tail.append(u)
             cur = u
             continue

@@ -289,6 +289,16 @@ def test_rewrite_maps_scaled_dot_product_attention_calls():
     assert len(calls) == 1
 
 
+def test_rewrite_follows_casts_of_the_weights():
+    """Model code casts the fp32 softmax back in several spellings (`.to(dtype)`, `.type(dtype)`, `.type_as(v)`,
+    `.bfloat16()`): all are passed through on the way to the second matmul."""
+    q, k, v = _qkv()
+    for cast in (lambda w, v: w.to(v.dtype), lambda w, v: w.type(v.dtype), lambda w, v: w.type_as(v), lambda w, v: w.bfloat16()):
+        fn = lambda q, k, v: cast(torch.softmax((q @ k.transpose(-2, -1) * 0.1).float(), dim=-1), v) @ v
+        gm, calls = _rewrite(fn, q, k, v)
+        assert len(calls) == 1 and "softmax" not in _leftover(gm)
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)

@@ -657,7 +657,7 @@ def _match_sdpa(n: fx.Node) -> _Region:
         if not qs.size(0) == ks.size(0) == vs.size(0):
             raise _NoMatch("scaled_dot_product_attention operands [N, L, E] with different batch sizes")
     elif qs.dim() != 4 or ks.dim() != 4 or vs.dim() != 4 or qs.size(1) % ks.size(1) or ks.size(1) != vs.size(1) or \
-            (qs.size(1) != ks.size(1) and not gqa):
+            (qs.size(1) != ks.size(1) and not gqa and ks.size(1) != 1):   # (one key / value head broadcasts: multi-query)
         raise _NoMatch("scaled_dot_product_attention operands are not [N, H, L, E] with grouped heads (or [N, L, E])")
     r = _Region()
     r.q, r.k, r.v, r.out, r.nodes = q, k, v, n, [n]
@@ -671,6 +671,27 @@ def _match_sdpa(n: fx.Node) -> _Region:
         else:
             r.biases.append(mask)
     return r
+
+
+_HALF = (torch.bfloat16, torch.float16)
+
+
+def _undo_upcasts(r: _Region):
+    """Model code that multiplies in fp32 (`query.to(torch.float32) @ key.to(torch.float32).transpose(-1, -2)`, GPT-J's
+    and GPT-Neo's attention) hands the region fp32 copies of 16-bit tensors.  The kernel multiplies the 16-bit values
+    exactly and accumulates in fp32, which is what the upcast product computes, so it takes the tensors as they were:
+    applied when that leaves query, key and value in one 16-bit type."""
+    def source(n):
+        while isinstance(n, fx.Node) and _name(n) in ("to", "float", "type") and _val(n).dtype == torch.float32 and \
+                n.args and isinstance(n.args[0], fx.Node) and _val(n.args[0]).dtype in _HALF and \
+                _val(n.args[0]).shape == _val(n).shape:
+            n = n.args[0]
+        return n
+    if not all(isinstance(x, fx.Node) for x in (r.q, r.k, r.v)):
+        return
+    q, k, v = source(r.q), source(r.k), source(r.v)
+    if (q, k, v) != (r.q, r.k, r.v) and _val(q).dtype in _HALF and _val(q).dtype == _val(k).dtype == _val(v).dtype:
+        r.q, r.k, r.v = q, k, v
 
 
 def _shapes(r: _Region):
@@ -855,6 +876,7 @@ def fuse_attention(gm: fx.GraphModule) -> int:
     for sm in [n for n in gm.graph.nodes if _name(n) in ("softmax", "scaled_dot_product_attention")]:
         try:
             r = _match(sm) if _name(sm) == "softmax" else _match_sdpa(sm)
+            _undo_upcasts(r)
             gqa, L, S, Hq = _shapes(r)
             if not gqa and _val(r.q).dim() == 4:
                 # key / value heads that were repeated to match the query heads: hand the kernel the originals
@@ -928,6 +950,11 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                 bias_nodes.append(gm.graph.get_attr(name))
             new = gm.graph.call_function(fused_attention, (r.q, r.k, r.v, doc_ids, bias_nodes, run_masks),
                                          dict(kwargs, mask_invert=tuple(run_invert)))
+            out_dtype = _val(r.out).dtype
+            if out_dtype != _val(r.q).dtype and _val(r.q).dtype in _HALF:
+                # (operands that the region upcast to fp32: what follows still gets the region's own result type)
+                fused, new = new, gm.graph.call_method("to", (new, out_dtype))
+                fused.meta.update(r.out.meta)
         new.meta.update(r.out.meta)
         r.out.replace_all_uses_with(new)
         for n in r.nodes:

@@ -299,6 +299,29 @@ def test_rewrite_follows_casts_of_the_weights():
         assert len(calls) == 1 and "softmax" not in _leftover(gm)
 
 
+def test_rewrite_takes_16_bit_operands_that_the_region_upcast():
+    """GPT-J / GPT-Neo multiply in fp32: `query.to(torch.float32) @ key.to(torch.float32).transpose(-1, -2)`.  The kernel
+    gets the 16-bit tensors themselves (exact products, fp32 accumulation either way); a region whose result was fp32
+    keeps that type through a cast behind the fused node."""
+    q, k, v = _qkv()
+
+    def gptj(q, k, v):
+        w = torch.softmax(q.to(torch.float32) @ k.to(torch.float32).transpose(-1, -2) / 8.0, dim=-1)
+        return w.to(v.dtype) @ v
+
+    gm, calls = _rewrite(gptj, q, k, v)
+    assert len(calls) == 1 and all(fusion._val(a).dtype == BF for a in calls[0].args[:3])
+    assert not any(fusion._name(n) == "to" for n in calls[0].users)
+
+    def all_fp32(q, k, v):
+        return torch.softmax(q.float() @ k.float().transpose(-1, -2) / 8.0, dim=-1) @ v.float()
+
+    gm, calls = _rewrite(all_fp32, q, k, v)
+    assert len(calls) == 1 and all(fusion._val(a).dtype == BF for a in calls[0].args[:3])
+    (cast,) = calls[0].users
+    assert fusion._name(cast) == "to" and cast.args[1] == torch.float32
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)

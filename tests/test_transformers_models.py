@@ -21,10 +21,17 @@ CONFIGS = {
                                 vocab_size=1000), False),
     "gemma2": ("Gemma2Config", dict(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
                                     num_key_value_heads=2, head_dim=64, vocab_size=1000, sliding_window=64), True),
+    "gptj": ("GPTJConfig", dict(n_embd=256, n_layer=2, n_head=4, rotary_dim=32, vocab_size=1000), True),          # fp32 q k^T
+    "gpt_neo": ("GPTNeoConfig", dict(hidden_size=256, num_layers=2, num_heads=4, attention_types=[[["global", "local"], 1]],
+                                     window_size=16, vocab_size=1000), True),
+    "falcon": ("FalconConfig", dict(hidden_size=256, num_hidden_layers=2, num_attention_heads=4, vocab_size=1000), True),  # one K/V head
+    "mpt": ("MptConfig", dict(d_model=256, n_layers=2, n_heads=4, vocab_size=1000), True),                         # ALiBi as a bias
 }
 CASES = [("llama", "eager", "flashlight_amd"), ("llama", "sdpa", "flashlight_amd"), ("llama", "eager", "flashlight_amd_inductor"),
          ("gpt2", "eager", "flashlight_amd"), ("bert", "eager", "flashlight_amd"), ("bert", "sdpa", "flashlight_amd"),
-         ("gemma2", "eager", "flashlight_amd"), ("gemma2", "sdpa", "flashlight_amd_inductor")]
+         ("gemma2", "eager", "flashlight_amd"), ("gemma2", "sdpa", "flashlight_amd_inductor"),
+         ("gptj", "eager", "flashlight_amd"), ("gpt_neo", "eager", "flashlight_amd"), ("falcon", "sdpa", "flashlight_amd"),
+         ("falcon", "eager", "flashlight_amd"), ("mpt", "eager", "flashlight_amd")]
 
 
 @pytest.mark.gpu

@@ -869,9 +869,72 @@ def _rewrite_multi_head_attention(gm: fx.GraphModule) -> int:
     return replaced
 
 
+def _lower_einsums(gm: fx.GraphModule) -> int:
+    """Two-operand `torch.einsum` calls that are a batched matrix product — one contracted letter, one letter of the
+    result from each operand alone, the rest batch letters present everywhere, e.g. "bhid,bhjd->bhij" and
+    "bhij,bhjd->bhid", or with sequence-major operands "bqhd,bkhd->bhqk" — are rewritten as permute / transpose / matmul
+    nodes (the same computation), so that attention spelled with einsum meets the matcher as matmuls.  Returns the
+    number of calls rewritten."""
+    lowered = 0
+    for n in list(gm.graph.nodes):
+        if _name(n) != "einsum" or not n.args or not isinstance(n.args[0], str) or n.kwargs:
+            continue
+        operands = tuple(n.args[1]) if len(n.args) == 2 and isinstance(n.args[1], (list, tuple)) else tuple(n.args[1:])
+        eq = n.args[0].replace(" ", "")
+        if len(operands) != 2 or not all(isinstance(x, fx.Node) for x in operands) or "." in eq or eq.count("->") != 1:
+            continue
+        lhs, C = eq.split("->")
+        if lhs.count(",") != 1:
+            continue
+        A, B = lhs.split(",")
+        sa, sb, sc = set(A), set(B), set(C)
+        if len(sa) != len(A) or len(sb) != len(B) or len(sc) != len(C):
+            continue
+        contracted, only_a, only_b, batch = (sa & sb) - sc, (sa & sc) - sb, (sb & sc) - sa, sa & sb & sc
+        if len(contracted) != 1 or len(only_a) != 1 or len(only_b) != 1 or sa != batch | contracted | only_a or \
+                sb != batch | contracted | only_b or sc != batch | only_a | only_b:
+            continue
+        (c,), (i,), (j,) = contracted, only_a, only_b
+        lead = [x for x in C if x in batch]
+        a, b = operands
+        try:
+            va, vb = _val(a), _val(b)
+            if va.dim() != len(A) or vb.dim() != len(B):
+                continue
+            perm_a = [A.index(x) for x in lead + [i, c]]
+            perm_b = [B.index(x) for x in lead + [j, c]]
+            perm_c = [(lead + [i, j]).index(x) for x in C]
+            ident = lambda perm: perm == list(range(len(perm)))
+            va1 = va if ident(perm_a) else va.permute(*perm_a)
+            direct_b = list(B) == lead + [c, j]            # already [.., contracted, j]: the second operand as it is
+            vb1 = vb if direct_b or ident(perm_b) else vb.permute(*perm_b)
+            vb2 = vb1 if direct_b else vb1.transpose(-2, -1)
+            vmm = torch.matmul(va1, vb2)
+            vout = vmm if ident(perm_c) else vmm.permute(*perm_c)
+        except Exception:  # noqa: BLE001 - an einsum this cannot express stays as it is
+            continue
+
+        def node(kind, target, args, value):
+            y = gm.graph.call_method(target, args) if kind == "method" else gm.graph.call_function(target, args)
+            y.meta["example_value"] = value
+            return y
+
+        with gm.graph.inserting_before(n):
+            a1 = a if ident(perm_a) else node("method", "permute", (a, *perm_a), va1)
+            b1 = b if direct_b or ident(perm_b) else node("method", "permute", (b, *perm_b), vb1)
+            b2 = b1 if direct_b else node("method", "transpose", (b1, -2, -1), vb2)
+            mm = node("function", torch.matmul, (a1, b2), vmm)
+            out = mm if ident(perm_c) else node("method", "permute", (mm, *perm_c), vout)
+        n.replace_all_uses_with(out)
+        gm.graph.erase_node(n)
+        lowered += 1
+    return lowered
+
+
 def fuse_attention(gm: fx.GraphModule) -> int:
     """Rewrites every attention region of `gm` (a Dynamo-captured graph with example values on its nodes) in place.
     Returns the number of regions replaced."""
+    lowered = _lower_einsums(gm)
     replaced = _rewrite_multi_head_attention(gm)
     for sm in [n for n in gm.graph.nodes if _name(n) in ("softmax", "scaled_dot_product_attention")]:
         try:
@@ -963,6 +1026,7 @@ def fuse_attention(gm: fx.GraphModule) -> int:
         replaced += 1
     if replaced:
         _merge_differential(gm)
+    if replaced or lowered:
         gm.graph.eliminate_dead_code()
         gm.graph.lint()
         gm.recompile()

@@ -221,3 +221,19 @@ def decoder_layer_attention_softcapped(query, key, value, attention_mask, softca
     attn_weights = attn_weights + attention_mask
     attn_weights = F.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query.dtype)
     return torch.matmul(attn_weights, value)
+
+
+def einsum_attention(q, k, v, mask=None):
+    """Attention spelled with einsum on [B, H, L, E] operands, as research code often writes it."""
+    s = torch.einsum("bhid,bhjd->bhij", q, k) * q.size(-1) ** -0.5
+    if mask is not None:
+        s = s.masked_fill(~mask, float("-inf"))
+    return torch.einsum("bhij,bhjd->bhid", s.softmax(dim=-1), v)
+
+
+def einsum_attention_seq_major(q, k, v):
+    """The same on [B, L, H, E] operands (the layout projections produce), causal, result [B, L, H, E]."""
+    L, S = q.size(1), k.size(1)
+    s = torch.einsum("bqhd,bkhd->bhqk", q, k) / math.sqrt(q.size(-1))
+    s = s.masked_fill(torch.ones(L, S, dtype=torch.bool, device=q.device).triu(1), float("-inf"))
+    return torch.einsum("bhqk,bkhd->bqhd", torch.softmax(s, dim=-1), v)

@@ -322,6 +322,22 @@ def test_rewrite_takes_16_bit_operands_that_the_region_upcast():
     assert fusion._name(cast) == "to" and cast.args[1] == torch.float32
 
 
+def test_rewrite_takes_attention_spelled_with_einsum():
+    """einsum calls that are batched matrix products become permute / matmul nodes first, so the matcher sees them; an
+    einsum of another kind stays."""
+    q, k, v = _qkv(Hq=4, Hkv=4)
+    keep = torch.rand(2, 1, 48, 48) > 0.2
+    gm, calls = _rewrite(E.einsum_attention, q, k, v, keep)
+    assert len(calls) == 1 and "einsum" not in {fusion._name(n) for n in gm.graph.nodes}
+    qs, ks, vs = (t.transpose(1, 2).contiguous() for t in (q, k, v))   # [N, L, H, E]
+    gm, calls = _rewrite(E.einsum_attention_seq_major, qs, ks, vs)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL
+    assert tuple(fusion._val(calls[0].args[0]).shape) == tuple(q.shape)   # handed over as [N, H, L, E] views
+    # an outer product and a trace are not matrix products of this kind
+    gm, calls = _rewrite(lambda a, b: torch.einsum("bhid,bhjd->bhijd", a, b).sum(-1), q, k)
+    assert calls == [] and "einsum" in {fusion._name(n) for n in gm.graph.nodes}
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)
@@ -748,3 +764,32 @@ def test_rewrite_followed_by_inductor_on_gpu():
             assert p16.grad is not None, f"{name}: {pn}"
             err = (p16.grad.float().cpu() - p32.grad).abs().max().item()
             assert err <= 4e-2 * p32.grad.abs().max().item() + 1e-3, f"{name}: gradient of {pn} off by {err}"
+
+
+@pytest.mark.gpu
+def test_rewritten_einsum_attention_on_gpu():
+    g = torch.Generator().manual_seed(17)
+    B, H, L, S, D = 2, 4, 150, 210, 64
+    q = torch.randn(B, H, L, D, generator=g).to(BF).to("cuda")
+    k, v = (torch.randn(B, H, S, D, generator=g).to(BF).to("cuda") for _ in range(2))
+    keep = (torch.rand(B, 1, L, S, generator=g) > 0.3).to("cuda")
+    keep[..., 0] = True
+    torch._dynamo.reset()
+    got = torch.compile(E.einsum_attention, backend=fusion.backend, dynamic=False, fullgraph=True)(q, k, v, keep)
+    assert_parity(got, E.einsum_attention(q.float().cpu(), k.float().cpu(), v.float().cpu(), keep.cpu()), "einsum, mask")
+    qs, ks, vs = (t.transpose(1, 2).contiguous() for t in (q, k, v))   # [B, L, H, E]
+    torch._dynamo.reset()
+    got = torch.compile(E.einsum_attention_seq_major, backend=fusion.backend, dynamic=False, fullgraph=True)(qs, ks, vs)
+    assert got.shape == (B, L, H, D)
+    assert_parity(got, E.einsum_attention_seq_major(qs.float().cpu(), ks.float().cpu(), vs.float().cpu()), "einsum, sequence-major")
+    # gradients through the lowered graph
+    torch._dynamo.reset()
+    leaves = [t.clone().requires_grad_(True) for t in (qs, ks, vs)]
+    out = torch.compile(E.einsum_attention_seq_major, backend=fusion.backend, dynamic=False, fullgraph=True)(*leaves)
+    w = torch.randn(out.shape, generator=g)
+    (out.float() * w.to("cuda")).sum().backward()
+    refs = [t.float().cpu().requires_grad_(True) for t in (qs, ks, vs)]
+    (E.einsum_attention_seq_major(*refs) * w).sum().backward()
+    for name, a, b in zip(("dq", "dk", "dv"), leaves, refs):
+        scale = max(1.0, b.grad.abs().max().item())
+        assert_parity(a.grad / scale, b.grad / scale, name)

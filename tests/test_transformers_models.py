@@ -112,3 +112,85 @@ def test_transformers_training_step(name, impl, backend):
         worst = max(worst, (pm.grad.float().cpu() - p32.grad).abs().max().item() / top)
         yard = max(yard, (pe.grad.float().cpu() - p32.grad).abs().max().item() / top)
     assert worst <= max(2.0 * yard, 0.03), (worst, yard)
+
+
+def _more_specs():
+    T = transformers
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(3, 1000, (2, 96), generator=g)
+    attend = torch.ones(2, 96, dtype=torch.long)
+    attend[1, 70:] = 0
+    text = dict(input_ids=ids, attention_mask=attend)
+    seq2seq = dict(input_ids=ids, attention_mask=attend, decoder_input_ids=ids[:, :40])
+    image = dict(pixel_values=torch.randn(2, 3, 64, 64, generator=g))
+    enc = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4, vocab_size=1000)
+    bart = dict(d_model=256, encoder_layers=2, decoder_layers=2, encoder_attention_heads=4, decoder_attention_heads=4,
+                encoder_ffn_dim=512, decoder_ffn_dim=512, vocab_size=1000)
+    lm, s2s, base = T.AutoModelForCausalLM, T.AutoModelForSeq2SeqLM, T.AutoModel
+    # name: (auto class, config class, config arguments, inputs, result field, fused launches expected)
+    return {
+        "t5": (s2s, "T5Config", dict(d_model=256, d_kv=64, d_ff=512, num_layers=2, num_heads=4, vocab_size=1000), seq2seq, "logits", 6),
+        "bart": (s2s, "BartConfig", bart, seq2seq, "logits", 6),
+        "marian": (s2s, "MarianConfig", dict(bart, pad_token_id=0, decoder_start_token_id=0), seq2seq, "logits", 6),
+        "gpt_neox": (lm, "GPTNeoXConfig", enc, text, "logits", 2),
+        "opt": (lm, "OPTConfig", dict(hidden_size=256, ffn_dim=512, num_hidden_layers=2, num_attention_heads=4,
+                                      word_embed_proj_dim=256, vocab_size=1000), text, "logits", 2),
+        "phi3": (lm, "Phi3Config", dict(enc, num_attention_heads=8, num_key_value_heads=2, pad_token_id=0), text, "logits", 2),
+        "qwen2": (lm, "Qwen2Config", dict(enc, num_attention_heads=8, num_key_value_heads=2), text, "logits", 2),
+        "mistral": (lm, "MistralConfig", dict(enc, num_attention_heads=8, num_key_value_heads=2, sliding_window=32), text, "logits", 2),
+        "distilbert": (base, "DistilBertConfig", dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, vocab_size=1000), text,
+                       "last_hidden_state", 2),
+        "roberta": (base, "RobertaConfig", enc, text, "last_hidden_state", 2),
+        "electra": (base, "ElectraConfig", dict(enc, embedding_size=128), text, "last_hidden_state", 2),
+        "esm": (base, "EsmConfig", dict(enc, vocab_size=33, pad_token_id=1, position_embedding_type="rotary"),
+                dict(input_ids=ids % 30 + 3, attention_mask=attend), "last_hidden_state", 2),
+        "vit": (base, "ViTConfig", dict(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                                        image_size=64, patch_size=8), image, "last_hidden_state", 2),
+        "swin": (base, "SwinConfig", dict(image_size=64, patch_size=4, embed_dim=64, depths=[2, 2], num_heads=[2, 4], window_size=4),
+                 image, "last_hidden_state", 4),
+        # attention of other shapes (disentangled / relative terms inside the scores, baddbmm on merged heads): left alone
+        "deberta-v2": (base, "DebertaV2Config", enc, text, "last_hidden_state", 0),
+        "xlnet": (base, "XLNetConfig", dict(d_model=256, n_layer=2, n_head=4, d_inner=512, vocab_size=1000), text, "last_hidden_state", 0),
+        "bloom": (lm, "BloomConfig", dict(hidden_size=256, n_layer=2, n_head=4, vocab_size=1000), text, "logits", 0),
+    }
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["t5", "bart", "marian", "gpt_neox", "opt", "phi3", "qwen2", "mistral", "distilbert", "roberta",
+                                  "electra", "esm", "vit", "swin", "deberta-v2", "xlnet", "bloom"])
+def test_more_architectures(name):
+    """Encoder-decoders (cross attention, T5's learned position bias as a run-time operand), more decoders and encoders,
+    vision models (Swin's windows with their bias table): matched and right — or, for attention of another shape, left
+    alone and right."""
+    auto, cls, kw, inputs, field, expected = _more_specs()[name]
+    if not hasattr(transformers, cls):
+        pytest.skip(f"this transformers has no {cls}")
+    torch.manual_seed(1)
+    model = auto.from_config(getattr(transformers, cls)(**kw), attn_implementation="eager").eval()
+    ref = copy.deepcopy(model).float()
+    m = model.to(torch.bfloat16).to("cuda")
+    dev = {k: (v.to(torch.bfloat16) if v.is_floating_point() else v).cuda() for k, v in inputs.items()}
+    launches = [0]
+    real = ops.dispatch
+
+    def counting(*a, **k):
+        launches[0] += 1
+        return real(*a, **k)
+
+    with torch.no_grad():
+        want = getattr(ref(**inputs), field)
+        eager = getattr(m(**dev), field).float().cpu()
+        torch._dynamo.reset()
+        ops.dispatch = counting
+        try:
+            got = getattr(torch.compile(m, backend="flashlight_amd", dynamic=False)(**dev), field).float().cpu()
+        finally:
+            ops.dispatch = real
+    assert launches[0] == expected
+    attend = inputs.get("attention_mask")
+    if attend is not None and "decoder_input_ids" not in inputs:
+        keep = attend.bool()
+        got, want, eager = got[keep], want[keep], eager[keep]
+    assert torch.isfinite(got).all()
+    err, yard = (got - want).abs().max().item(), (eager - want).abs().max().item()
+    assert err <= max(2.5 * yard, 0.02 * want.abs().max().item()), (err, yard)

@@ -992,8 +992,17 @@ def fuse_attention(gm: fx.GraphModule) -> int:
                 if isinstance(b, torch.Tensor):
                     if plain and kwargs["alibi_heads"] == 0 and _is_alibi(b, Hq, L, S):
                         kwargs["alibi_heads"] = Hq
-                    else:
-                        const_biases.append(b)
+                        continue
+                    # a constant additive mask (zeros and fills <= -1e9, the way model code builds its causal mask when
+                    # no padding mask is given): the same positional forms as a boolean one
+                    as_mask = b <= -1e9
+                    if b.is_floating_point() and kwargs["mask_kind"] == _ffi.MASK_NONE and bool(as_mask.any()) and \
+                            bool(((b == 0) | as_mask).all()):
+                        got = _classify_constant_mask(as_mask, L, S)
+                        if got is not None and got[0] != _ffi.MASK_NONE:
+                            kwargs.update(mask_kind=got[0], window=got[1], prefix=got[2])
+                            continue
+                    const_biases.append(b)
                 else:
                     run_biases.append(node)
             if r.dropout_p:
@@ -1052,7 +1061,29 @@ def backend_inductor(gm: fx.GraphModule, example_inputs):
         if n.op == "call_function" and n.target in (fused_attention, fused_multi_head_attention) and n.kwargs.get("dropout_p", 0.0):
             return gm.forward
     from torch._inductor.compile_fx import compile_fx
-    return compile_fx(gm, example_inputs)
+    # constants of the rewrite (dense masks it evaluated) become inputs of the graph: the compiler takes tensors through
+    # placeholders, not through attributes added to a captured module
+    consts: List[torch.Tensor] = []
+    last_placeholder = None
+    for n in gm.graph.nodes:
+        if n.op == "placeholder":
+            last_placeholder = n
+    for n in list(gm.graph.nodes):
+        if n.op == "get_attr" and isinstance(n.target, str) and n.target.startswith("_flashlight_const_"):
+            t = getattr(gm, n.target)
+            with (gm.graph.inserting_after(last_placeholder) if last_placeholder is not None else gm.graph.inserting_before(None)):
+                ph = gm.graph.placeholder(n.target)
+            ph.meta.update(n.meta)
+            n.replace_all_uses_with(ph)
+            gm.graph.erase_node(n)
+            last_placeholder = ph
+            consts.append(t)
+    if not consts:
+        return compile_fx(gm, example_inputs)
+    gm.graph.lint()
+    gm.recompile()
+    compiled = compile_fx(gm, list(example_inputs) + consts)
+    return lambda *args: compiled(*args, *consts)
 
 
 torch._dynamo.register_backend(compiler_fn=backend, name="flashlight_amd")

@@ -338,6 +338,32 @@ def test_rewrite_takes_attention_spelled_with_einsum():
     assert calls == [] and "einsum" in {fusion._name(n) for n in gm.graph.nodes}
 
 
+def test_rewrite_reads_constant_additive_masks_as_positional_masks():
+    """Model code that gets no padding mask builds its causal (or sliding-window) mask as a constant additive tensor, zeros
+    and the dtype's most negative number: it becomes the kernel's positional mask, not a dense bias operand."""
+    q, k, v = _qkv()
+    L = q.size(2)
+
+    def causal_additive(q, k, v):
+        mask = torch.full((L, L), torch.finfo(q.dtype).min, dtype=q.dtype).triu(1)[None, None]
+        return torch.softmax(q @ k.transpose(-2, -1) * 0.125 + mask, dim=-1) @ v
+
+    gm, calls = _rewrite(causal_additive, q, k, v)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_CAUSAL and not calls[0].args[4]
+
+    def window_additive(q, k, v):
+        i = torch.arange(L)
+        out = (i[None, :] > i[:, None]) | (i[:, None] - i[None, :] > 7)
+        mask = torch.zeros(L, L).masked_fill(out, float("-inf"))
+        return torch.softmax(q @ k.transpose(-2, -1) * 0.125 + mask, dim=-1) @ v
+
+    gm, calls = _rewrite(window_additive, q, k, v)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_SLIDING and calls[0].kwargs["window"] == 7
+    # a constant bias with other values stays a dense operand
+    gm, calls = _rewrite(lambda q, k, v: torch.softmax(q @ k.transpose(-2, -1) * 0.125 + torch.ones(L, L).tril() * -3.0, dim=-1) @ v, q, k, v)
+    assert len(calls) == 1 and calls[0].kwargs["mask_kind"] == _ffi.MASK_NONE and len(calls[0].args[4]) == 1
+
+
 def test_rewrite_leaves_other_graphs_alone():
     q, k, v = _qkv()
     gm, calls = _rewrite(E.returns_weights, q, k, v)
@@ -740,6 +766,18 @@ def test_rewrite_followed_by_inductor_on_gpu():
     x = torch.randn(2, 200, 256).to(BF)
     pad = torch.zeros(2, 200, dtype=torch.bool)
     pad[1, 120:] = True
+    # a constant mask of no positional form is a dense operand the rewrite made: it reaches Inductor as a graph input
+    pattern = torch.rand(200, 200, generator=torch.Generator().manual_seed(9)) > 0.4
+    pattern[:, 0] = True
+
+    def patterned(q, k, v):
+        s = (q @ k.transpose(-2, -1)) * 0.125
+        return torch.softmax(s.masked_fill(~pattern.to(q.device), float("-inf")), dim=-1) @ v
+
+    q, k, v = (torch.randn(2, 4, 200, 64).to(BF).to("cuda") for _ in range(3))
+    torch._dynamo.reset()
+    got = torch.compile(patterned, backend="flashlight_amd_inductor", dynamic=False)(q, k, v)
+    assert_parity(got, patterned(q.float().cpu(), k.float().cpu(), v.float().cpu()), "constant pattern")
     for name, mod, kwargs in (("block", Block(), {}),
                               ("encoder layer", nn.TransformerEncoderLayer(256, 4, 512, dropout=0.0, batch_first=True, activation=torch.tanh),
                                dict(src_key_padding_mask=pad))):

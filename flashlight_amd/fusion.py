@@ -473,7 +473,7 @@ def _peel_scores(n: Any, r: _Region, qk_memo, mods_below: List[str]):
     nm = _name(n)
     if nm is None:
         raise _NoMatch("scores do not come from a matmul")
-    if nm in ("to", "type_as", "float", "contiguous", "clone"):
+    if nm in _PASS_OPS:
         r.nodes.append(n)
         return _peel_scores(n.args[0], r, qk_memo, mods_below)
     if nm == "matmul":

@@ -271,6 +271,39 @@ def _pad_head_dims(q, k, v, gate, diff, bias_only=True, min_dim=32):
             None if gate is None else pad(gate, (0, pv - dv)))
 
 
+def _split_over_keys(q, k, v, scale, softcap):
+    """Few queries against many keys (a decoding step over a long cache): B * Hq workgroups cannot fill 256 CUs, so the
+    keys are cut into C chunks that run as C times as many heads of one launch, each leaving a normalised partial result
+    and its row statistic, and the partial results are merged with the weights 2^(lse_c - max).  Returns None when the
+    call is not of that shape (enough workgroups already, short or indivisible key length, key / value tensors whose
+    heads are not contiguous in memory), and the caller launches as usual."""
+    B, Hq, Lq, D = q.shape
+    Hkv, Lk, Dv = k.size(1), k.size(2), v.size(3)
+    groups = B * Hq * ((Lq + 127) // 128)
+    # (a workgroup walks about 64 keys per microsecond and the merge below costs about 50: worth it from 8192 keys on)
+    if groups >= 256 or Lk < 8192 or Hq % Hkv or not (k.is_contiguous() and v.is_contiguous()):
+        return None
+    chunks = 0
+    for c in (64, 32, 16, 8, 4, 2):
+        if Lk % c == 0 and Lk // c >= 512 and (Lk // c) % 8 == 0 and groups * c <= 2048:
+            chunks = c
+            break
+    if not chunks:
+        return None
+    G, Lc = Hq // Hkv, Lk // chunks
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    # chunk c of key / value head h becomes head h * C + c; its G query heads are copies of the G of head h
+    qc = q.reshape(B, Hkv, 1, G, Lq, D).expand(B, Hkv, chunks, G, Lq, D).reshape(B, Hkv * chunks * G, Lq, D)
+    kc, vc = k.view(B, Hkv * chunks, Lc, D), v.view(B, Hkv * chunks, Lc, Dv)
+    lse = torch.empty(B, Hkv * chunks * G, Lq, dtype=torch.float32, device=q.device)
+    part = _ffi.attn_fwd(qc, kc, vc, scale=scale, softcap=softcap, lse=lse)
+    lse = lse.view(B, Hkv, chunks, G, Lq)
+    w = torch.exp2(lse - lse.amax(dim=2, keepdim=True))
+    merged = (w.unsqueeze(-1) * part.view(B, Hkv, chunks, G, Lq, Dv)).sum(dim=2) / w.sum(dim=2).unsqueeze(-1)
+    return merged.to(q.dtype).view(B, Hq, Lq, Dv)
+
+
 def _being_traced(*tensors) -> bool:
     """True while Dynamo captures the caller, and while a tracer (AOTAutograd / make_fx under a compiler backend) runs
     it on stand-in tensors: fake, functional or proxy tensors are subclasses and hold no memory to launch on, so such
@@ -340,6 +373,11 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),
                         doc_ids, int(alibi_heads), float(softcap), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), gate,
                         bool(diff), float(lambda_full), bool(seq_major_out), fn_kind, fn_c[0], fn_c[1], fn_c[2], fn_c[3])
+    if mask_kind == _ffi.MASK_NONE and not biases and gate is None and not diff and doc_ids is None and not alibi_heads \
+            and score_fn is None and dropout_p == 0.0 and not seq_major_out:
+        split = _split_over_keys(q, k, v, scale, softcap)
+        if split is not None:
+            return split
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None
     return _ffi.attn_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                          alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,

@@ -857,3 +857,30 @@ def test_calls_from_several_threads_on_streams_of_their_own():
         t.join(120)
     assert not any(t.is_alive() for t in threads), "a worker did not finish"
     assert errors == [], errors
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 32, 8, 1, 32768, 128), (2, 8, 8, 7, 8192, 64), (1, 4, 1, 130, 12288, 128), (1, 16, 4, 1, 65536, 128),
+                                   (1, 6, 2, 3, 8200, 64)])
+def test_few_queries_against_a_long_cache_are_split_over_the_keys(shape):
+    """A decoding step: B * Hq workgroups cannot fill the chip, so the front end runs the key chunks as extra heads of one
+    launch and merges the partial results by their row statistics.  Against eager fp32; the last shape's key length has
+    no usable divisor and takes the ordinary launch."""
+    import torch.nn.functional as F
+    from flashlight_amd import ops
+    B, Hq, Hkv, Lq, Lk, D = shape
+    g = torch.Generator().manual_seed(Lk + Lq)
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(torch.bfloat16)
+    k, v = (torch.randn(B, Hkv, Lk, D, generator=g).to(torch.bfloat16) for _ in range(2))
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    assert (ops._split_over_keys(qd, kd, vd, None, 0.0) is not None) == (Lk % 16 == 0)
+    got = A.attention_pytorch(qd, kd, vd, enable_gqa=True)
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), enable_gqa=True)
+    assert_parity(got, want, str(shape), max_tol=2e-3, mean_tol=2e-4)
+    # a soft-cap goes along; a cache whose heads are not contiguous (a slice of a longer buffer) is not split
+    got = A.attention_softcapped(qd, kd, vd, score_mod=A.generate_tanh_softcap(20.0), enable_gqa=True)
+    want = O.attention_softcapped(q.float(), k.float(), v.float(), score_mod=20.0, enable_gqa=True)
+    assert_parity(got.reshape(want.shape), want, str(shape) + " soft-cap", max_tol=2e-3, mean_tol=2e-4)
+    longer = torch.randn(B, Hkv, Lk + 64, D, generator=g).to(torch.bfloat16).cuda()
+    if B * Hkv > 1:   # (with one head in all the slice is still one contiguous block)
+        assert ops._split_over_keys(qd, longer[:, :, :Lk], longer[:, :, :Lk], None, 0.0) is None

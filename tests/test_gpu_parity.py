@@ -884,3 +884,31 @@ def test_few_queries_against_a_long_cache_are_split_over_the_keys(shape):
     longer = torch.randn(B, Hkv, Lk + 64, D, generator=g).to(torch.bfloat16).cuda()
     if B * Hkv > 1:   # (with one head in all the slice is still one contiguous block)
         assert ops._split_over_keys(qd, longer[:, :, :Lk], longer[:, :, :Lk], None, 0.0) is None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(4, 32, 8, 1, 2048, 128), (3, 12, 2, 5, 333, 64), (2, 8, 1, 16, 1000, 32), (1, 64, 8, 2, 8192, 128),
+                                   (2, 6, 3, 40, 77, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_grouped_heads_with_few_queries_are_packed_as_rows(shape, dtype):
+    """Unmasked grouped-query attention with few queries per head (decoding): the front end hands the kernel the G query
+    heads of a key / value head as G times as many rows of that head.  Same results as eager fp32, through every variant
+    that has no mask; a causal call is not packed and stays right."""
+    import torch.nn.functional as F
+    B, Hq, Hkv, Lq, Lk, D = shape
+    g = torch.Generator().manual_seed(Lk * 7 + Lq)
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(dtype)
+    k, v = (torch.randn(B, Hkv, Lk, D, generator=g).to(dtype) for _ in range(2))
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), enable_gqa=True)
+    assert_parity(A.attention_pytorch(qd, kd, vd, enable_gqa=True), want, f"{shape} vanilla")
+    want = O.attention_softcapped(q.float(), k.float(), v.float(), score_mod=20.0, enable_gqa=True)
+    got = A.attention_softcapped(qd, kd, vd, score_mod=A.generate_tanh_softcap(20.0), enable_gqa=True)
+    assert_parity(got.reshape(want.shape), want, f"{shape} soft-cap")
+    want = O.attention_causal(q.float(), k.float(), v.float(), enable_gqa=True)
+    got = A.attention_pytorch_causal(qd, kd, vd, enable_gqa=True)
+    assert_parity(got.reshape(want.shape), want, f"{shape} causal")
+    # a query tensor that is a strided view is not packed (no view of it has the rows adjacent) and stays right
+    wide = torch.randn(B, Hq, Lq, D + 8, generator=g).to(dtype).cuda()
+    want = F.scaled_dot_product_attention(wide[..., :D].float().cpu(), k.float(), v.float(), enable_gqa=True)
+    assert_parity(A.attention_pytorch(wide[..., :D], kd, vd, enable_gqa=True), want, f"{shape} strided q")

@@ -373,17 +373,19 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),
                         doc_ids, int(alibi_heads), float(softcap), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), gate,
                         bool(diff), float(lambda_full), bool(seq_major_out), fn_kind, fn_c[0], fn_c[1], fn_c[2], fn_c[3])
-    if mask_kind == _ffi.MASK_NONE and not biases and gate is None and not diff and doc_ids is None and not alibi_heads \
-            and score_fn is None and dropout_p == 0.0 and not seq_major_out:
+    if mask_kind == _ffi.MASK_NONE and gate is None and not diff and doc_ids is None and not alibi_heads \
+            and score_fn is None and dropout_p == 0.0 and not seq_major_out and \
+            all(b.dim() == 4 and b.size(1) == 1 and b.size(2) == 1 for b, _ in biases):
         Hq, Hkv, Lq = q.size(1), k.size(1), q.size(2)
         if Hq > Hkv and Hq % Hkv == 0 and (Hq // Hkv) * Lq <= 128 and q.is_contiguous():
             # few queries per head under grouped heads (a decoding step): without a mask the rows of a score matrix are
             # independent, so the G query heads of one key / value head are G times as many rows of that head (a view
             # of q), and one workgroup reads the keys for all of them instead of G workgroups reading them G times
-            packed = dispatch(q.view(q.size(0), Hkv, (Hq // Hkv) * Lq, q.size(3)), k, v, softcap=softcap,
+            # (a bias that is one row of keys per batch entry, a padding mask, is the same for every row and goes along)
+            packed = dispatch(q.view(q.size(0), Hkv, (Hq // Hkv) * Lq, q.size(3)), k, v, softcap=softcap, biases=biases,
                               scale=scale if scale is not None else 1.0 / math.sqrt(q.size(-1)))
             return packed.view(q.size(0), Hq, Lq, v.size(3))
-        split = _split_over_keys(q, k, v, scale, softcap)
+        split = None if biases else _split_over_keys(q, k, v, scale, softcap)
         if split is not None:
             return split
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None

@@ -908,6 +908,14 @@ def test_grouped_heads_with_few_queries_are_packed_as_rows(shape, dtype):
     want = O.attention_causal(q.float(), k.float(), v.float(), enable_gqa=True)
     got = A.attention_pytorch_causal(qd, kd, vd, enable_gqa=True)
     assert_parity(got.reshape(want.shape), want, f"{shape} causal")
+    # a padding mask (one row of keys per batch entry, added to every head and row) goes along with the packed rows
+    pad = torch.zeros(B, 1, 1, Lk)
+    pad[:, :, :, Lk // 3:Lk // 2] = float("-inf")
+    pad[0, :, :, :Lk // 4] = -1e9
+    from flashlight_amd import ops
+    got = ops.dispatch(qd, kd, vd, biases=[(pad.to(dtype).cuda(), 1)])
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=pad, enable_gqa=True)
+    assert_parity(got, want, f"{shape} padding mask")
     # a query tensor that is a strided view is not packed (no view of it has the rows adjacent) and stays right
     wide = torch.randn(B, Hq, Lq, D + 8, generator=g).to(dtype).cuda()
     want = F.scaled_dot_product_attention(wide[..., :D].float().cpu(), k.float(), v.float(), enable_gqa=True)

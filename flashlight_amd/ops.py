@@ -271,7 +271,7 @@ def _pad_head_dims(q, k, v, gate, diff, bias_only=True, min_dim=32):
             None if gate is None else pad(gate, (0, pv - dv)))
 
 
-def _split_over_keys(q, k, v, scale, softcap):
+def _split_over_keys(q, k, v, scale, softcap, biases=()):
     """Few queries against many keys (a decoding step over a long cache): B * Hq workgroups cannot fill 256 CUs, so the
     keys are cut into C chunks that run as C times as many heads of one launch, each leaving a normalised partial result
     and its row statistic, and the partial results are merged with the weights 2^(lse_c - max).  Returns None when the
@@ -296,11 +296,16 @@ def _split_over_keys(q, k, v, scale, softcap):
     # chunk c of key / value head h becomes head h * C + c; its G query heads are copies of the G of head h
     qc = q.reshape(B, Hkv, 1, G, Lq, D).expand(B, Hkv, chunks, G, Lq, D).reshape(B, Hkv * chunks * G, Lq, D)
     kc, vc = k.view(B, Hkv * chunks, Lc, D), v.view(B, Hkv * chunks, Lc, Dv)
+    # (biases here are rows of keys, [Nb, 1, 1, Lk]: chunk c of a row goes with chunk c of every head)
+    bc = [(b.view(b.size(0), 1, chunks, 1, Lc).expand(b.size(0), Hkv, chunks, G, Lc).reshape(b.size(0), Hkv * chunks * G, 1, Lc), d)
+          for b, d in biases]
     lse = torch.empty(B, Hkv * chunks * G, Lq, dtype=torch.float32, device=q.device)
-    part = _ffi.attn_fwd(qc, kc, vc, scale=scale, softcap=softcap, lse=lse)
+    part = _ffi.attn_fwd(qc, kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
     lse = lse.view(B, Hkv, chunks, G, Lq)
-    w = torch.exp2(lse - lse.amax(dim=2, keepdim=True))
-    merged = (w.unsqueeze(-1) * part.view(B, Hkv, chunks, G, Lq, Dv)).sum(dim=2) / w.sum(dim=2).unsqueeze(-1)
+    lse = torch.where(lse == float("inf"), torch.full_like(lse, float("-inf")), lse)   # (the kernel's mark for "no keys")
+    top = lse.amax(dim=2, keepdim=True)
+    w = torch.exp2(lse - torch.where(top == float("-inf"), torch.zeros_like(top), top))   # (a chunk, or a row, without keys: 0)
+    merged = (w.unsqueeze(-1) * part.view(B, Hkv, chunks, G, Lq, Dv)).sum(dim=2) / w.sum(dim=2).clamp_min(1e-30).unsqueeze(-1)
     return merged.to(q.dtype).view(B, Hq, Lq, Dv)
 
 
@@ -385,7 +390,7 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
             packed = dispatch(q.view(q.size(0), Hkv, (Hq // Hkv) * Lq, q.size(3)), k, v, softcap=softcap, biases=biases,
                               scale=scale if scale is not None else 1.0 / math.sqrt(q.size(-1)))
             return packed.view(q.size(0), Hq, Lq, v.size(3))
-        split = None if biases else _split_over_keys(q, k, v, scale, softcap)
+        split = _split_over_keys(q, k, v, scale, softcap, biases) if all(b.is_contiguous() for b, _ in biases) else None
         if split is not None:
             return split
     out = _alloc_out(q, v, diff, seq_major_out) if seq_major_out else None

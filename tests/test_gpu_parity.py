@@ -881,6 +881,16 @@ def test_few_queries_against_a_long_cache_are_split_over_the_keys(shape):
     got = A.attention_softcapped(qd, kd, vd, score_mod=A.generate_tanh_softcap(20.0), enable_gqa=True)
     want = O.attention_softcapped(q.float(), k.float(), v.float(), score_mod=20.0, enable_gqa=True)
     assert_parity(got.reshape(want.shape), want, str(shape) + " soft-cap", max_tol=2e-3, mean_tol=2e-4)
+    if Lk % 16 == 0:
+        # a padding mask is cut with the keys; a chunk it removes entirely, and a row it removes entirely, come out as zeros
+        pad = torch.zeros(B, 1, 1, Lk)
+        pad[:, :, :, Lk // 64:Lk // 3] = float("-inf")
+        pad[0, :, :, Lk // 2:] = -1e9
+        got = ops.dispatch(qd, kd, vd, biases=[(pad.to(torch.bfloat16).cuda(), 1)])
+        want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=pad, enable_gqa=True)
+        assert_parity(got, want, str(shape) + " padding mask", max_tol=2e-3, mean_tol=2e-4)
+        got = ops.dispatch(qd, kd, vd, biases=[(torch.full((B, 1, 1, Lk), float("-inf")).to(torch.bfloat16).cuda(), 1)])
+        assert torch.count_nonzero(got).item() == 0
     longer = torch.randn(B, Hkv, Lk + 64, D, generator=g).to(torch.bfloat16).cuda()
     if B * Hkv > 1:   # (with one head in all the slice is still one contiguous block)
         assert ops._split_over_keys(qd, longer[:, :, :Lk], longer[:, :, :Lk], None, 0.0) is None

@@ -124,6 +124,9 @@ def load_library(path: os.PathLike | str | None = None) -> C.CDLL:
     lib.fl_attn_bwd.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
     lib.fl_attn_bwd_static.restype = C.c_int
     lib.fl_attn_bwd_static.argtypes = [C.POINTER(FlAttnBwdParams), C.c_void_p]
+    lib.fl_attn_merge_chunks.restype = C.c_int
+    lib.fl_attn_merge_chunks.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_int32,
+                                         C.c_int32, C.c_void_p]
     lib.fl_ipa_pack.restype = C.c_int
     lib.fl_ipa_pack.argtypes = [C.POINTER(FlIpaPackParams), C.c_void_p]
     if lib.fl_version() != ABI_VERSION:
@@ -589,3 +592,19 @@ def probe_coissue(mfma_rows: int, valu_kind: str, valu_per_mfma: int, waves_per_
     c = cyc.double()
     per = 8.0 * iters * waves_per_simd
     return {"slowest_wave": float(c.max()) / per, "mean_wave": float(c.mean()) / per}
+
+
+def merge_chunks(part: torch.Tensor, lse: torch.Tensor) -> torch.Tensor:
+    """`fl_attn_merge_chunks`: part [outer, chunks, inner, dv] (bf16 / fp16) and lse [outer, chunks, inner] (fp32) of one
+    launch over key chunks -> [outer, inner, dv], the attention over all the keys.  One launch on the current stream."""
+    _require_gpu_half("part", part, None)
+    outer, chunks, inner, dv = part.shape
+    if lse.dtype != torch.float32 or tuple(lse.shape) != (outer, chunks, inner) or not (part.is_contiguous() and lse.is_contiguous()):
+        raise ValueError("merge_chunks: lse must be float32 [outer, chunks, inner], both operands contiguous")
+    out = torch.empty((outer, inner, dv), dtype=part.dtype, device=part.device)
+    rc = load_library().fl_attn_merge_chunks(C.c_void_p(part.data_ptr()), C.c_void_p(lse.data_ptr()), C.c_void_p(out.data_ptr()),
+                                             outer, chunks, inner, dv, _HALF_TYPES[part.dtype],
+                                             C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc != 0:
+        raise FlashlightError(rc, "fl_attn_merge_chunks rejected its arguments or could not launch")
+    return out

@@ -129,7 +129,7 @@ def build(force: bool = True, jobs: int | None = None, verbose: bool = False) ->
             tasks.append(([cc, *HIPCC_FLAGS, f"-DFL_INST_F16={f16}", "-c", str(CSRC / "pairbias_unit.hip"), "-o", str(o)], o))
     # the instance tables are host data only: compiling them for the device would reference the host launchers
     for src, extra in (("instances_table.hip", ["--cuda-host-only"]), ("bwd_table.hip", ["--cuda-host-only"]),
-                       ("api.hip", []), ("ipa_pack.hip", [])):
+                       ("api.hip", []), ("ipa_pack.hip", []), ("merge_chunks.hip", [])):
         o = objdir / (Path(src).stem + ".o")
         objs.append(o)
         if not o.exists():

@@ -274,14 +274,15 @@ def _pad_head_dims(q, k, v, gate, diff, bias_only=True, min_dim=32):
 def _split_over_keys(q, k, v, scale, softcap, biases=()):
     """Few queries against many keys (a decoding step over a long cache): B * Hq workgroups cannot fill 256 CUs, so the
     keys are cut into C chunks that run as C times as many heads of one launch, each leaving a normalised partial result
-    and its row statistic, and the partial results are merged with the weights 2^(lse_c - max).  Returns None when the
+    and its row statistic, and a second small launch merges the partial results with the weights 2^(lse_c - max).  Returns None when the
     call is not of that shape (enough workgroups already, short or indivisible key length, key / value tensors whose
     heads are not contiguous in memory), and the caller launches as usual."""
     B, Hq, Lq, D = q.shape
     Hkv, Lk, Dv = k.size(1), k.size(2), v.size(3)
     groups = B * Hq * ((Lq + 127) // 128)
-    # (a workgroup walks about 64 keys per microsecond and the merge below costs about 50: worth it from 8192 keys on)
-    if groups >= 256 or Lk < 8192 or Hq % Hkv or not (k.is_contiguous() and v.is_contiguous()):
+    # (a workgroup walks about 64 keys per microsecond; the copy of q, the row statistics and the merge launch cost
+    # about 20: worth it from 4096 keys on)
+    if groups >= 256 or Lk < 4096 or Hq % Hkv or not (k.is_contiguous() and v.is_contiguous()):
         return None
     chunks = 0
     for c in (64, 32, 16, 8, 4, 2):
@@ -301,12 +302,9 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
           for b, d in biases]
     lse = torch.empty(B, Hkv * chunks * G, Lq, dtype=torch.float32, device=q.device)
     part = _ffi.attn_fwd(qc, kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
-    lse = lse.view(B, Hkv, chunks, G, Lq)
-    lse = torch.where(lse == float("inf"), torch.full_like(lse, float("-inf")), lse)   # (the kernel's mark for "no keys")
-    top = lse.amax(dim=2, keepdim=True)
-    w = torch.exp2(lse - torch.where(top == float("-inf"), torch.zeros_like(top), top))   # (a chunk, or a row, without keys: 0)
-    merged = (w.unsqueeze(-1) * part.view(B, Hkv, chunks, G, Lq, Dv)).sum(dim=2) / w.sum(dim=2).clamp_min(1e-30).unsqueeze(-1)
-    return merged.to(q.dtype).view(B, Hq, Lq, Dv)
+    # one small launch: weights 2^(lse_c - max) over the chunks of a row; a chunk, or a row, without keys counts as zeros
+    merged = _ffi.merge_chunks(part.view(B * Hkv, chunks, G * Lq, Dv), lse.view(B * Hkv, chunks, G * Lq))
+    return merged.view(B, Hq, Lq, Dv)
 
 
 def _being_traced(*tensors) -> bool:

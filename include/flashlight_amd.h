@@ -265,6 +265,16 @@ typedef struct fl_ipa_pack_params {
 } fl_ipa_pack_params;
 int fl_ipa_pack(const fl_ipa_pack_params* p, void* stream);
 
+/* Merges partial results of one attention over `chunks` disjoint chunks of its keys (no counterpart in the reference,
+ * whose kernel walks all keys of a row in one program, monkeypatch/fusion/reduction_kernel_fusion.py:1102; used by the
+ * front end for decoding steps, where a few query rows meet a long key sequence and the chunks run as extra heads of
+ * one fl_attn_fwd launch).  part [outer, chunks, inner, dv] (element type `dtype`, contiguous) holds the chunks' results
+ * as fl_attn_fwd wrote them, lse [outer, chunks, inner] the row statistics of the same launch (fl_attn_params.lse: +inf
+ * for a row that attends nothing in a chunk); out [outer, inner, dv] receives sum_c w_c part_c / sum_c w_c with
+ * w_c = 2^(lse_c - max_c lse_c), zeros for a row that attends nothing at all.  dv even. */
+int fl_attn_merge_chunks(const void* part, const float* lse, void* out, int64_t outer, int32_t chunks, int64_t inner,
+                         int32_t dv, int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -861,7 +861,7 @@ def test_calls_from_several_threads_on_streams_of_their_own():
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(1, 32, 8, 1, 32768, 128), (2, 8, 8, 7, 8192, 64), (1, 4, 1, 130, 12288, 128), (1, 16, 4, 1, 65536, 128),
-                                   (1, 6, 2, 3, 8200, 64)])
+                                   (3, 4, 4, 2, 4096, 32), (1, 6, 2, 3, 8200, 64)])
 def test_few_queries_against_a_long_cache_are_split_over_the_keys(shape):
     """A decoding step: B * Hq workgroups cannot fill the chip, so the front end runs the key chunks as extra heads of one
     launch and merges the partial results by their row statistics.  Against eager fp32; the last shape's key length has
@@ -930,3 +930,23 @@ def test_grouped_heads_with_few_queries_are_packed_as_rows(shape, dtype):
     wide = torch.randn(B, Hq, Lq, D + 8, generator=g).to(dtype).cuda()
     want = F.scaled_dot_product_attention(wide[..., :D].float().cpu(), k.float(), v.float(), enable_gqa=True)
     assert_parity(A.attention_pytorch(wide[..., :D], kd, vd, enable_gqa=True), want, f"{shape} strided q")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_merge_of_key_chunks_through_the_abi(dtype):
+    """fl_attn_merge_chunks against the same sum in fp32 tensor operations: random statistics, chunks marked as holding no
+    keys for some rows (+inf), rows without keys in any chunk (zeros), value widths from 2 to 512."""
+    g = torch.Generator().manual_seed(5)
+    for outer, chunks, inner, dv in ((3, 4, 5, 128), (1, 64, 1, 512), (7, 2, 130, 2), (2, 9, 3, 96)):
+        part = torch.randn(outer, chunks, inner, dv, generator=g).to(dtype).cuda()
+        lse = (torch.randn(outer, chunks, inner, generator=g) * 6 + 10).cuda()
+        lse[torch.rand(outer, chunks, inner, generator=g).cuda() < 0.2] = float("inf")
+        lse[0, :, 0] = float("inf")
+        got = _ffi.merge_chunks(part, lse)
+        l = torch.where(lse == float("inf"), torch.full_like(lse, float("-inf")), lse)
+        top = l.amax(dim=1, keepdim=True)
+        w = torch.exp2(l - torch.where(top == float("-inf"), torch.zeros_like(top), top))
+        want = (w.unsqueeze(-1) * part.float()).sum(dim=1) / w.sum(dim=1).clamp_min(1e-30).unsqueeze(-1)
+        assert torch.count_nonzero(got[0, 0]).item() == 0
+        assert_parity(got, want, f"{(outer, chunks, inner, dv)}", max_tol=2e-2 if dtype == torch.bfloat16 else 4e-3, mean_tol=2e-3)

@@ -370,15 +370,10 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
         return _differentiable(q, k, v, scale=scale, mask_kind=mask_kind, window=window, prefix=prefix, doc_ids=doc_ids,
                                alibi_heads=alibi_heads, softcap=softcap, biases=biases, gate=gate, diff=diff,
                                lambda_full=lambda_full, dropout_p=dropout_p, dropout_seed=dropout_seed)
-    if _being_traced(q, k, v):
-        bl = list(biases) + [(None, 1)] * (2 - len(biases))
-        fn_kind, fn_c = (int(score_fn[0]), [float(c) for c in score_fn[1]]) if score_fn is not None else (0, [0.0] * 4)
-        return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),
-                        doc_ids, int(alibi_heads), float(softcap), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), gate,
-                        bool(diff), float(lambda_full), bool(seq_major_out), fn_kind, fn_c[0], fn_c[1], fn_c[2], fn_c[3])
-    if mask_kind == _ffi.MASK_NONE and gate is None and not diff and doc_ids is None and not alibi_heads \
-            and score_fn is None and dropout_p == 0.0 and not seq_major_out and \
-            all(b.dim() == 4 and b.size(1) == 1 and b.size(2) == 1 for b, _ in biases):
+    rows_independent = mask_kind == _ffi.MASK_NONE and gate is None and not diff and doc_ids is None and not alibi_heads \
+        and score_fn is None and dropout_p == 0.0 and not seq_major_out and \
+        all(b.dim() == 4 and b.size(1) == 1 and b.size(2) == 1 for b, _ in biases)
+    if rows_independent:
         Hq, Hkv, Lq = q.size(1), k.size(1), q.size(2)
         if Hq > Hkv and Hq % Hkv == 0 and (Hq // Hkv) * Lq <= 128 and q.is_contiguous():
             # few queries per head under grouped heads (a decoding step): without a mask the rows of a score matrix are
@@ -388,6 +383,13 @@ def dispatch(q, k, v, *, scale=None, mask_kind=_ffi.MASK_NONE, window=0, prefix=
             packed = dispatch(q.view(q.size(0), Hkv, (Hq // Hkv) * Lq, q.size(3)), k, v, softcap=softcap, biases=biases,
                               scale=scale if scale is not None else 1.0 / math.sqrt(q.size(-1)))
             return packed.view(q.size(0), Hq, Lq, v.size(3))
+    if _being_traced(q, k, v):
+        bl = list(biases) + [(None, 1)] * (2 - len(biases))
+        fn_kind, fn_c = (int(score_fn[0]), [float(c) for c in score_fn[1]]) if score_fn is not None else (0, [0.0] * 4)
+        return attn_fwd(q, k, v, float(scale) if scale is not None else -1.0, int(mask_kind), int(window), int(prefix),
+                        doc_ids, int(alibi_heads), float(softcap), bl[0][0], int(bl[0][1]), bl[1][0], int(bl[1][1]), gate,
+                        bool(diff), float(lambda_full), bool(seq_major_out), fn_kind, fn_c[0], fn_c[1], fn_c[2], fn_c[3])
+    if rows_independent:
         split = _split_over_keys(q, k, v, scale, softcap, biases) if all(b.is_contiguous() for b, _ in biases) else None
         if split is not None:
             return split

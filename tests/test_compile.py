@@ -61,7 +61,9 @@ CASES = {
 def test_variant_traces_into_one_operator(name):
     nodes = _trace(CASES[name], *_qkv())
     assert len(nodes) == 1
-    assert tuple(nodes[0].meta["example_value"].shape) == (1, 4, 64, 64)
+    # (unmasked grouped heads with so few queries reach the operator packed: the 2 query heads of a key / value head as
+    # 128 rows of that head)
+    assert tuple(nodes[0].meta["example_value"].shape) == ((1, 2, 128, 64) if name in ("vanilla", "softcap") else (1, 4, 64, 64))
 
 
 def test_document_diff_and_evoformer_trace():

@@ -276,13 +276,19 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
     keys are cut into C chunks that run as C times as many heads of one launch, each leaving a normalised partial result
     and its row statistic, and a second small launch merges the partial results with the weights 2^(lse_c - max).  Returns None when the
     call is not of that shape (enough workgroups already, short or indivisible key length, key / value tensors whose
-    heads are not contiguous in memory), and the caller launches as usual."""
+    heads are not contiguous in memory when there is more than one batch entry), and the caller launches as usual."""
     B, Hq, Lq, D = q.shape
     Hkv, Lk, Dv = k.size(1), k.size(2), v.size(3)
     groups = B * Hq * ((Lq + 127) // 128)
     # (a workgroup walks about 64 keys per microsecond; the copy of q, the row statistics and the merge launch cost
     # about 20: worth it from 4096 keys on)
-    if groups >= 256 or Lk < 4096 or Hq % Hkv or not (k.is_contiguous() and v.is_contiguous()):
+    if groups >= 256 or Lk < 4096 or Hq % Hkv:
+        return None
+    whole = k.is_contiguous() and v.is_contiguous()
+    # a cache that is a slice of a longer buffer (dense rows, heads further apart): with one batch entry the chunks can
+    # be the batch entries of the launch instead of heads
+    rows_dense = B == 1 and k.stride(3) == 1 and v.stride(3) == 1 and k.stride(2) == D and v.stride(2) == Dv
+    if not (whole or rows_dense):
         return None
     chunks = 0
     for c in (64, 32, 16, 8, 4, 2):
@@ -294,6 +300,13 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
     G, Lc = Hq // Hkv, Lk // chunks
     if scale is None:
         scale = 1.0 / math.sqrt(D)
+    if not whole:
+        kc = k.as_strided((chunks, Hkv, Lc, D), (Lc * D, k.stride(1), D, 1), k.storage_offset())
+        vc = v.as_strided((chunks, Hkv, Lc, Dv), (Lc * Dv, v.stride(1), Dv, 1), v.storage_offset())
+        bc = [(b.reshape(chunks, 1, 1, Lc), 1) for b, _ in biases]      # ([1, 1, 1, Lk] rows: chunk c is batch entry c)
+        lse = torch.empty(chunks, Hq, Lq, dtype=torch.float32, device=q.device)
+        part = _ffi.attn_fwd(q.expand(chunks, Hq, Lq, D), kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
+        return _ffi.merge_chunks(part.view(1, chunks, Hq * Lq, Dv), lse.view(1, chunks, Hq * Lq)).view(1, Hq, Lq, Dv)
     # chunk c of key / value head h becomes head h * C + c; its G query heads are copies of the G of head h
     qc = q.reshape(B, Hkv, 1, G, Lq, D).expand(B, Hkv, chunks, G, Lq, D).reshape(B, Hkv * chunks * G, Lq, D)
     kc, vc = k.view(B, Hkv * chunks, Lc, D), v.view(B, Hkv * chunks, Lc, Dv)

@@ -892,8 +892,16 @@ def test_few_queries_against_a_long_cache_are_split_over_the_keys(shape):
         got = ops.dispatch(qd, kd, vd, biases=[(torch.full((B, 1, 1, Lk), float("-inf")).to(torch.bfloat16).cuda(), 1)])
         assert torch.count_nonzero(got).item() == 0
     longer = torch.randn(B, Hkv, Lk + 64, D, generator=g).to(torch.bfloat16).cuda()
-    if B * Hkv > 1:   # (with one head in all the slice is still one contiguous block)
-        assert ops._split_over_keys(qd, longer[:, :, :Lk], longer[:, :, :Lk], None, 0.0) is None
+    ks, vs = longer[:, :, :Lk], torch.flip(longer, dims=(1,))[:, :, 64:]
+    if B > 1:   # (heads further apart than their rows: only one batch entry can be cut, its chunks as batch entries)
+        assert ops._split_over_keys(qd, ks, vs, None, 0.0) is None
+    elif Lk % 16 == 0:
+        assert ops._split_over_keys(qd, ks, vs, None, 0.0) is not None
+        pad = torch.zeros(1, 1, 1, Lk)
+        pad[..., 5:Lk // 2 + 3] = float("-inf")
+        got = ops.dispatch(qd, ks, vs, biases=[(pad.to(torch.bfloat16).cuda(), 1)])
+        want = F.scaled_dot_product_attention(q.float(), ks.float().cpu(), vs.float().cpu(), attn_mask=pad, enable_gqa=True)
+        assert_parity(got, want, str(shape) + " cache slice", max_tol=2e-3, mean_tol=2e-4)
 
 
 @pytest.mark.gpu

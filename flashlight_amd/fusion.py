@@ -1071,7 +1071,9 @@ def backend_inductor(gm: fx.GraphModule, example_inputs):
     for n in list(gm.graph.nodes):
         if n.op == "get_attr" and isinstance(n.target, str) and n.target.startswith("_flashlight_const_"):
             t = getattr(gm, n.target)
-            with (gm.graph.inserting_after(last_placeholder) if last_placeholder is not None else gm.graph.inserting_before(None)):
+            if last_placeholder is None:   # (a graph without inputs: nothing for a compiler to specialise on)
+                return gm.forward
+            with gm.graph.inserting_after(last_placeholder):
                 ph = gm.graph.placeholder(n.target)
             ph.meta.update(n.meta)
             n.replace_all_uses_with(ph)

@@ -165,7 +165,7 @@ def write_results_csv(rows: List[tuple], path: str) -> None:
 
 def parse_args(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer", "ipa", "backward"), default="variants",
+    ap.add_argument("--suite", choices=("variants", "diffattn", "evoformer", "ipa", "backward", "decode"), default="variants",
                     help="variants: run_flex_variants.py; diffattn: run_diff_attn.py (model dim 2048, head dims 64 and "
                          "128, published FLOP estimate 8 B S^2 H D); evoformer: run_evoformer.py (N_seq = S = 256, 4 "
                          "heads, mask bias + pair bias, FLOPs 4 B 256 S^2 H D); ipa: invariant point attention of "
@@ -197,7 +197,8 @@ def main(argv=None) -> List[tuple]:
     torch.manual_seed(0)
     rows: List[tuple] = []
     if args.suite != "variants":
-        rows = _run_backward_suite(args) if args.suite == "backward" else _run_other_suite(args)
+        rows = _run_backward_suite(args) if args.suite == "backward" else _run_decode_suite(args) if args.suite == "decode" \
+            else _run_other_suite(args)
         write_results_csv(rows, f"{args.output}.csv")
         return rows
     variants = registry() if args.dropout_p == 0.0 else dropout_registry(args.dropout_p)
@@ -216,6 +217,46 @@ def main(argv=None) -> List[tuple]:
                     rows.append((name, ms, tflops, *config))
                     print(f"{name:28s} {ms:9.4f} ms {tflops:8.1f} TFLOP/s")
     write_results_csv(rows, f"{args.output}.csv")
+    return rows
+
+
+DECODE_SHAPES = (  # batch, query heads, key / value heads, queries, keys, head dim
+    (1, 32, 8, 1, 32768, 128), (8, 32, 8, 1, 8192, 128), (32, 32, 8, 1, 2048, 128), (128, 32, 8, 1, 512, 128),
+    (16, 64, 8, 1, 4096, 128), (8, 32, 8, 16, 8192, 128), (4, 32, 32, 1, 4096, 64))
+
+
+def _run_decode_suite(args) -> List[tuple]:
+    """Decoding steps (no counterpart in the reference's sweeps): a few queries per sequence against a long key / value
+    cache, unmasked, grouped heads.  Times `attention_pytorch` (the front end packs the query heads of a key / value head
+    as rows and splits long key sequences into chunks) and, as `torch_sdpa`, torch's scaled_dot_product_attention on the
+    same operands (warm caches: a cache that was just written).  The TFLOP/s column is replaced by the rate at which the
+    keys and values are read, in TB/s."""
+    import torch
+    import torch.nn.functional as F
+    from ..attention_variants import attention_pytorch
+
+    def warm(fn, n=50):
+        for _ in range(10):
+            fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(n):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / n
+
+    rows: List[tuple] = []
+    for B, Hq, Hkv, Lq, Lk, D in DECODE_SHAPES:
+        q = torch.randn(B, Hq, Lq, D, device="cuda", dtype=torch.bfloat16)
+        k, v = (torch.randn(B, Hkv, Lk, D, device="cuda", dtype=torch.bfloat16) for _ in range(2))
+        print(f"### Config: B={B} Hq={Hq} Hkv={Hkv} Lq={Lq} Lk={Lk} D={D} ###")
+        for name, fn in (("decode", lambda: attention_pytorch(q, k, v, enable_gqa=True)),
+                         ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v, enable_gqa=True))):
+            ms = warm(fn)
+            tbs = 2 * k.numel() * 2 / ms / 1e9
+            rows.append((name, ms, tbs, B, Lk, Hq, D, Hq // Hkv, 0.0))
+            print(f"{name:28s} {ms:9.4f} ms {tbs:8.2f} TB/s of keys and values")
     return rows
 
 

@@ -19,26 +19,35 @@ __global__ void __launch_bounds__(64) merge_chunks_kernel(const E* __restrict__ 
   const int64_t row = blockIdx.x, o = row / inner, i = row % inner;
   const int lane = threadIdx.x;
   const float* l = lse + (o * chunks) * inner + i;
+  // maximum and sum over the chunks: the lanes take a chunk each, then the wave reduces
   float top = -INFINITY;
-  for (int c = 0; c < chunks; ++c) {
+  for (int c = lane; c < chunks; c += 64) {
     const float x = l[(int64_t)c * inner];
-    if (x != INFINITY) top = fmaxf(top, x);
+    top = fmaxf(top, x == INFINITY ? -INFINITY : x);
   }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) top = fmaxf(top, __shfl_xor(top, d, 64));
+  const float ref = top == -INFINITY ? 0.f : top;   // (no keys anywhere: every weight below is 0)
   float total = 0.f;
-  for (int c = 0; c < chunks; ++c) {
+  for (int c = lane; c < chunks; c += 64) {
     const float x = l[(int64_t)c * inner];
-    if (x != INFINITY && top != -INFINITY) total += exp2f(x - top);
+    total += x == INFINITY ? 0.f : exp2f(x - ref);
   }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) total += __shfl_xor(total, d, 64);
   const float inv = total > 0.f ? 1.0f / total : 0.f;
-  for (int d = 2 * lane; d < dv; d += 128) {   // dv is even: two elements per lane and step
+  // the weighted sum: two elements per lane and step (dv is even); the loads of the chunks do not depend on one another
+  const int64_t chunk_stride = inner * dv;
+  for (int d = 2 * lane; d < dv; d += 128) {
+    const E* p = part + ((o * chunks * inner + i) * dv + d);
     float a0 = 0.f, a1 = 0.f;
+#pragma unroll 8
     for (int c = 0; c < chunks; ++c) {
       const float x = l[(int64_t)c * inner];
-      if (x == INFINITY || top == -INFINITY) continue;
-      const float w = exp2f(x - top);
-      const E* p = part + (((o * chunks + c) * inner + i) * dv + d);
-      a0 += w * (float)p[0];
-      a1 += w * (float)p[1];
+      const float w = x == INFINITY ? 0.f : exp2f(x - ref);
+      const float v0 = (float)p[c * chunk_stride], v1 = (float)p[c * chunk_stride + 1];
+      a0 += w * v0;
+      a1 += w * v1;
     }
     E* q = out + (row * dv + d);
     q[0] = (E)(a0 * inv);

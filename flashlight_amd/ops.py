@@ -300,7 +300,7 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
     G, Lc = Hq // Hkv, Lk // chunks
     if scale is None:
         scale = 1.0 / math.sqrt(D)
-    if not whole:
+    if rows_dense:   # (also when the cache is one block: no copy of q, which the launch reads with batch stride 0)
         kc = k.as_strided((chunks, Hkv, Lc, D), (Lc * D, k.stride(1), D, 1), k.storage_offset())
         vc = v.as_strided((chunks, Hkv, Lc, Dv), (Lc * Dv, v.stride(1), Dv, 1), v.storage_offset())
         bc = [(b.reshape(chunks, 1, 1, Lc), 1) for b, _ in biases]      # ([1, 1, 1, Lk] rows: chunk c is batch entry c)

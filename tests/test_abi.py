@@ -270,6 +270,20 @@ def test_ipa_pack_rejects_bad_arguments_without_a_gpu(lib):
     assert lib.fl_ipa_pack(C.byref(p), None) == -2                       # no rows
 
 
+def test_merge_chunks_rejects_bad_arguments_without_a_gpu(lib):
+    assert "fl_attn_merge_chunks" in declared_functions()
+    ptr = C.c_void_p(0x10000)
+    merge = lambda part, lse, out, outer, chunks, inner, dv, dtype: lib.fl_attn_merge_chunks(part, lse, out, outer, chunks, inner, dv, dtype, None)
+    assert merge(None, ptr, ptr, 1, 2, 3, 64, 0) == -1      # null operands
+    assert merge(ptr, None, ptr, 1, 2, 3, 64, 0) == -1
+    assert merge(ptr, ptr, None, 1, 2, 3, 64, 0) == -1
+    assert merge(ptr, ptr, ptr, 0, 2, 3, 64, 0) == -2       # no rows
+    assert merge(ptr, ptr, ptr, 1, 0, 3, 64, 0) == -2       # no chunks
+    assert merge(ptr, ptr, ptr, 1, 2, 3, 63, 0) == -2       # odd value width
+    assert merge(ptr, ptr, ptr, 1 << 20, 2, 1 << 20, 64, 0) == -2   # more rows than a launch has workgroups
+    assert merge(ptr, ptr, ptr, 1, 2, 3, 64, 1) == -4       # fp32 partial results are not produced by any kernel here
+
+
 def test_probe_library_is_separate_and_rejects_bad_arguments_without_a_gpu(lib):
     # the measurement aids live in a bench-only library: the product library exports none of them, the probe library
     # exports every function its header declares, and each checks its arguments on the host before launching anything

@@ -290,6 +290,28 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
     rows_dense = B == 1 and k.stride(3) == 1 and v.stride(3) == 1 and k.stride(2) == D and v.stride(2) == Dv
     if not (whole or rows_dense):
         return None
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    if rows_dense:
+        # one batch entry (also when the cache is one block): the chunks are the batch entries of the launch, which reads
+        # the queries with batch stride 0 (no copy).  Chunks of a multiple of 8 keys; what is left over at the end of a key
+        # length that does not divide is one more, shorter chunk from a launch of its own
+        chunks = next((c for c in (64, 32, 16, 8, 4, 2) if (Lk // c) // 8 * 8 >= 512 and groups * c <= 2048), 0)
+        if not chunks:
+            return None
+        Lc = (Lk // chunks) // 8 * 8
+        main = chunks * Lc
+        kc = k.as_strided((chunks, Hkv, Lc, D), (Lc * D, k.stride(1), D, 1), k.storage_offset())
+        vc = v.as_strided((chunks, Hkv, Lc, Dv), (Lc * Dv, v.stride(1), Dv, 1), v.storage_offset())
+        bc = [(b[..., :main].reshape(chunks, 1, 1, Lc), 1) for b, _ in biases]   # ([1, 1, 1, Lk] rows: chunk c is entry c)
+        lse = torch.empty(chunks, Hq, Lq, dtype=torch.float32, device=q.device)
+        part = _ffi.attn_fwd(q.expand(chunks, Hq, Lq, D), kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
+        if main < Lk:
+            lse_tail = torch.empty(1, Hq, Lq, dtype=torch.float32, device=q.device)
+            tail = _ffi.attn_fwd(q, k[:, :, main:], v[:, :, main:], scale=scale, softcap=softcap, lse=lse_tail,
+                                 biases=[(b[..., main:], 1) for b, _ in biases])
+            part, lse, chunks = torch.cat((part, tail)), torch.cat((lse, lse_tail)), chunks + 1
+        return _ffi.merge_chunks(part.view(1, chunks, Hq * Lq, Dv), lse.view(1, chunks, Hq * Lq)).view(1, Hq, Lq, Dv)
     chunks = 0
     for c in (64, 32, 16, 8, 4, 2):
         if Lk % c == 0 and Lk // c >= 512 and (Lk // c) % 8 == 0 and groups * c <= 2048:
@@ -298,15 +320,6 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
     if not chunks:
         return None
     G, Lc = Hq // Hkv, Lk // chunks
-    if scale is None:
-        scale = 1.0 / math.sqrt(D)
-    if rows_dense:   # (also when the cache is one block: no copy of q, which the launch reads with batch stride 0)
-        kc = k.as_strided((chunks, Hkv, Lc, D), (Lc * D, k.stride(1), D, 1), k.storage_offset())
-        vc = v.as_strided((chunks, Hkv, Lc, Dv), (Lc * Dv, v.stride(1), Dv, 1), v.storage_offset())
-        bc = [(b.reshape(chunks, 1, 1, Lc), 1) for b, _ in biases]      # ([1, 1, 1, Lk] rows: chunk c is batch entry c)
-        lse = torch.empty(chunks, Hq, Lq, dtype=torch.float32, device=q.device)
-        part = _ffi.attn_fwd(q.expand(chunks, Hq, Lq, D), kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
-        return _ffi.merge_chunks(part.view(1, chunks, Hq * Lq, Dv), lse.view(1, chunks, Hq * Lq)).view(1, Hq, Lq, Dv)
     # chunk c of key / value head h becomes head h * C + c; its G query heads are copies of the G of head h
     qc = q.reshape(B, Hkv, 1, G, Lq, D).expand(B, Hkv, chunks, G, Lq, D).reshape(B, Hkv * chunks * G, Lq, D)
     kc, vc = k.view(B, Hkv * chunks, Lc, D), v.view(B, Hkv * chunks, Lc, Dv)

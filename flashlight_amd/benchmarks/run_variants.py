@@ -222,7 +222,7 @@ def main(argv=None) -> List[tuple]:
 
 DECODE_SHAPES = (  # batch, query heads, key / value heads, queries, keys, head dim
     (1, 32, 8, 1, 32768, 128), (8, 32, 8, 1, 8192, 128), (32, 32, 8, 1, 2048, 128), (128, 32, 8, 1, 512, 128),
-    (16, 64, 8, 1, 4096, 128), (8, 32, 8, 16, 8192, 128), (4, 32, 32, 1, 4096, 64))
+    (16, 64, 8, 1, 4096, 128), (8, 32, 8, 16, 8192, 128), (4, 32, 32, 1, 4096, 64), (1, 32, 8, 1, 40001, 128))
 
 
 def _run_decode_suite(args) -> List[tuple]:

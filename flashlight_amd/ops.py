@@ -304,14 +304,15 @@ def _split_over_keys(q, k, v, scale, softcap, biases=()):
         kc = k.as_strided((chunks, Hkv, Lc, D), (Lc * D, k.stride(1), D, 1), k.storage_offset())
         vc = v.as_strided((chunks, Hkv, Lc, Dv), (Lc * Dv, v.stride(1), Dv, 1), v.storage_offset())
         bc = [(b[..., :main].reshape(chunks, 1, 1, Lc), 1) for b, _ in biases]   # ([1, 1, 1, Lk] rows: chunk c is entry c)
-        lse = torch.empty(chunks, Hq, Lq, dtype=torch.float32, device=q.device)
-        part = _ffi.attn_fwd(q.expand(chunks, Hq, Lq, D), kc, vc, scale=scale, softcap=softcap, lse=lse, biases=bc)
+        total = chunks + (1 if main < Lk else 0)   # (both launches write into one pair of buffers)
+        lse = torch.empty(total, Hq, Lq, dtype=torch.float32, device=q.device)
+        part = torch.empty(total, Hq, Lq, Dv, dtype=q.dtype, device=q.device)
+        _ffi.attn_fwd(q.expand(chunks, Hq, Lq, D), kc, vc, scale=scale, softcap=softcap, lse=lse[:chunks], biases=bc,
+                      out=part[:chunks])
         if main < Lk:
-            lse_tail = torch.empty(1, Hq, Lq, dtype=torch.float32, device=q.device)
-            tail = _ffi.attn_fwd(q, k[:, :, main:], v[:, :, main:], scale=scale, softcap=softcap, lse=lse_tail,
-                                 biases=[(b[..., main:], 1) for b, _ in biases])
-            part, lse, chunks = torch.cat((part, tail)), torch.cat((lse, lse_tail)), chunks + 1
-        return _ffi.merge_chunks(part.view(1, chunks, Hq * Lq, Dv), lse.view(1, chunks, Hq * Lq)).view(1, Hq, Lq, Dv)
+            _ffi.attn_fwd(q, k[:, :, main:], v[:, :, main:], scale=scale, softcap=softcap, lse=lse[chunks:],
+                          biases=[(b[..., main:], 1) for b, _ in biases], out=part[chunks:])
+        return _ffi.merge_chunks(part.view(1, total, Hq * Lq, Dv), lse.view(1, total, Hq * Lq)).view(1, Hq, Lq, Dv)
     chunks = 0
     for c in (64, 32, 16, 8, 4, 2):
         if Lk % c == 0 and Lk // c >= 512 and (Lk // c) % 8 == 0 and groups * c <= 2048:

@@ -160,3 +160,33 @@ def test_results_repeat_bit_for_bit():
     torch.cuda.synchronize()
     for a, b in zip(first, second):
         assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 32, 8, 1, 32768, 128), (1, 8, 2, 2, 8201, 64), (4, 16, 4, 1, 8192, 128), (16, 32, 8, 1, 1024, 128)])
+def test_decoding_steps_replay_from_a_graph(shape):
+    """A serving loop replays its decoding step from a graph.  The front end's reshapes for such calls (query heads as
+    rows; key chunks as batch entries or heads, a shorter last chunk, the merge launch) allocate their buffers inside the
+    capture and record plain launches only: every replay, on new cache contents, equals the eager call."""
+    B, Hq, Hkv, Lq, Lk, D = shape
+    g = torch.Generator().manual_seed(Lk)
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(torch.bfloat16).to(DEV)
+    k, v = (torch.randn(B, Hkv, Lk, D, generator=g).to(torch.bfloat16).to(DEV) for _ in range(2))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            A.attention_pytorch(q, k, v, enable_gqa=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = A.attention_pytorch(q, k, v, enable_gqa=True)
+    for step in range(3):
+        q.copy_(torch.randn(q.shape, generator=g).to(torch.bfloat16))
+        k[:, :, step::3].mul_(-0.5)
+        v.copy_(torch.randn(v.shape, generator=g).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = A.attention_pytorch(q, k, v, enable_gqa=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), (shape, step)
